@@ -1,0 +1,167 @@
+// Shared device/host helpers for libjsgrad_hip.so (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/jsgrad_hip.h"
+
+namespace jsg {
+
+// ---------------------------------------------------------------- host side state / errors
+struct State {
+  bool ready = false;
+  int device = -1;
+  int cu_count = 0;
+  hipStream_t stream = nullptr;
+  bool capturing = false;
+};
+State &state();
+int fail(const char *fmt, ...);
+int fail_hip(hipError_t e, const char *what);
+
+#define JSG_HIP(call)                                   \
+  do {                                                  \
+    hipError_t e_ = (call);                             \
+    if (e_ != hipSuccess) return jsg::fail_hip(e_, #call); \
+  } while (0)
+#define JSG_REQUIRE(cond, ...)               \
+  do {                                       \
+    if (!(cond)) return jsg::fail(__VA_ARGS__); \
+  } while (0)
+#define JSG_READY() JSG_REQUIRE(jsg::state().ready, "jsgrad_hip_init has not been called")
+// after a kernel launch
+#define JSG_LAUNCHED() JSG_HIP(hipGetLastError())
+
+// ---------------------------------------------------------------- device helpers
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
+typedef float f4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
+
+// Reinterpret a 32-bit word as two halves.  Always go through this by-value helper: __builtin_bit_cast applied
+// directly to an element of an ext_vector (e.g. bit_cast(h2_t, vec[i])) reads element 0 whatever i is.
+__device__ __forceinline__ h2_t as_h2(uint32_t u) { return __builtin_bit_cast(h2_t, u); }
+__device__ __forceinline__ float h2f(_Float16 h) { return (float)h; }
+__device__ __forceinline__ _Float16 f2h(float f) { return (_Float16)f; }  // round-to-nearest-even
+__device__ __forceinline__ float rn16(float f) { return (float)(_Float16)f; }
+// RN16(a * b) with the sign of zero intact.  Written the plain way, the compiler fuses the multiply and the
+// conversion into v_fma_mixlo_f16 a, b, +0, and (-0) + (+0) is +0; the empty asm keeps the product a separate value.
+__device__ __forceinline__ _Float16 mul_rn16(float a, float b) {
+  float p = a * b;
+  asm volatile("" : "+v"(p));
+  return (_Float16)p;
+}
+
+// activation dtype traits: float tensors keep float, half tensors round to fp16 at every store
+template <typename AT> struct Act;
+template <> struct Act<float> {
+  static constexpr bool is16 = false;
+  __device__ static __forceinline__ float rn(float f) { return f; }
+  __device__ static __forceinline__ float ld(const float *p) { return *p; }
+  __device__ static __forceinline__ void st(float *p, float f) { *p = f; }
+};
+template <> struct Act<_Float16> {
+  static constexpr bool is16 = true;
+  __device__ static __forceinline__ float rn(float f) { return rn16(f); }
+  __device__ static __forceinline__ float ld(const _Float16 *p) { return (float)*p; }
+  __device__ static __forceinline__ void st(_Float16 *p, float f) { *p = (_Float16)f; }
+};
+
+// DPP cross-lane moves inside a 64-lane wavefront
+template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float readlane_f(float v, int lane) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane)); }
+
+// sum over the 64 lanes; every lane gets the total
+__device__ __forceinline__ float wave_sum(float v) {
+  v += dpp_f<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += dpp_f<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += dpp_f<0x141>(v);  // row_half_mirror
+  v += dpp_f<0x140>(v);  // row_mirror: every lane of a 16-lane row now holds the row total
+  return (readlane_f(v, 0) + readlane_f(v, 16)) + (readlane_f(v, 32) + readlane_f(v, 48));
+}
+__device__ __forceinline__ float wave_max(float v) {
+  v = fmaxf(v, dpp_f<0xB1>(v));
+  v = fmaxf(v, dpp_f<0x4E>(v));
+  v = fmaxf(v, dpp_f<0x141>(v));
+  v = fmaxf(v, dpp_f<0x140>(v));
+  return fmaxf(fmaxf(readlane_f(v, 0), readlane_f(v, 16)), fmaxf(readlane_f(v, 32), readlane_f(v, 48)));
+}
+// sum over aligned groups of 16 lanes (one DPP row); every lane of the group gets the group total
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_f<0xB1>(v);
+  v += dpp_f<0x4E>(v);
+  v += dpp_f<0x141>(v);
+  v += dpp_f<0x140>(v);
+  return v;
+}
+// sum over aligned groups of 8 lanes
+__device__ __forceinline__ float row8_sum(float v) {
+  v += dpp_f<0xB1>(v);
+  v += dpp_f<0x4E>(v);
+  v += dpp_f<0x141>(v);
+  return v;
+}
+
+// ---------------------------------------------------------------- jsgrad's polynomial exp2 / sin
+// The reference's CPU backend has no native exp2/sin and lowers them to polynomials
+// (/root/reference/jsgrad/ops.ts:1625-1676, renderer/cstyle.ts:215).  These follow the same
+// operation order without FMA contraction so that results agree to the bit with a C evaluation.
+
+__device__ __forceinline__ float pow2i(int q) { return __int_as_float((uint32_t)(q + 127) << 23); }
+__device__ __forceinline__ int rintk(float d) {
+  float t = __fadd_rn(d, d < 0.0f ? -0.5f : 0.5f);
+  if (!(t > -2147483000.0f) || !(t < 2147483000.0f)) return (int)0x80000000;
+  return (int)t;
+}
+__device__ __forceinline__ float mask_nonfinite(float d) { return (d != INFINITY) ? ((d != d) ? 0.0f : ((d != -INFINITY) ? d : 0.0f)) : 0.0f; }
+
+// xexp2 for float32 (ops.ts:1650-1673)
+__device__ __forceinline__ float xexp2f(float d) {
+  const float c[7] = {0.1535920892e-3f, 0.1339262701e-2f, 0.9618384764e-2f, 0.5550347269e-1f, 0.2402264476e+0f, 0.6931471825e+0f, 1.0f};
+  float x = mask_nonfinite(d);
+  int q = rintk(x);
+  float s = __fsub_rn(x, (float)q);
+  float u = c[0];
+#pragma unroll
+  for (int i = 1; i < 7; i++) u = __fadd_rn(__fmul_rn(u, s), c[i]);
+  u = __fmul_rn(__fmul_rn(u, pow2i(q >> 1)), pow2i(q - (q >> 1)));
+  if (d >= 128.0f) u = INFINITY;
+  if (d < -150.0f) u = 0.0f;
+  if (d != d) u = NAN;
+  return u;
+}
+// xexp2 for half tensors: fp16-rounded coefficients, float Horner chain, bounds [23, -22]
+__device__ __forceinline__ float xexp2h(float d) {
+  const float c[7] = {0.1535920892e-3f, 0.1339262701e-2f, 0.9618384764e-2f, 0.5550347269e-1f, 0.2402264476e+0f, 0.6931471825e+0f, 1.0f};
+  float x = mask_nonfinite(d);
+  int q = rintk(x);
+  float s = __fsub_rn(x, (float)q);
+  float u = rn16(c[0]);
+#pragma unroll
+  for (int i = 1; i < 7; i++) u = __fadd_rn(__fmul_rn(u, s), rn16(c[i]));
+  q = q > 60 ? 60 : (q < -60 ? -60 : q);
+  u = __fmul_rn(__fmul_rn(u, pow2i(q >> 1)), pow2i(q - (q >> 1)));
+  if (d >= 23.0f) u = INFINITY;
+  if (d < -22.0f) u = 0.0f;
+  if (d != d) u = NAN;
+  return u;
+}
+// Tensor.exp on float tensors (tensor.ts:147-154)
+__device__ __forceinline__ float exp_f32(float x) { return xexp2f(__fmul_rn(x, 1.4426950408889634f)); }
+
+// silu(a) = a * 1/(1 + exp2(a * -1/ln2)) (tensor.ts:2909-2911, 3210-3226) in the activation dtype's arithmetic
+template <typename AT> __device__ __forceinline__ float silu_act(float a);
+template <> __device__ __forceinline__ float silu_act<float>(float a) {
+  float u = xexp2f(__fmul_rn(a, -1.4426950408889634f));
+  return __fmul_rn(a, __fdiv_rn(1.0f, __fadd_rn(1.0f, u)));
+}
+template <> __device__ __forceinline__ float silu_act<_Float16>(float a) {
+  float u = xexp2h(rn16(__fmul_rn(a, rn16(-1.4426950408889634f))));
+  return __fmul_rn(a, __fdiv_rn(1.0f, __fadd_rn(1.0f, u)));
+}
+
+}  // namespace jsg

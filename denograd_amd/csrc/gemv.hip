@@ -1,0 +1,390 @@
+// One-row linear layers (GEMV) with in-register dequantisation for gfx950.
+//
+// y[out] = x[in] . W^T for W stored as float32, float16, int8 (+ fp16 scale per output row) or NF4
+// (+ fp16 scale per 64 elements): Linear.call / Int8Linear.call / NF4Linear.call of the reference
+// (/root/reference/jsgrad/nn/index.ts:411, /root/reference/jsgrad/models/llama3.ts:35,91-97) at batch 1,
+// where the whole cost is streaming W once from HBM.
+//
+// Mapping: a block first stages the input row in LDS (optionally applying RMSNorm,
+// nn/index.ts:586-588), then each 64-lane wavefront owns ROWS consecutive output rows and walks the
+// reduce axis in steps of 64 lanes x 16 bytes: one 128-bit coalesced weight load per lane per row,
+// dequantised in registers, accumulated in float.  A wavefront needs no barrier after staging; the
+// final cross-lane sum is DPP.  Fused epilogues: plain store (+ residual), rotary embedding with the
+// KV-cache write (models/llama.ts:61-87), SwiGLU (llama.ts:108-110).
+#include "common.h"
+
+namespace jsg {
+
+enum { EPI_STORE = 0, EPI_ROPE_KV = 1, EPI_SWIGLU = 2 };
+
+struct GemvArgs {
+  const void *w[3];       // up to three matrices sharing the input row: (wq, wk, wv) or (w1, w3)
+  const void *s[3];       // their scales (int8: per row, nf4: per 64 elements)
+  int rows[3];            // rows of each matrix (0 = unused)
+  int in_f;
+  const void *x;          // input row, activation dtype
+  const void *norm_w;     // RMSNorm weight or nullptr
+  float eps;
+  float inv_d;            // float(1/in_f), the constant the mean is multiplied with (tensor.ts:2113-2117)
+  void *y;                // EPI_STORE: y[rows0]; EPI_SWIGLU: g[rows0]; EPI_ROPE_KV: q_out[rows0]
+  const void *residual;   // EPI_STORE only, may be nullptr
+  const void *rope_table; // [2*max_context][hd/2][2], activation dtype
+  const int32_t *st;      // device {token, start_pos}
+  void *cache_k, *cache_v;
+  int head_dim, max_context;
+};
+
+// ---- weight formats: VEC elements per 16-byte load --------------------------------------------
+template <int KIND> struct WFmt;
+template <> struct WFmt<JSGRAD_W_F32> { static constexpr int VEC = 4; };
+template <> struct WFmt<JSGRAD_W_F16> { static constexpr int VEC = 8; };
+template <> struct WFmt<JSGRAD_W_I8> { static constexpr int VEC = 16; };
+template <> struct WFmt<JSGRAD_W_NF4> { static constexpr int VEC = 32; };
+
+// NF4 code book (llama3.ts:80-81); the CODE tensor is float16, so every literal is rounded to fp16 first
+#define JSG_C16(x) ((float)(_Float16)(x))
+__device__ __constant__ float NF4_CODE[16] = {JSG_C16(-1.0f), JSG_C16(-0.6961928009986877f), JSG_C16(-0.5250730514526367f), JSG_C16(-0.39491748809814453f),
+                                              JSG_C16(-0.28444138169288635f), JSG_C16(-0.18477343022823334f), JSG_C16(-0.09105003625154495f), JSG_C16(0.0f),
+                                              JSG_C16(0.07958029955625534f), JSG_C16(0.16093020141124725f), JSG_C16(0.24611230194568634f), JSG_C16(0.33791524171829224f),
+                                              JSG_C16(0.44070982933044434f), JSG_C16(0.5626170039176941f), JSG_C16(0.7229568362236023f), JSG_C16(1.0f)};
+
+// x fragment of one lane for one step: VEC activations
+template <typename AT, int VEC> struct XFrag;
+template <int VEC> struct XFrag<_Float16, VEC> {
+  h2_t v[VEC / 2];
+  __device__ __forceinline__ void load(const _Float16 *xs) {
+    const u4_t *p = (const u4_t *)xs;
+#pragma unroll
+    for (int i = 0; i < VEC / 8; i++) {
+      u4_t t = p[i];
+#pragma unroll
+      for (int j = 0; j < 4; j++) v[i * 4 + j] = as_h2(t[j]);
+    }
+  }
+  __device__ __forceinline__ float get(int i) const { return (float)v[i >> 1][i & 1]; }
+};
+template <int VEC> struct XFrag<float, VEC> {
+  float v[VEC];
+  __device__ __forceinline__ void load(const float *xs) {
+    const f4_t *p = (const f4_t *)xs;
+#pragma unroll
+    for (int i = 0; i < VEC / 4; i++) {
+      f4_t t = p[i];
+#pragma unroll
+      for (int j = 0; j < 4; j++) v[i * 4 + j] = t[j];
+    }
+  }
+  __device__ __forceinline__ float get(int i) const { return v[i]; }
+};
+
+// dot of one 16-byte weight vector with the lane's x fragment, accumulated into acc
+template <int KIND, typename AT> struct Dot {
+  static constexpr int VEC = WFmt<KIND>::VEC;
+  // generic float path
+  __device__ static __forceinline__ float run(u4_t wv, const XFrag<AT, VEC> &xf, float acc, float blk_scale, const float *lut) {
+    if constexpr (KIND == JSGRAD_W_F32) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) acc = fmaf(xf.get(i), __uint_as_float(wv[i]), acc);
+    } else if constexpr (KIND == JSGRAD_W_F16) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        h2_t w2 = as_h2(wv[i]);
+        acc = fmaf(xf.get(2 * i), (float)w2[0], acc);
+        acc = fmaf(xf.get(2 * i + 1), (float)w2[1], acc);
+      }
+    } else if constexpr (KIND == JSGRAD_W_I8) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        int d = (int)wv[i];
+        acc = fmaf(xf.get(4 * i + 0), (float)((d << 24) >> 24), acc);
+        acc = fmaf(xf.get(4 * i + 1), (float)((d << 16) >> 24), acc);
+        acc = fmaf(xf.get(4 * i + 2), (float)((d << 8) >> 24), acc);
+        acc = fmaf(xf.get(4 * i + 3), (float)(d >> 24), acc);
+      }
+    } else {
+      // 32 codes; element 2j is the high nibble of byte j (llama3.ts:92-94,105). One scale per lane-step
+      // because 32 | 64 and k is a multiple of 32.  Each term is x * (code * scale) as the reference forms it:
+      // the inner product is exact in float (11 x 11 significant bits).
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        uint32_t d = wv[i];
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+          uint32_t byte = (d >> (8 * b)) & 0xffu;
+          acc = fmaf(xf.get(8 * i + 2 * b), lut[byte >> 4] * blk_scale, acc);
+          acc = fmaf(xf.get(8 * i + 2 * b + 1), lut[byte & 15u] * blk_scale, acc);
+        }
+      }
+    }
+    return acc;
+  }
+};
+// fp16 activations x fp16 weights: packed dot with float accumulation
+template <> struct Dot<JSGRAD_W_F16, _Float16> {
+  static constexpr int VEC = 8;
+  __device__ static __forceinline__ float run(u4_t wv, const XFrag<_Float16, 8> &xf, float acc, float, const float *) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) acc = __builtin_amdgcn_fdot2(as_h2(wv[i]), xf.v[i], acc, false);
+    return acc;
+  }
+};
+// fp16 activations x int8 weights: bytes -> exact fp16 integers through the 0x6400 exponent trick
+// (0x6400 | u is the half 1024 + u for u in 0..255), then the packed dot
+template <> struct Dot<JSGRAD_W_I8, _Float16> {
+  static constexpr int VEC = 16;
+  __device__ static __forceinline__ float run(u4_t wv, const XFrag<_Float16, 16> &xf, float acc, float, const float *) {
+    const h2_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};  // 1024 + 128
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      uint32_t u = wv[i] ^ 0x80808080u;  // signed byte w -> unsigned w + 128
+      h2_t lo = as_h2(__builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias;
+      h2_t hi = as_h2(__builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias;
+      acc = __builtin_amdgcn_fdot2(lo, xf.v[2 * i], acc, false);
+      acc = __builtin_amdgcn_fdot2(hi, xf.v[2 * i + 1], acc, false);
+    }
+    return acc;
+  }
+};
+
+template <int KIND> __device__ __forceinline__ u4_t load_w(const void *w, size_t row, int in_f, int k) {
+  // element (row, k) sits at bit offset (row*in_f + k) * bits
+  constexpr int BITS = KIND == JSGRAD_W_F32 ? 32 : KIND == JSGRAD_W_F16 ? 16 : KIND == JSGRAD_W_I8 ? 8 : 4;
+  const char *p = (const char *)w + ((row * (size_t)in_f + (size_t)k) * BITS) / 8;
+  return __builtin_nontemporal_load((const u4_t *)p);
+}
+
+// stage x (optionally RMSNorm'ed) into LDS in the activation dtype
+template <typename AT> __device__ __forceinline__ void stage_x(const GemvArgs &a, AT *xs, float *red) {
+  const AT *x = (const AT *)a.x;
+  const int n = a.in_f, tid = threadIdx.x, nt = blockDim.x;
+  if (a.norm_w == nullptr) {
+    for (int i = tid; i < n; i += nt) xs[i] = x[i];
+    __syncthreads();
+    return;
+  }
+  float ss = 0.0f;
+  for (int i = tid; i < n; i += nt) {
+    AT v = x[i];
+    xs[i] = v;
+    float f = (float)v;
+    ss = fmaf(f, f, ss);
+  }
+  ss = wave_sum(ss);
+  const int wave = tid >> 6, nw = nt >> 6;
+  if ((tid & 63) == 0) red[wave] = ss;
+  __syncthreads();
+  float tot = 0.0f;
+  for (int i = 0; i < nw; i++) tot += red[i];
+  // sqrt(1 / (mean + eps)), mean = sum * float(1/d)  (nn/index.ts:586, tensor.ts:2944-2946)
+  const float r = __fsqrt_rn(__fdiv_rn(1.0f, __fadd_rn(__fmul_rn(tot, a.inv_d), a.eps)));
+  const AT *nw_ = (const AT *)a.norm_w;
+  for (int i = tid; i < n; i += nt) {
+    float v = Act<AT>::rn(__fmul_rn((float)xs[i], r));       // .cast(x.dtype) before the weight multiply
+    xs[i] = (AT)Act<AT>::rn(__fmul_rn(v, (float)nw_[i]));
+  }
+  __syncthreads();
+}
+
+template <int KIND, typename AT, int EPI, int ROWS>
+__global__ __launch_bounds__(256) void gemv_kernel(GemvArgs a) {
+  constexpr int VEC = WFmt<KIND>::VEC;
+  constexpr int NM = EPI == EPI_SWIGLU ? 2 : 1;  // matrices a wavefront evaluates on the same rows
+  extern __shared__ __align__(16) unsigned char smem[];
+  AT *xs = (AT *)smem;
+  __shared__ float red[8];
+  __shared__ float lut[16];
+  if (KIND == JSGRAD_W_NF4 && threadIdx.x < 16) lut[threadIdx.x] = NF4_CODE[threadIdx.x];
+  stage_x<AT>(a, xs, red);  // ends with a barrier, which also publishes lut
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const int total = EPI == EPI_SWIGLU ? a.rows[0] : a.rows[0] + a.rows[1] + a.rows[2];
+  const int g0 = (blockIdx.x * nw + wave) * ROWS;  // first row of this wavefront in the combined row space
+  if (g0 >= total) return;
+
+  // which matrix the group lies in (EPI_ROPE_KV stacks wq, wk, wv; group boundaries are multiples of ROWS)
+  int m = 0, r0 = g0;
+  if (EPI == EPI_ROPE_KV) {
+    if (r0 >= a.rows[0]) { r0 -= a.rows[0]; m = 1; }
+    if (m == 1 && r0 >= a.rows[1]) { r0 -= a.rows[1]; m = 2; }
+  }
+  const int mrows = a.rows[m];
+  const void *wp[NM];
+  const void *sp[NM];
+  wp[0] = a.w[m]; sp[0] = a.s[m];
+  if (NM == 2) { wp[1] = a.w[1]; sp[1] = a.s[1]; }
+
+  float acc[NM][ROWS];
+#pragma unroll
+  for (int j = 0; j < NM; j++)
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) acc[j][r] = 0.0f;
+
+  const int in_f = a.in_f;
+  for (int k = lane * VEC; k < in_f; k += 64 * VEC) {
+    u4_t wv[NM][ROWS];
+#pragma unroll
+    for (int j = 0; j < NM; j++)
+#pragma unroll
+      for (int r = 0; r < ROWS; r++) {
+        int row = r0 + r < mrows ? r0 + r : mrows - 1;  // clamp: tail rows reload the last row, never stored
+        wv[j][r] = load_w<KIND>(wp[j], (size_t)row, in_f, k);
+      }
+    XFrag<AT, VEC> xf;
+    xf.load(xs + k);
+#pragma unroll
+    for (int j = 0; j < NM; j++)
+#pragma unroll
+      for (int r = 0; r < ROWS; r++) {
+        float bs = 1.0f;
+        if constexpr (KIND == JSGRAD_W_NF4) {
+          int row = r0 + r < mrows ? r0 + r : mrows - 1;
+          bs = (float)((const _Float16 *)sp[j])[((size_t)row * in_f + k) >> 6];
+        }
+        acc[j][r] = Dot<KIND, AT>::run(wv[j][r], xf, acc[j][r], bs, lut);
+      }
+  }
+#pragma unroll
+  for (int j = 0; j < NM; j++)
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) acc[j][r] = wave_sum(acc[j][r]);
+
+  // per-row results in the activation dtype: RN_act(sum [* scale])
+  float val[NM][ROWS];
+#pragma unroll
+  for (int j = 0; j < NM; j++)
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+      float v = acc[j][r];
+      if constexpr (KIND == JSGRAD_W_I8) {
+        int row = r0 + r < mrows ? r0 + r : mrows - 1;
+        v = __fmul_rn(v, (float)((const _Float16 *)sp[j])[row]);
+      }
+      val[j][r] = Act<AT>::rn(v);
+    }
+
+  if constexpr (EPI == EPI_STORE) {
+    AT *y = (AT *)a.y;
+    const AT *res = (const AT *)a.residual;
+#pragma unroll
+    for (int r = 0; r < ROWS; r++)
+      if (lane == r && r0 + r < mrows) {
+        float v = val[0][r];
+        if (res) v = Act<AT>::rn(__fadd_rn((float)res[r0 + r], v));
+        y[r0 + r] = (AT)v;
+      }
+  } else if constexpr (EPI == EPI_SWIGLU) {
+    AT *g = (AT *)a.y;
+#pragma unroll
+    for (int r = 0; r < ROWS; r++)
+      if (lane == r && r0 + r < mrows) g[r0 + r] = (AT)Act<AT>::rn(__fmul_rn(silu_act<AT>(val[0][r]), val[1][r]));
+  } else {
+    static_assert(ROWS % 2 == 0 || EPI != EPI_ROPE_KV, "rotary pairs need an even row group");
+    const int pos = a.st[1];
+    if (pos < 0 || pos >= a.max_context) return;  // never write outside the cache
+    const int hd = a.head_dim;
+    if (m == 2) {  // value rows: plain copy into the cache row
+      AT *cv = (AT *)a.cache_v + (size_t)pos * a.rows[2];
+#pragma unroll
+      for (int r = 0; r < ROWS; r++)
+        if (lane == r && r0 + r < mrows) cv[r0 + r] = (AT)val[0][r];
+    } else {       // query / key rows: rotate interleaved pairs (llama.ts:17-32)
+      const AT *tab = (const AT *)a.rope_table + (size_t)pos * hd;
+      AT *dst = m == 0 ? (AT *)a.y : (AT *)a.cache_k + (size_t)pos * a.rows[1];
+#pragma unroll
+      for (int r = 0; r < ROWS; r += 2)
+        if (lane == r && r0 + r + 1 < mrows) {
+          const int i = ((r0 + r) % hd) >> 1;
+          const float c = (float)tab[2 * i], d = (float)tab[2 * i + 1];
+          const float av = val[0][r], bv = val[0][r + 1];
+          dst[r0 + r] = (AT)Act<AT>::rn(__fsub_rn(__fmul_rn(av, c), __fmul_rn(bv, d)));
+          dst[r0 + r + 1] = (AT)Act<AT>::rn(__fadd_rn(__fmul_rn(av, d), __fmul_rn(bv, c)));
+        }
+    }
+  }
+}
+
+// ---- host-side dispatch ------------------------------------------------------------------------
+
+template <int KIND, typename AT, int EPI> static int launch_rows(const GemvArgs &a, int total_rows) {
+  constexpr int ROWS = 4, NW = 4;
+  const int rows_per_block = ROWS * NW;
+  dim3 grid((total_rows + rows_per_block - 1) / rows_per_block), block(NW * 64);
+  size_t lds = (size_t)a.in_f * sizeof(AT);
+  hipLaunchKernelGGL((gemv_kernel<KIND, AT, EPI, ROWS>), grid, block, lds, state().stream, a);
+  JSG_LAUNCHED();
+  return 0;
+}
+template <int EPI> static int dispatch(int kind, int act, const GemvArgs &a, int total_rows) {
+#define JSG_CASE(K)                                                          \
+  case K:                                                                    \
+    return act == JSGRAD_F16 ? launch_rows<K, _Float16, EPI>(a, total_rows) : launch_rows<K, float, EPI>(a, total_rows);
+  switch (kind) {
+    JSG_CASE(JSGRAD_W_F32)
+    JSG_CASE(JSGRAD_W_F16)
+    JSG_CASE(JSGRAD_W_I8)
+    JSG_CASE(JSGRAD_W_NF4)
+  }
+#undef JSG_CASE
+  return fail("unknown weight kind %d", kind);
+}
+
+static int check_common(const char *who, int kind, int act, int in_f, const void *x) {
+  JSG_REQUIRE(act == JSGRAD_F16 || act == JSGRAD_F32, "%s: unknown activation dtype %d", who, act);
+  JSG_REQUIRE(kind >= JSGRAD_W_F32 && kind <= JSGRAD_W_NF4, "%s: unknown weight kind %d", who, kind);
+  JSG_REQUIRE(x, "%s: null input", who);
+  const int vec = kind == JSGRAD_W_F32 ? 4 : kind == JSGRAD_W_F16 ? 8 : kind == JSGRAD_W_I8 ? 16 : 64;
+  JSG_REQUIRE(in_f > 0 && in_f % vec == 0, "%s: in_features %d must be a positive multiple of %d for this weight format", who, in_f, vec);
+  JSG_REQUIRE((size_t)in_f * (act == JSGRAD_F16 ? 2 : 4) <= 64 * 1024, "%s: in_features %d does not fit the 64 KiB LDS staging buffer", who, in_f);
+  return 0;
+}
+
+}  // namespace jsg
+
+using namespace jsg;
+
+extern "C" {
+
+int jsgrad_hip_linear(int kind, const void *w, const void *scale, int out_f, int in_f, const void *x, void *y, const void *norm_weight, float eps,
+                      const void *residual, int act) {
+  JSG_READY();
+  if (int e = check_common("jsgrad_hip_linear", kind, act, in_f, x)) return e;
+  JSG_REQUIRE(w && y && out_f > 0, "jsgrad_hip_linear: null weight/output or out_features %d", out_f);
+  JSG_REQUIRE(kind < JSGRAD_W_I8 || scale, "jsgrad_hip_linear: quantised weight needs a scale");
+  JSG_REQUIRE(y != x, "jsgrad_hip_linear: output must not alias the input");
+  GemvArgs a = {};
+  a.w[0] = w; a.s[0] = scale; a.rows[0] = out_f; a.in_f = in_f; a.x = x; a.norm_w = norm_weight; a.eps = eps;
+  a.inv_d = (float)(1.0 / (double)in_f); a.y = y; a.residual = residual;
+  return dispatch<EPI_STORE>(kind, act, a, out_f);
+}
+
+int jsgrad_hip_ffn_gate(int kind, const void *w1, const void *s1, const void *w3, const void *s3, const void *x, const void *norm_weight, float eps,
+                        void *g, int dim, int hidden, int act) {
+  JSG_READY();
+  if (int e = check_common("jsgrad_hip_ffn_gate", kind, act, dim, x)) return e;
+  JSG_REQUIRE(w1 && w3 && g && hidden > 0, "jsgrad_hip_ffn_gate: null weight/output or hidden %d", hidden);
+  JSG_REQUIRE(kind < JSGRAD_W_I8 || (s1 && s3), "jsgrad_hip_ffn_gate: quantised weights need scales");
+  GemvArgs a = {};
+  a.w[0] = w1; a.s[0] = s1; a.w[1] = w3; a.s[1] = s3; a.rows[0] = hidden; a.rows[1] = hidden; a.in_f = dim; a.x = x;
+  a.norm_w = norm_weight; a.eps = eps; a.inv_d = (float)(1.0 / (double)dim); a.y = g;
+  return dispatch<EPI_SWIGLU>(kind, act, a, hidden);
+}
+
+int jsgrad_hip_qkv_rope(int kind, const void *wq, const void *sq, const void *wk, const void *sk, const void *wv, const void *sv, const void *x,
+                        const void *norm_weight, float eps, const void *rope_table, const int32_t *st, void *q_out, void *cache_k, void *cache_v, int dim,
+                        int n_heads, int n_kv_heads, int head_dim, int max_context, int act) {
+  JSG_READY();
+  if (int e = check_common("jsgrad_hip_qkv_rope", kind, act, dim, x)) return e;
+  JSG_REQUIRE(wq && wk && wv && rope_table && st && q_out && cache_k && cache_v, "jsgrad_hip_qkv_rope: null pointer argument");
+  JSG_REQUIRE(kind < JSGRAD_W_I8 || (sq && sk && sv), "jsgrad_hip_qkv_rope: quantised weights need scales");
+  JSG_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0, "jsgrad_hip_qkv_rope: n_heads %d must be a multiple of n_kv_heads %d", n_heads, n_kv_heads);
+  JSG_REQUIRE(head_dim > 0 && head_dim % 4 == 0, "jsgrad_hip_qkv_rope: head_dim %d must be a multiple of 4", head_dim);
+  JSG_REQUIRE(max_context > 0, "jsgrad_hip_qkv_rope: max_context %d", max_context);
+  GemvArgs a = {};
+  a.w[0] = wq; a.s[0] = sq; a.w[1] = wk; a.s[1] = sk; a.w[2] = wv; a.s[2] = sv;
+  a.rows[0] = n_heads * head_dim; a.rows[1] = n_kv_heads * head_dim; a.rows[2] = n_kv_heads * head_dim;
+  a.in_f = dim; a.x = x; a.norm_w = norm_weight; a.eps = eps; a.inv_d = (float)(1.0 / (double)dim); a.y = q_out;
+  a.rope_table = rope_table; a.st = st; a.cache_k = cache_k; a.cache_v = cache_v; a.head_dim = head_dim; a.max_context = max_context;
+  return dispatch<EPI_ROPE_KV>(kind, act, a, a.rows[0] + a.rows[1] + a.rows[2]);
+}
+
+}  // extern "C"

@@ -1,0 +1,232 @@
+// Device, memory, program loading, launch, timing and graph capture for libjsgrad_hip.so.
+// Stands behind jsgrad's Compiled / Allocator / Program contracts
+// (/root/reference/jsgrad/runtime/allocator.ts:28-47,99-107,166-191).
+#include <stdarg.h>
+#include <string.h>
+
+#include <vector>
+
+#include "common.h"
+
+namespace jsg {
+
+static thread_local char g_err[1024] = "";
+
+State &state() {
+  static State s;
+  return s;
+}
+int fail(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return 1;
+}
+int fail_hip(hipError_t e, const char *what) {
+  snprintf(g_err, sizeof(g_err), "%s: %s (%d)", what, hipGetErrorString(e), (int)e);
+  return (int)e ? (int)e : 1;
+}
+
+}  // namespace jsg
+
+using jsg::state;
+
+extern "C" {
+
+const char *jsgrad_hip_last_error(void) { return jsg::g_err; }
+
+int jsgrad_hip_init(int device) {
+  jsg::State &s = state();
+  if (s.ready && s.device == device) return 0;
+  JSG_REQUIRE(!s.ready, "jsgrad_hip_init: already initialised on device %d", s.device);
+  int n = 0;
+  JSG_HIP(hipGetDeviceCount(&n));
+  JSG_REQUIRE(device >= 0 && device < n, "jsgrad_hip_init: device %d out of range (%d devices)", device, n);
+  JSG_HIP(hipSetDevice(device));
+  hipDeviceProp_t p;
+  JSG_HIP(hipGetDeviceProperties(&p, device));
+  JSG_REQUIRE(strncmp(p.gcnArchName, "gfx950", 6) == 0, "jsgrad_hip_init: this library holds gfx950 code only, device is %s", p.gcnArchName);
+  s.cu_count = p.multiProcessorCount;
+  JSG_HIP(hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking));
+  s.device = device;
+  s.ready = true;
+  return 0;
+}
+
+int jsgrad_hip_device_name(char *host_out, size_t cap) {
+  JSG_READY();
+  hipDeviceProp_t p;
+  JSG_HIP(hipGetDeviceProperties(&p, state().device));
+  snprintf(host_out, cap, "%s (%s)", p.name, p.gcnArchName);
+  return 0;
+}
+int jsgrad_hip_cu_count(int *host_out) {
+  JSG_READY();
+  *host_out = state().cu_count;
+  return 0;
+}
+
+int jsgrad_hip_malloc(size_t nbytes, void **host_out_ptr) {
+  JSG_READY();
+  JSG_REQUIRE(nbytes > 0, "alloc size must be positive, getting %zu", nbytes);
+  JSG_REQUIRE(!state().capturing, "jsgrad_hip_malloc during graph capture");
+  JSG_HIP(hipMalloc(host_out_ptr, nbytes));
+  return 0;
+}
+int jsgrad_hip_free(void *ptr) {
+  JSG_READY();
+  if (!ptr) return 0;
+  JSG_REQUIRE(!state().capturing, "jsgrad_hip_free during graph capture");
+  JSG_HIP(hipStreamSynchronize(state().stream));
+  JSG_HIP(hipFree(ptr));
+  return 0;
+}
+int jsgrad_hip_copyin(void *dst, const void *host_src, size_t nbytes) {
+  JSG_READY();
+  JSG_REQUIRE(!state().capturing, "jsgrad_hip_copyin during graph capture");
+  if (nbytes == 0) return 0;
+  JSG_HIP(hipMemcpyAsync(dst, host_src, nbytes, hipMemcpyHostToDevice, state().stream));
+  JSG_HIP(hipStreamSynchronize(state().stream));  // the caller may reuse host_src as soon as this returns
+  return 0;
+}
+int jsgrad_hip_copyout(void *host_dst, const void *src, size_t nbytes) {
+  JSG_READY();
+  JSG_REQUIRE(!state().capturing, "jsgrad_hip_copyout during graph capture");
+  if (nbytes == 0) return 0;
+  JSG_HIP(hipMemcpyAsync(host_dst, src, nbytes, hipMemcpyDeviceToHost, state().stream));
+  JSG_HIP(hipStreamSynchronize(state().stream));
+  return 0;
+}
+int jsgrad_hip_copy(void *dst, const void *src, size_t nbytes) {
+  JSG_READY();
+  if (nbytes == 0) return 0;
+  JSG_HIP(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToDevice, state().stream));
+  return 0;
+}
+int jsgrad_hip_sync(void) {
+  JSG_READY();
+  JSG_REQUIRE(!state().capturing, "jsgrad_hip_sync during graph capture");
+  JSG_HIP(hipStreamSynchronize(state().stream));
+  return 0;
+}
+
+int jsgrad_hip_module_load(const void *host_image, size_t nbytes, void **host_out_module) {
+  JSG_READY();
+  JSG_REQUIRE(host_image && nbytes > 0, "jsgrad_hip_module_load: empty image");
+  hipModule_t m;
+  JSG_HIP(hipModuleLoadData(&m, host_image));
+  *host_out_module = (void *)m;
+  return 0;
+}
+int jsgrad_hip_module_unload(void *module) {
+  JSG_READY();
+  JSG_HIP(hipStreamSynchronize(state().stream));
+  JSG_HIP(hipModuleUnload((hipModule_t)module));
+  return 0;
+}
+int jsgrad_hip_module_get(void *module, const char *name, void **host_out_function) {
+  JSG_READY();
+  hipFunction_t f;
+  JSG_HIP(hipModuleGetFunction(&f, (hipModule_t)module, name));
+  *host_out_function = (void *)f;
+  return 0;
+}
+
+int jsgrad_hip_launch(void *function, const uint32_t host_grid[3], const uint32_t host_block[3], void *const *host_bufs, int nbufs,
+                      const int32_t *host_vals, int nvals, int wait, double *host_seconds) {
+  JSG_READY();
+  JSG_REQUIRE(function, "jsgrad_hip_launch: null function");
+  JSG_REQUIRE(nbufs >= 0 && nvals >= 0 && nbufs + nvals <= 64, "jsgrad_hip_launch: %d buffers + %d vals exceeds 64 arguments", nbufs, nvals);
+  for (int i = 0; i < 3; i++) JSG_REQUIRE(host_grid[i] > 0 && host_block[i] > 0, "jsgrad_hip_launch: zero grid/block dimension");
+  JSG_REQUIRE((uint64_t)host_block[0] * host_block[1] * host_block[2] <= 1024, "jsgrad_hip_launch: block of %u x %u x %u exceeds 1024 threads", host_block[0], host_block[1], host_block[2]);
+  // argument block laid out as the generated kernel declares it: pointers first, then int32 values
+  struct {
+    void *p[64];
+  } packed;
+  size_t off = 0;
+  char *base = (char *)&packed;
+  for (int i = 0; i < nbufs; i++) { memcpy(base + off, &host_bufs[i], sizeof(void *)); off += sizeof(void *); }
+  for (int i = 0; i < nvals; i++) { memcpy(base + off, &host_vals[i], sizeof(int32_t)); off += sizeof(int32_t); }
+  size_t size = off;
+  void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, base, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  if (wait) {
+    JSG_REQUIRE(!state().capturing, "jsgrad_hip_launch: wait during graph capture");
+    JSG_HIP(hipEventCreate(&e0));
+    JSG_HIP(hipEventCreate(&e1));
+    JSG_HIP(hipEventRecord(e0, state().stream));
+  }
+  JSG_HIP(hipModuleLaunchKernel((hipFunction_t)function, host_grid[0], host_grid[1], host_grid[2], host_block[0], host_block[1], host_block[2], 0, state().stream, nullptr, config));
+  if (wait) {
+    JSG_HIP(hipEventRecord(e1, state().stream));
+    JSG_HIP(hipEventSynchronize(e1));
+    float ms = 0;
+    JSG_HIP(hipEventElapsedTime(&ms, e0, e1));
+    if (host_seconds) *host_seconds = (double)ms * 1e-3;
+    JSG_HIP(hipEventDestroy(e0));
+    JSG_HIP(hipEventDestroy(e1));
+  }
+  return 0;
+}
+
+int jsgrad_hip_event_create(void **host_out_event) {
+  JSG_READY();
+  hipEvent_t e;
+  JSG_HIP(hipEventCreate(&e));
+  *host_out_event = (void *)e;
+  return 0;
+}
+int jsgrad_hip_event_record(void *event) {
+  JSG_READY();
+  JSG_HIP(hipEventRecord((hipEvent_t)event, state().stream));
+  return 0;
+}
+int jsgrad_hip_event_elapsed_ms(void *start, void *stop, float *host_out_ms) {
+  JSG_READY();
+  JSG_HIP(hipEventSynchronize((hipEvent_t)stop));
+  JSG_HIP(hipEventElapsedTime(host_out_ms, (hipEvent_t)start, (hipEvent_t)stop));
+  return 0;
+}
+int jsgrad_hip_event_destroy(void *event) {
+  JSG_READY();
+  JSG_HIP(hipEventDestroy((hipEvent_t)event));
+  return 0;
+}
+
+int jsgrad_hip_graph_begin(void) {
+  JSG_READY();
+  JSG_REQUIRE(!state().capturing, "jsgrad_hip_graph_begin: capture already in progress");
+  JSG_HIP(hipStreamSynchronize(state().stream));
+  JSG_HIP(hipStreamBeginCapture(state().stream, hipStreamCaptureModeThreadLocal));
+  state().capturing = true;
+  return 0;
+}
+int jsgrad_hip_graph_end(void **host_out_graph) {
+  JSG_READY();
+  JSG_REQUIRE(state().capturing, "jsgrad_hip_graph_end: no capture in progress");
+  state().capturing = false;
+  hipGraph_t g = nullptr;
+  JSG_HIP(hipStreamEndCapture(state().stream, &g));
+  hipGraphExec_t ge = nullptr;
+  hipError_t e = hipGraphInstantiate(&ge, g, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(g);
+  if (e != hipSuccess) return jsg::fail_hip(e, "hipGraphInstantiate");
+  *host_out_graph = (void *)ge;
+  return 0;
+}
+int jsgrad_hip_graph_launch(void *graph) {
+  JSG_READY();
+  JSG_REQUIRE(graph, "jsgrad_hip_graph_launch: null graph");
+  JSG_HIP(hipGraphLaunch((hipGraphExec_t)graph, state().stream));
+  return 0;
+}
+int jsgrad_hip_graph_destroy(void *graph) {
+  JSG_READY();
+  if (!graph) return 0;
+  JSG_HIP(hipStreamSynchronize(state().stream));
+  JSG_HIP(hipGraphExecDestroy((hipGraphExec_t)graph));
+  return 0;
+}
+
+}  // extern "C"

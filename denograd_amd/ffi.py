@@ -1,0 +1,88 @@
+"""ctypes bindings of libjsgrad_hip.so -- the same symbols a Deno `Deno.dlopen` binding would name
+(the pattern of /root/reference/dawn/bindings.ts:5-8 and /root/reference/jsgrad/env/deno.ts:17).
+
+The library is the product: nothing here falls back to a CPU path.  If the shared object is missing
+or a call fails, a `HipError` is raised.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libjsgrad_hip.so")
+
+F32, F16 = 0, 1
+W_F32, W_F16, W_I8, W_NF4 = 0, 1, 2, 3
+
+
+class HipError(RuntimeError):
+    pass
+
+
+_vp, _i32, _f32, _sz, _u64 = C.c_void_p, C.c_int, C.c_float, C.c_size_t, C.c_uint64
+_pp = C.POINTER(C.c_void_p)
+
+# name -> (argtypes, restype); every entry point declared in include/jsgrad_hip.h
+SIGNATURES: dict[str, tuple[list, object]] = {
+    "jsgrad_hip_init": ([_i32], _i32),
+    "jsgrad_hip_last_error": ([], C.c_char_p),
+    "jsgrad_hip_device_name": ([C.c_char_p, _sz], _i32),
+    "jsgrad_hip_cu_count": ([C.POINTER(_i32)], _i32),
+    "jsgrad_hip_malloc": ([_sz, _pp], _i32),
+    "jsgrad_hip_free": ([_vp], _i32),
+    "jsgrad_hip_copyin": ([_vp, _vp, _sz], _i32),
+    "jsgrad_hip_copyout": ([_vp, _vp, _sz], _i32),
+    "jsgrad_hip_copy": ([_vp, _vp, _sz], _i32),
+    "jsgrad_hip_memset": ([_vp, _i32, _sz], _i32),
+    "jsgrad_hip_sync": ([], _i32),
+    "jsgrad_hip_module_load": ([_vp, _sz, _pp], _i32),
+    "jsgrad_hip_module_unload": ([_vp], _i32),
+    "jsgrad_hip_module_get": ([_vp, C.c_char_p, _pp], _i32),
+    "jsgrad_hip_launch": ([_vp, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), _pp, _i32, C.POINTER(C.c_int32), _i32, _i32, C.POINTER(C.c_double)], _i32),
+    "jsgrad_hip_event_create": ([_pp], _i32),
+    "jsgrad_hip_event_record": ([_vp], _i32),
+    "jsgrad_hip_event_elapsed_ms": ([_vp, _vp, C.POINTER(_f32)], _i32),
+    "jsgrad_hip_event_destroy": ([_vp], _i32),
+    "jsgrad_hip_graph_begin": ([], _i32),
+    "jsgrad_hip_graph_end": ([_pp], _i32),
+    "jsgrad_hip_graph_launch": ([_vp], _i32),
+    "jsgrad_hip_graph_destroy": ([_vp], _i32),
+    "jsgrad_hip_rope_table": ([_vp, _i32, _i32, _f32, _i32], _i32),
+    "jsgrad_hip_embed": ([_i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32], _i32),
+    "jsgrad_hip_rmsnorm": ([_vp, _vp, _vp, _i32, _f32, _i32], _i32),
+    "jsgrad_hip_linear": ([_i32, _vp, _vp, _i32, _i32, _vp, _vp, _vp, _f32, _vp, _i32], _i32),
+    "jsgrad_hip_qkv_rope": ([_i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32], _i32),
+    "jsgrad_hip_attn_workspace_bytes": ([_i32, _i32, _i32], _sz),
+    "jsgrad_hip_attn_decode": ([_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32], _i32),
+    "jsgrad_hip_ffn_gate": ([_i32, _vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _i32, _i32, _i32], _i32),
+    "jsgrad_hip_argmax": ([_vp, _i32, _vp, _vp, _i32, _i32], _i32),
+    "jsgrad_hip_int8_quantize": ([_vp, _i32, _i32, _vp, _vp, _i32], _i32),
+    "jsgrad_hip_int8_dequant": ([_vp, _vp, _i32, _i32, _vp], _i32),
+    "jsgrad_hip_nf4_quantize": ([_vp, _sz, _vp, _vp, _i32], _i32),
+    "jsgrad_hip_nf4_dequant": ([_vp, _vp, _sz, _vp], _i32),
+    "jsgrad_hip_randn": ([_vp, _sz, _i32, _u64, _f32], _i32),
+    "jsgrad_hip_fill": ([_vp, _sz, _i32, _f32], _i32),
+}
+
+_lib: C.CDLL | None = None
+
+
+def load() -> C.CDLL:
+    """dlopen the library and type every entry point.  No GPU call is made."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise HipError(f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+                           "(make -C denograd_amd/csrc); there is no CPU fallback")
+        lib = C.CDLL(LIB_PATH)
+        for name, (args, res) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.argtypes, fn.restype = args, res
+        _lib = lib
+    return _lib
+
+
+def check(status: int) -> None:
+    if status != 0:
+        raise HipError(load().jsgrad_hip_last_error().decode(errors="replace"))

@@ -1,0 +1,240 @@
+"""Llama decoder on the HIP device: the classes of /root/reference/jsgrad/models/llama.ts with the same
+names, constructor arguments and call order, executing hand-written gfx950 kernels instead of a lazy graph.
+
+Decode (one token, one sequence) is five launches per layer:
+  attention_norm + wq/wk/wv + rotary + KV-cache write | GQA attention over the cache | wo + residual |
+  ffn_norm + w1/w3 + SwiGLU | w2 + residual
+plus the embedding gather, final norm + lm_head, and the greedy argmax.  The token id and start_pos live
+in a device int32[2] (`state`) that the kernels read, so the whole step is position-independent and can
+be captured once as a HIP graph (the role TinyJit's symbolic `start_pos` plays at llama.ts:214-220).
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import ffi
+from .ffi import check
+from .nn import Embedding, Linear, RMSNorm, act_code
+from .tensor import Tensor
+
+
+def precompute_freqs_cis(dim: int, end: int, theta: float = 10000.0, dtype: str = "float32", device: str = "HIP") -> Tensor:
+    """llama.ts:10-14 -> [1, end, 1, dim//2, 2] (cos, sin); `dtype` applies the cast of llama.ts:205."""
+    t = Tensor.empty((1, end, 1, dim // 2, 2), dtype, device)
+    check(ffi.load().jsgrad_hip_rope_table(t.ptr, dim, end, float(theta), act_code(dtype)))
+    return t
+
+
+class Attention:
+    def __init__(self, dim: int, n_heads: int, n_kv_heads: int | None, max_context: int, linear=Linear):
+        self.n_heads = n_heads
+        self.n_kv_heads = n_kv_heads if n_kv_heads is not None else n_heads
+        self.head_dim = dim // n_heads
+        self.n_rep = self.n_heads // self.n_kv_heads
+        self.max_context = max_context
+        self.dim = dim
+        self.wq = linear(dim, self.n_heads * self.head_dim, False)
+        self.wk = linear(dim, self.n_kv_heads * self.head_dim, False)
+        self.wv = linear(dim, self.n_kv_heads * self.head_dim, False)
+        self.wo = linear(self.n_heads * self.head_dim, dim, False)
+        self.cache_kv: Tensor | None = None
+
+    def _ensure_cache(self, dtype: str, device: str) -> None:
+        # Tensor.zeros([2, bsz, max_context, n_kv_heads, head_dim]) (llama.ts:78-80), bsz = 1
+        if self.cache_kv is None:
+            self.cache_kv = Tensor.zeros((2, 1, self.max_context, self.n_kv_heads, self.head_dim), dtype, device)
+
+    def call(self, x: Tensor, state: Tensor, freqs_cis: Tensor, norm: RMSNorm, ctx: "_Scratch") -> Tensor:
+        """x: the block input row; returns x + wo(attention(norm(x))) in ctx.h2."""
+        lib = ffi.load()
+        act = act_code(x.dtype)
+        self._ensure_cache(x.dtype, x.device)
+        half = self.cache_kv.nbytes // 2
+        ck, cv = self.cache_kv.ptr, self.cache_kv.ptr + half
+        sp = lambda l: l.scale.ptr if l.scale is not None else None
+        check(lib.jsgrad_hip_qkv_rope(self.wq.kind, self.wq.weight.ptr, sp(self.wq), self.wk.weight.ptr, sp(self.wk), self.wv.weight.ptr, sp(self.wv),
+                                      x.ptr, norm.weight.ptr, norm.eps, freqs_cis.ptr, state.ptr, ctx.q.ptr, ck, cv,
+                                      self.dim, self.n_heads, self.n_kv_heads, self.head_dim, self.max_context, act))
+        check(lib.jsgrad_hip_attn_decode(ctx.q.ptr, ck, cv, state.ptr, ctx.attn.ptr, ctx.workspace.ptr,
+                                         self.n_heads, self.n_kv_heads, self.head_dim, self.max_context, act))
+        return self.wo.call(ctx.attn, out=ctx.h2, residual=x)
+
+
+class FeedForward:
+    def __init__(self, dim: int, hidden_dim: int, linear=Linear):
+        self.dim, self.hidden_dim = dim, hidden_dim
+        self.w1 = linear(dim, hidden_dim, False)
+        self.w2 = linear(hidden_dim, dim, False)
+        self.w3 = linear(dim, hidden_dim, False)  # the gate in Gated Linear Unit
+
+    def call(self, x: Tensor, norm: RMSNorm, ctx: "_Scratch", out: Tensor) -> Tensor:
+        """out = x + w2( silu(w1 n) * (w3 n) ), n = norm(x)  (SwiGLU, llama.ts:108-110 with the residual of :126)."""
+        sp = lambda l: l.scale.ptr if l.scale is not None else None
+        check(ffi.load().jsgrad_hip_ffn_gate(self.w1.kind, self.w1.weight.ptr, sp(self.w1), self.w3.weight.ptr, sp(self.w3), x.ptr, norm.weight.ptr, norm.eps,
+                                             ctx.g.ptr, self.dim, self.hidden_dim, act_code(x.dtype)))
+        return self.w2.call(ctx.g, out=out, residual=x)
+
+
+class TransformerBlock:
+    def __init__(self, dim: int, hidden_dim: int, n_heads: int, n_kv_heads: int | None, norm_eps: float, max_context: int, linear=Linear, feed_forward=FeedForward):
+        self.attention = Attention(dim, n_heads, n_kv_heads, max_context, linear)
+        self.feed_forward = feed_forward(dim, hidden_dim, linear)
+        self.attention_norm = RMSNorm(dim, norm_eps)
+        self.ffn_norm = RMSNorm(dim, norm_eps)
+
+    def call(self, x: Tensor, state: Tensor, freqs_cis: Tensor, ctx: "_Scratch") -> Tensor:
+        h = self.attention.call(x, state, freqs_cis, self.attention_norm, ctx)     # ctx.h2
+        return self.feed_forward.call(h, self.ffn_norm, ctx, out=x)                # back into x
+
+
+class _Scratch:
+    """Per-model activation rows and the attention workspace, allocated once (nothing is allocated per token)."""
+
+    def __init__(self, dim: int, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int, vocab: int, dtype: str, device: str):
+        self.h = Tensor.empty((dim,), dtype, device)
+        self.h2 = Tensor.empty((dim,), dtype, device)
+        self.q = Tensor.empty((n_heads * head_dim,), dtype, device)
+        self.attn = Tensor.empty((n_heads * head_dim,), dtype, device)
+        self.g = Tensor.empty((hidden,), dtype, device)
+        self.logits = Tensor.empty((vocab,), dtype, device)
+        nbytes = ffi.load().jsgrad_hip_attn_workspace_bytes(n_heads, n_kv_heads, head_dim)
+        self.workspace = Tensor.zeros((nbytes,), "uint8", device)
+
+
+class TinyJit:
+    """Capture-and-replay of one decode step (engine/jit.ts:236-352): call 0 runs eagerly, call 1 runs and is
+    captured into a HIP graph, later calls replay the graph."""
+
+    def __init__(self, fxn):
+        self.fxn, self.cnt, self.graph = fxn, 0, C.c_void_p()
+        self.on_replay = None   # host bookkeeping that the captured function would have done
+
+    def call(self, *args):
+        lib = ffi.load()
+        if self.cnt == 0:
+            ret = self.fxn(*args)
+        elif self.cnt == 1:
+            check(lib.jsgrad_hip_graph_begin())
+            try:
+                ret = self.fxn(*args)
+            finally:
+                check(lib.jsgrad_hip_graph_end(C.byref(self.graph)))
+            self._ret = ret
+            check(lib.jsgrad_hip_graph_launch(self.graph))   # capture records, it does not execute
+        else:
+            check(lib.jsgrad_hip_graph_launch(self.graph))
+            ret = self._ret
+            if self.on_replay is not None:
+                self.on_replay()
+        self.cnt += 1
+        return ret
+
+    def reset(self):
+        if self.graph:
+            ffi.load().jsgrad_hip_graph_destroy(self.graph)
+        self.cnt, self.graph = 0, C.c_void_p()
+
+
+class Transformer:
+    def __init__(self, dim: int, hidden_dim: int, n_heads: int, n_layers: int, norm_eps: float, vocab_size: int, linear=Linear, embedding=Embedding,
+                 n_kv_heads: int | None = None, rope_theta: float = 10000, max_context: int = 1024, jit: bool = True, feed_forward=FeedForward, device: str = "HIP"):
+        self.dim, self.hidden_dim, self.n_heads, self.vocab_size, self.max_context = dim, hidden_dim, n_heads, vocab_size, max_context
+        self.n_kv_heads = n_kv_heads if n_kv_heads is not None else n_heads
+        self.rope_theta, self.device = rope_theta, device
+        self.layers = [TransformerBlock(dim, hidden_dim, n_heads, n_kv_heads, norm_eps, max_context, linear, feed_forward) for _ in range(n_layers)]
+        self.norm = RMSNorm(dim, norm_eps)
+        self.tok_embeddings = embedding(vocab_size, dim)
+        self.output = Linear(dim, vocab_size, False) if embedding is Embedding else linear(dim, vocab_size, False)
+        self.freqs_cis: Tensor | None = None          # built on first use in the activation dtype (llama.ts:198,205)
+        self.forward_jit = TinyJit(self._step) if jit else None
+        if self.forward_jit is not None:
+            self.forward_jit.on_replay = self._advance_host_pos
+        self.state = Tensor(np.zeros(2, np.int32), device=device)            # {token, start_pos}
+        self.tokens_out = Tensor.zeros((max_context,), "int32", device)      # token produced at each start_pos
+        self._ctx: _Scratch | None = None
+        self._pos = 0                                                        # host mirror of state[1]
+
+    # ---- plumbing
+    @property
+    def dtype(self) -> str:
+        return self.tok_embeddings.out_dtype
+
+    def _prepare(self) -> _Scratch:
+        if self._ctx is None:
+            hd = self.dim // self.n_heads
+            self._ctx = _Scratch(self.dim, self.hidden_dim, self.n_heads, self.n_kv_heads, hd, self.vocab_size, self.dtype, self.device)
+            self.freqs_cis = precompute_freqs_cis(hd, self.max_context * 2, self.rope_theta, self.dtype, self.device)
+            for layer in self.layers:
+                layer.attention._ensure_cache(self.dtype, self.device)
+        return self._ctx
+
+    def _step(self) -> Tensor:
+        """One decode step for the token / position in `state`; leaves the greedy token in state[0] and
+        advances state[1].  Pure kernel launches: safe to capture."""
+        ctx = self._prepare()
+        if self._pos >= self.max_context:
+            raise ValueError(f"KV cache of {self.max_context} positions is full")
+        self._pos += 1
+        h = self.tok_embeddings.call(self.state, out=ctx.h)
+        for layer in self.layers:
+            h = layer.call(h, self.state, self.freqs_cis, ctx)
+        self.output.call(h, out=ctx.logits, norm=self.norm)
+        check(ffi.load().jsgrad_hip_argmax(ctx.logits.ptr, self.vocab_size, self.state.ptr, self.tokens_out.ptr, 1, act_code(self.dtype)))
+        return Tensor(buffer=self.state.lazydata.view(1, "int32", 0), shape=(), dtype="int32", device=self.device)
+
+    def _advance_host_pos(self) -> None:
+        self._pos += 1
+
+    def set_state(self, token: int, start_pos: int) -> None:
+        if not (0 <= start_pos < self.max_context):
+            raise ValueError(f"start_pos {start_pos} outside the KV cache of {self.max_context} positions")
+        if not (0 <= token < self.vocab_size):
+            raise ValueError(f"token {token} outside the vocabulary of {self.vocab_size}")
+        self.state.lazydata.copyin(np.array([token, start_pos], np.int32))
+        self._pos = start_pos
+
+    @property
+    def logits(self) -> Tensor:
+        """lm_head output of the last step, `.float()` of llama.ts:210 left to the caller (`numpy().astype`)."""
+        return self._prepare().logits
+
+    # ---- the reference's entry points
+    def forward(self, tokens, start_pos: int, temperature: float = 0.0, top_k: int = 0, top_p: float = 0.8, alpha_f: float = 0.0, alpha_p: float = 0.0) -> Tensor:
+        """llama.ts:201-213 for one sequence.  Several tokens are fed position by position (the reference's own
+        prefill is token-serial, models/llama3.ts:307-311); the returned tensor is the greedy token of the last one."""
+        if temperature >= 1e-6:
+            raise NotImplementedError("only greedy decoding (temperature 0 -> argmax, llama.ts:137) is built on this device")
+        toks = np.asarray(tokens.numpy() if isinstance(tokens, Tensor) else tokens, np.int32)
+        if toks.ndim != 2 or toks.shape[0] != 1:
+            raise ValueError(f"tokens must have shape [1, seqlen], got {toks.shape}")
+        ret = None
+        for i, t in enumerate(toks[0]):
+            self.set_state(int(t), start_pos + i)
+            ret = self._step()
+        return ret
+
+    def call(self, tokens, start_pos: int, temperature: float = 0.0, top_k: int = 0, top_p: float = 0.8, alpha_f: float = 0.0, alpha_p: float = 0.0) -> Tensor:
+        """llama.ts:214-220: single-token calls past position 0 go through the jit (a captured graph)."""
+        toks = np.asarray(tokens.numpy() if isinstance(tokens, Tensor) else tokens, np.int32)
+        if toks.shape == (1, 1) and self.forward_jit is not None and start_pos != 0:
+            if temperature >= 1e-6:
+                raise NotImplementedError("only greedy decoding (temperature 0 -> argmax, llama.ts:137) is built on this device")
+            self.set_state(int(toks[0, 0]), start_pos)
+            return self.forward_jit.call()
+        return self.forward(toks, start_pos, temperature, top_k, top_p, alpha_f, alpha_p)
+
+    def generate(self, n_steps: int) -> None:
+        """Free-running greedy decode: n_steps replays with the token fed back on the device (state[0] -> embedding),
+        no host round trip per token.  Tokens land in `tokens_out[start_pos]`."""
+        if n_steps <= 0:
+            return
+        if self.forward_jit is None:
+            for _ in range(n_steps):
+                self._step()
+            return
+        if self._pos + n_steps > self.max_context:
+            raise ValueError(f"{n_steps} steps from position {self._pos} overrun the KV cache of {self.max_context} positions")
+        for _ in range(n_steps):
+            self.forward_jit.call()

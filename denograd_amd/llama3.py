@@ -1,0 +1,237 @@
+"""Weight-only-quantised layers and the user-facing Llama3 runner of
+/root/reference/jsgrad/models/llama3.ts on the HIP device.
+
+Int8Linear / Int8Embedding / NF4Linear keep the reference's storage (int8 codes + one fp16 scale per output
+row; two 4-bit codes per byte + one fp16 scale per 64 elements) and its quantisers; `call` runs the fused
+dequantising GEMV.  Llama3 drives a Transformer the way the reference does: token-serial prefill, greedy
+decode, per-token `.item()`; `generate` is the free-running variant that keeps the token on the device.
+Downloading checkpoints and the tokenizer are out of scope here: a model is built from a state dict
+(host arrays, a .safetensors file, or seeded random-init weights made on the device).
+"""
+from __future__ import annotations
+
+import time
+
+import numpy as np
+
+from . import ffi, synthetic
+from .device import DTYPES
+from .ffi import check
+from .llama import Transformer
+from .nn import Embedding, Linear, act_code
+from .state import load_state_dict, safe_load
+from .tensor import Tensor
+
+
+class Int8Linear(Linear):
+    """llama3.ts:27-61."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = False):
+        if bias is not False:
+            raise ValueError("Int8Linear bias has to be false")
+        super().__init__(in_features, out_features, False)
+
+    @staticmethod
+    def quantize(tensors: dict[str, Tensor], device=None, scale_dtype: str = "float16", quantize_embeds: bool = False) -> dict[str, Tensor]:
+        """llama3.ts:37-60: every `feed_forward` / `attention.w` weight (and the embedding table when asked) becomes
+        int8 codes + a `.scale`; with quantised embeddings the lm_head shares the table."""
+        if scale_dtype != "float16":
+            raise NotImplementedError("scales are fp16 on this device")
+        lib = ffi.load()
+        new_tensors: dict[str, Tensor] = {}
+        for name, v in tensors.items():
+            if "feed_forward" in name or "attention.w" in name or (quantize_embeds and "tok_embeddings.weight" in name):
+                if "weight" not in name:
+                    raise ValueError(name)
+                out_f, in_f = v.shape
+                codes = Tensor.empty((out_f, in_f), "int8", v.device)
+                scale = Tensor.empty((out_f,), "float16", v.device)
+                check(lib.jsgrad_hip_int8_quantize(v.ptr, out_f, in_f, codes.ptr, scale.ptr, act_code(v.dtype)))
+                new_tensors[name] = codes
+                new_tensors[name.replace("weight", "scale")] = scale
+            else:
+                new_tensors[name] = v
+        if quantize_embeds:
+            new_tensors["output.weight"] = new_tensors["tok_embeddings.weight"]
+            new_tensors["output.scale"] = new_tensors["tok_embeddings.scale"]
+        return new_tensors
+
+
+class Int8Embedding(Embedding):
+    """llama3.ts:63-78: int8 table + fp16 row scales; `call` gathers RN16(code * scale[row])."""
+
+
+def NF4Linear(block_size: int):
+    """llama3.ts:79-117; only block_size 64 (what Llama3 uses, llama3.ts:198) is built."""
+    if block_size != 64:
+        raise NotImplementedError("NF4 kernels are built for block_size 64")
+
+    class _NF4Linear(Linear):
+        def __init__(self, in_features: int, out_features: int, bias: bool = False):
+            if bias:
+                raise ValueError("bias not supported")
+            super().__init__(in_features, out_features, False)
+
+        @staticmethod
+        def quantize(state_dict: dict[str, Tensor], device=None, scale_dtype: str = "float16") -> dict[str, Tensor]:
+            if scale_dtype != "float16":
+                raise NotImplementedError("scales are fp16 on this device")
+            lib = ffi.load()
+            new_state_dict: dict[str, Tensor] = {}
+            for k, v in state_dict.items():
+                if "feed_forward" in k or "attention.w" in k:
+                    n = v.numel
+                    packed = Tensor.empty((n // 2,), "uint8", v.device)
+                    scale = Tensor.empty((n // block_size, 1), "float16", v.device)
+                    check(lib.jsgrad_hip_nf4_quantize(v.ptr, n, packed.ptr, scale.ptr, act_code(v.dtype)))
+                    new_state_dict[k] = packed
+                    new_state_dict[k.replace(".weight", ".scale")] = scale
+                else:
+                    new_state_dict[k] = v
+            return new_state_dict
+
+    return _NF4Linear
+
+
+MODEL_PARAMS = {
+    "1B": {"args": {"dim": 2048, "n_heads": 32, "n_kv_heads": 8, "n_layers": 16, "norm_eps": 1e-5, "rope_theta": 500000, "vocab_size": 128256, "hidden_dim": 8192}, "files": 1},
+    "8B": {"args": {"dim": 4096, "n_heads": 32, "n_kv_heads": 8, "n_layers": 32, "norm_eps": 1e-5, "rope_theta": 500000, "vocab_size": 128256, "hidden_dim": 14336}, "files": 1},
+    "70B": {"args": {"dim": 8192, "n_heads": 64, "n_kv_heads": 8, "n_layers": 80, "norm_eps": 1e-5, "rope_theta": 500000, "vocab_size": 128256, "hidden_dim": 28672}, "files": 8},
+}
+
+
+def _classes(quantize: str | None):
+    """llama3.ts:193-199."""
+    if quantize == "int8":
+        return Int8Linear, Int8Embedding, True
+    if quantize == "nf4":
+        return NF4Linear(64), Embedding, False
+    return Linear, Embedding, False
+
+
+class Llama3:
+    """llama3.ts:170-338 without the download / tokenizer plumbing: construct from shape parameters (`size` or an
+    explicit `args` dict), load a state dict, then `_prefill` / `_call` / `generate` token ids."""
+
+    def __init__(self, size: str | None = None, quantize: str | None = None, device: str = "HIP", max_context: int = 8192, temperature: float = 0.0,
+                 top_k: int = 0, top_p: float = 0.0, alpha_f: float = 0.0, alpha_p: float = 0.0, args: dict | None = None):
+        self.size, self.quantize, self.device, self.max_context = size, quantize, device, max_context
+        self.temperature, self.top_k, self.top_p, self.alpha_f, self.alpha_p = temperature, top_k, top_p, alpha_f, alpha_p
+        self.linear, self.embedding, self.quantize_embeds = _classes(quantize)
+        params = dict(MODEL_PARAMS[size]["args"]) if args is None else dict(args)
+        self.params = params
+        self.model = Transformer(params["dim"], params["hidden_dim"], params["n_heads"], params["n_layers"], params["norm_eps"], params["vocab_size"],
+                                 self.linear, self.embedding, params.get("n_kv_heads"), params["rope_theta"], self.max_context, True, device=device)
+        self.start_pos = 0
+        self.last_seen_toks: list[int] = []
+
+    # ---- loading
+    @staticmethod
+    def from_config(cfg: dict, device: str = "HIP") -> "Llama3":
+        args = {k: cfg[k] for k in ("dim", "hidden_dim", "n_heads", "n_kv_heads", "n_layers", "norm_eps", "rope_theta", "vocab_size")}
+        q = cfg["quantize"] if cfg["quantize"] in ("int8", "nf4") else None
+        return Llama3(quantize=q, device=device, max_context=cfg["max_context"], args=args)
+
+    def load_weights(self, weights: dict, quantized: bool = False) -> "Llama3":
+        """llama3.ts:233-255: `weights` holds unquantised Meta-style tensors (host arrays or device Tensors) unless
+        `quantized` says the codes and scales are already there; quantise per self.quantize, then load."""
+        dev = {k: (v if isinstance(v, Tensor) else Tensor(np.ascontiguousarray(v), device=self.device)) for k, v in weights.items()}
+        if not quantized:
+            if self.quantize == "int8":
+                dev = Int8Linear.quantize(dev, self.device, "float16", self.quantize_embeds)
+            elif self.quantize == "nf4":
+                dev = self.linear.quantize(dev, self.device, "float16")
+        load_state_dict(self.model, dev, strict=False)
+        return self
+
+    def load(self, fn: str) -> "Llama3":
+        return self.load_weights(safe_load(fn))
+
+    def random_init(self, seed: int = 0, std: float = 0.02, tied: bool = True) -> "Llama3":
+        """Seeded N(0, std) weights generated on the device in fp16 (fp32 for a float32 model is not offered here),
+        quantised on the device; RMSNorm weights are ones.  For shapes too large to ship from the host."""
+        p, sd, i = self.params, {}, 0
+        cfg = dict(p, quantize=self.quantize, act_dtype="float16")
+
+        def randn(shape):
+            nonlocal i
+            i += 1
+            return Tensor.randn(shape, "float16", seed * 100003 + i, std, self.device)
+
+        def quantise_one(name, t):
+            one = {name: t}
+            if self.quantize == "int8":
+                return Int8Linear.quantize(one, self.device, "float16", "tok_embeddings" in name and self.quantize_embeds)
+            if self.quantize == "nf4":
+                return self.linear.quantize(one, self.device, "float16")
+            return one
+
+        sd.update({k: v for k, v in quantise_one("tok_embeddings.weight", randn((p["vocab_size"], p["dim"]))).items() if k.startswith("tok_embeddings")})
+        for l in range(p["n_layers"]):
+            for name, shp in synthetic.linear_shapes(cfg).items():
+                sd.update(quantise_one(f"layers.{l}.{name}.weight", randn(shp)))   # the fp16 source is freed right after
+            sd[f"layers.{l}.attention_norm.weight"] = Tensor.ones((p["dim"],), "float16", self.device)
+            sd[f"layers.{l}.ffn_norm.weight"] = Tensor.ones((p["dim"],), "float16", self.device)
+        sd["norm.weight"] = Tensor.ones((p["dim"],), "float16", self.device)
+        if self.quantize_embeds or tied:
+            sd["output.weight"] = sd["tok_embeddings.weight"]
+            if "tok_embeddings.scale" in sd:
+                sd["output.scale"] = sd["tok_embeddings.scale"]
+        else:
+            sd["output.weight"] = randn((p["vocab_size"], p["dim"]))
+        load_state_dict(self.model, sd, strict=False)
+        return self
+
+    # ---- inference (token ids in, token ids out)
+    def _call(self, tok: int) -> int:
+        """llama3.ts:334-337: one model call and the per-token device->host read."""
+        res = self.model.call(np.array([[tok]], np.int32), self.start_pos, self.temperature, self.top_k, self.top_p, self.alpha_f, self.alpha_p)
+        return int(res.item())
+
+    def _prefill(self, toks: list[int]) -> None:
+        """llama3.ts:297-312: skip the shared prefix of the previous prompt when starting over, then feed tokens one at a time."""
+        toks = [int(t) for t in toks]
+        if self.start_pos == 0:
+            same = all(a == b for a, b in zip(toks, self.last_seen_toks))
+            i = min(len(toks), len(self.last_seen_toks)) if same else 0
+            self.start_pos += i
+            self.last_seen_toks = toks
+            toks = toks[i:]
+        for tok in toks:
+            self._call(tok)
+            self.start_pos += 1
+
+    def chat_tokens(self, toks: list[int], max_new_tokens: int, stop_tokens=()) -> dict:
+        """The loop of Llama3.chat (llama3.ts:270-296) on token ids: prefill all but the last prompt token, then decode
+        greedily, syncing once per token as the reference does.  Returns tokens and the reference's usage fields."""
+        st = time.perf_counter()
+        self._prefill(toks[:-1])
+        ttft = time.perf_counter() - st
+        last, out = int(toks[-1]), []
+        st = time.perf_counter()
+        while len(out) < max_new_tokens:
+            tok = self._call(last)
+            self.start_pos += 1
+            out.append(tok)
+            last = tok
+            if tok in stop_tokens:
+                break
+        dt = time.perf_counter() - st
+        return {"tokens": out, "usage": {"input_tokens": len(toks) - 1, "output_tokens": len(out), "time_to_first_token": ttft,
+                                          "tokens_per_second": len(out) / dt if dt > 0 else float("inf")}}
+
+    def generate(self, prompt, n_new: int) -> np.ndarray:
+        """Token-serial prefill, then n_new greedy tokens with the token fed back on the device (no per-token host
+        sync); one read of the token history at the end."""
+        prompt = [int(t) for t in prompt]
+        self._prefill(prompt[:-1])
+        first_pos = self.start_pos
+        first = self._call(prompt[-1])
+        self.start_pos += 1
+        if n_new > 1:
+            self.model.generate(n_new - 1)
+            self.start_pos += n_new - 1
+        hist = self.model.tokens_out.numpy()
+        out = hist[first_pos:first_pos + n_new].astype(np.int32)
+        assert out[0] == first
+        return out

@@ -1,0 +1,156 @@
+/*
+ * jsgrad_hip.h -- C ABI of libjsgrad_hip.so, the MI355X (gfx950) backend for jsgrad's
+ * Llama-3 inference path.
+ *
+ * Plain C: `int` status returns (0 = ok, non-zero = error; text via jsgrad_hip_last_error),
+ * no C++ types and no exceptions across the boundary.  Every pointer is a DEVICE pointer
+ * unless its name starts with `host_`.  All work is queued on one library-owned HIP stream
+ * (default priority); calls are asynchronous unless stated otherwise.  The caller is a
+ * single thread (a JS event loop through Deno.dlopen, or Python ctypes); the library takes
+ * no locks.
+ *
+ * Each entry point cites the reference interface it stands behind
+ * (/root/reference/<file>:<line>).
+ */
+#ifndef JSGRAD_HIP_H
+#define JSGRAD_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* dtype of activations / tables: jsgrad dtypes.float32 and dtypes.float16 (jsgrad/dtype.ts) */
+enum { JSGRAD_F32 = 0, JSGRAD_F16 = 1 };
+/* storage of a Linear weight: nn.Linear float32 / float16 (jsgrad/nn/index.ts:403-412),
+ * Int8Linear int8 + per-output-row fp16 scale (jsgrad/models/llama3.ts:27-36),
+ * NF4Linear(64) two 4-bit codes per byte + one fp16 scale per 64 elements (llama3.ts:79-97) */
+enum { JSGRAD_W_F32 = 0, JSGRAD_W_F16 = 1, JSGRAD_W_I8 = 2, JSGRAD_W_NF4 = 3 };
+
+/* ---------------------------------------------------------------------------------
+ * Device, memory, programs: what a `Compiled` device needs (jsgrad/runtime/allocator.ts:166-191)
+ * --------------------------------------------------------------------------------- */
+
+/* Compiled.init (allocator.ts:179; awaited lazily from engine/realize.ts:133,157): select the
+ * device, create the stream.  Idempotent. */
+int jsgrad_hip_init(int device);
+/* Text of the last error on this thread's library state; never NULL. */
+const char *jsgrad_hip_last_error(void);
+/* Device name and gcnArchName ("gfx950...") for the `Device` registry entry (jsgrad/device.ts:26-35). */
+int jsgrad_hip_device_name(char *host_out, size_t cap);
+/* Number of compute units (used to size grids host-side). */
+int jsgrad_hip_cu_count(int *host_out);
+
+/* Allocator._alloc / _free (allocator.ts:40-41).  size 0 is an error as in Allocator.alloc (:30-33).
+ * free may be called at any time (Buffer finalisers, jsgrad/device.ts:72-74): it waits for the stream. */
+int jsgrad_hip_malloc(size_t nbytes, void **host_out_ptr);
+int jsgrad_hip_free(void *ptr);
+/* Allocator._copyin / _copyout (allocator.ts:42-43).  copyout returns after the data is in host memory. */
+int jsgrad_hip_copyin(void *dst, const void *host_src, size_t nbytes);
+int jsgrad_hip_copyout(void *host_dst, const void *src, size_t nbytes);
+/* BufferCopy between two device buffers (engine/realize.ts:92-122, Allocator._transfer allocator.ts:46). */
+int jsgrad_hip_copy(void *dst, const void *src, size_t nbytes);
+/* Tensor.zeros(...).contiguous().realize() for the KV cache (models/llama.ts:79): byte fill. */
+int jsgrad_hip_memset(void *dst, int byte, size_t nbytes);
+/* Compiled.synchronize (allocator.ts:185-186). */
+int jsgrad_hip_sync(void);
+
+/* Program.init(name, lib) (allocator.ts:101-103; ops_clang.ts:30-38 is the CPU counterpart): load a
+ * gfx950 code object and look a kernel up by name. */
+int jsgrad_hip_module_load(const void *host_image, size_t nbytes, void **host_out_module);
+int jsgrad_hip_module_unload(void *module);
+int jsgrad_hip_module_get(void *module, const char *name, void **host_out_function);
+/* Program.call(bufs, {global_size, local_size, vals}, wait) (allocator.ts:104-106, called from
+ * engine/realize.ts:62-80): grid is in BLOCKS, `vals` are int32 kernel arguments appended after the
+ * buffer pointers (ops_clang.ts:46).  With wait != 0 the call blocks and *host_seconds gets the
+ * kernel time measured with HIP events on the library stream. */
+int jsgrad_hip_launch(void *function, const uint32_t host_grid[3], const uint32_t host_block[3], void *const *host_bufs, int nbufs,
+                      const int32_t *host_vals, int nvals, int wait, double *host_seconds);
+
+/* Timing on the library stream (the `wait` contract of Program.call and DEBUG>=2 per-kernel
+ * statistics, engine/realize.ts:168-178). */
+int jsgrad_hip_event_create(void **host_out_event);
+int jsgrad_hip_event_record(void *event);
+int jsgrad_hip_event_elapsed_ms(void *start, void *stop, float *host_out_ms); /* waits for `stop` */
+int jsgrad_hip_event_destroy(void *event);
+
+/* TinyJit capture / replay as a device graph (engine/jit.ts:14-69 apply_graph_to_jit, :71 GraphRunner,
+ * `Compiled.graph` allocator.ts:176): everything queued between begin and end becomes one HIP graph. */
+int jsgrad_hip_graph_begin(void);
+int jsgrad_hip_graph_end(void **host_out_graph);
+int jsgrad_hip_graph_launch(void *graph);
+int jsgrad_hip_graph_destroy(void *graph);
+
+/* ---------------------------------------------------------------------------------
+ * Llama-3 decode kernels (one sequence, one new position).
+ *
+ * `state` is a device int32[2] = { token, start_pos } that the kernels read, so that a captured
+ * graph replays unchanged while start_pos advances (the role of the bound `start_pos` Variable,
+ * models/llama.ts:217).  Activations, norm weights, the RoPE table and the KV cache are in the
+ * activation dtype `act` (JSGRAD_F32 / JSGRAD_F16).
+ * --------------------------------------------------------------------------------- */
+
+/* precompute_freqs_cis(dim=head_dim, end, theta) (models/llama.ts:10-14) followed by the cast to the
+ * activation dtype (llama.ts:205): table [end][head_dim/2][2] = (cos, sin). */
+int jsgrad_hip_rope_table(void *table, int head_dim, int end, float theta, int act);
+
+/* Embedding.call (nn/index.ts:607-619) / Int8Embedding.call (llama3.ts:71-77) for the token in
+ * state[0]: out[dim] = row of the table (int8: RN16(code * scale[row])).  kind: F32 / F16 / I8. */
+int jsgrad_hip_embed(int kind, const void *table, const void *scale, const int32_t *state, void *out, int dim, int vocab, int act);
+
+/* RMSNorm.call (nn/index.ts:586-588) on one row. */
+int jsgrad_hip_rmsnorm(const void *x, const void *weight, void *y, int dim, float eps, int act);
+
+/* Linear.call / Int8Linear.call / NF4Linear.call on one row (nn/index.ts:411, llama3.ts:35,91-97):
+ * y[out_f] = x[in_f] . W^T, float accumulation, result in the activation dtype.
+ * norm_weight != NULL fuses RMSNorm(x) in front (TransformerBlock.call, models/llama.ts:125-126);
+ * residual != NULL adds it after the cast: y = residual + linear (the `x.add(...)` of llama.ts:125-126). */
+int jsgrad_hip_linear(int kind, const void *w, const void *scale, int out_f, int in_f, const void *x, void *y,
+                      const void *norm_weight, float eps, const void *residual, int act);
+
+/* attention_norm + wq/wk/wv + apply_rotary_emb + KV-cache assign (models/llama.ts:61-87) for the
+ * position state[1]: q_out[n_heads*head_dim] gets the rotated query; the rotated key and the value are
+ * written into row state[1] of cache_k / cache_v ([max_context][n_kv_heads][head_dim], one layer). */
+int jsgrad_hip_qkv_rope(int kind, const void *wq, const void *sq, const void *wk, const void *sk, const void *wv, const void *sv,
+                        const void *x, const void *norm_weight, float eps, const void *rope_table, const int32_t *state,
+                        void *q_out, void *cache_k, void *cache_v, int dim, int n_heads, int n_kv_heads, int head_dim, int max_context, int act);
+
+/* repeat_kv + scaled_dot_product_attention over cache rows [0, state[1]] (models/llama.ts:89-95,
+ * tensor.ts:3920-3934), grouped-query: query head h reads kv head h / (n_heads/n_kv_heads).
+ * workspace: jsgrad_hip_attn_workspace_bytes() bytes, zero-filled once before first use. */
+size_t jsgrad_hip_attn_workspace_bytes(int n_heads, int n_kv_heads, int head_dim);
+int jsgrad_hip_attn_decode(const void *q, const void *cache_k, const void *cache_v, const int32_t *state, void *out, void *workspace,
+                           int n_heads, int n_kv_heads, int head_dim, int max_context, int act);
+
+/* ffn_norm + w1, w3 + SwiGLU (FeedForward.call, models/llama.ts:108-110): g[hidden] = silu(w1 x) * (w3 x). */
+int jsgrad_hip_ffn_gate(int kind, const void *w1, const void *s1, const void *w3, const void *s3, const void *x,
+                        const void *norm_weight, float eps, void *g, int dim, int hidden, int act);
+
+/* sample() at temperature 0 (models/llama.ts:137 -> Tensor.argmax tensor.ts:2314-2320): lowest index among
+ * the maxima of logits[n] (activation dtype).  Writes the token to state[0] and, when advance != 0,
+ * increments state[1]; tokens_out != NULL also receives the token at tokens_out[old start_pos]. */
+int jsgrad_hip_argmax(const void *logits, int n, int32_t *state, int32_t *tokens_out, int advance, int act);
+
+/* ---------------------------------------------------------------------------------
+ * Load-time kernels
+ * --------------------------------------------------------------------------------- */
+
+/* Int8Linear.quantize for one [out_f][in_f] matrix given in the activation dtype (llama3.ts:37-60). */
+int jsgrad_hip_int8_quantize(const void *w, int out_f, int in_f, int8_t *codes, void *scale_f16, int act);
+/* weight.cast(half) * scale materialised (llama3.ts:35,75): w16[out_f][in_f] = RN16(code * scale[row]). */
+int jsgrad_hip_int8_dequant(const int8_t *codes, const void *scale_f16, int out_f, int in_f, void *w16);
+/* NF4Linear(64).quantize / the dequantisation of NF4Linear.call for n elements (llama3.ts:91-96,98-114). */
+int jsgrad_hip_nf4_quantize(const void *w, size_t n, uint8_t *packed, void *scale_f16, int act);
+int jsgrad_hip_nf4_dequant(const uint8_t *packed, const void *scale_f16, size_t n, void *w16);
+/* Random-init weights ~ N(0, std) in the given dtype (the role of Tensor.randn / Linear's random
+ * initialisation, nn/index.ts:406-409, for synthetic models); counter-based, reproducible from seed. */
+int jsgrad_hip_randn(void *out, size_t n, int dtype, uint64_t seed, float std);
+/* Fill n elements of the given dtype with a constant (Tensor.ones for RMSNorm weights, nn/index.ts:583). */
+int jsgrad_hip_fill(void *out, size_t n, int dtype, float value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* JSGRAD_HIP_H */

@@ -1,0 +1,296 @@
+"""Per-kernel parity of the HIP path against the CPU oracle, through the C ABI.  Integer / byte results
+(quantiser codes, scales, dequantised weights, argmax indices, gathered rows) must be bit-exact; floating
+point results must agree within the tolerance written in each test (north star: rtol/atol 1e-2 for fp16)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle as orc
+from denograd_amd import ffi
+from denograd_amd.ffi import check
+from denograd_amd.tensor import Tensor
+
+pytestmark = pytest.mark.gpu
+RNG = np.random.default_rng(11)
+NPDT = {"float32": np.float32, "float16": np.float16}
+
+
+def act_code(dt): return ffi.F16 if dt == "float16" else ffi.F32
+def f32(t): return t.numpy().astype(np.float32)
+
+
+def assert_close(got, ref, act16, what="", composed=False):
+    """Two layers: the north-star tolerance (1e-2 of the output scale for fp16 activations, 1e-4 for float32), and the
+    much tighter statement that the two paths differ only by float summation order: at most 2 ulp of the activation
+    dtype (plus float summation noise at the output scale, which matters for results that cancel) and mostly identical values."""
+    got, ref = np.asarray(got, np.float32), np.asarray(ref, np.float32)
+    scale = max(1.0, float(np.abs(ref).max()))
+    assert np.max(np.abs(got - ref)) <= (1e-2 if act16 else 1e-4) * scale, what
+    if act16:
+        ulp = np.spacing(np.abs(ref).astype(np.float16)).astype(np.float32)
+        if composed:   # a fused RMSNorm in front: a few inputs differ by one fp16 ulp, which moves every output a little
+            assert np.all(np.abs(got - ref) <= 4 * ulp + scale * 2.0 ** -11), what
+            assert np.mean(got == ref) > 0.5, what
+        else:
+            assert np.all(np.abs(got - ref) <= 2 * ulp + scale * 2.0 ** -18), what    # + float-sum noise for results that cancel to ~0
+            assert np.mean(got == ref) > 0.9, what
+    else:
+        assert np.all(np.abs(got - ref) <= scale * 2.0 ** (-15 if composed else -18)), what
+
+
+def test_device_is_gfx950(hip):
+    buf = C.create_string_buffer(256)
+    check(hip.jsgrad_hip_device_name(buf, 256))
+    assert b"gfx950" in buf.value
+    n = C.c_int()
+    check(hip.jsgrad_hip_cu_count(C.byref(n)))
+    assert n.value >= 64
+
+
+def test_copy_roundtrip_and_memset(hip):
+    x = RNG.integers(0, 255, 100003, dtype=np.uint8)
+    t = Tensor(x)
+    assert np.array_equal(t.numpy(), x)
+    check(hip.jsgrad_hip_memset(t.ptr, 0x5A, 100003))
+    assert np.all(t.numpy() == 0x5A)
+    z = Tensor.zeros((4096,), "float32")
+    assert np.all(z.numpy() == 0)
+    with pytest.raises(ffi.HipError, match="positive"):
+        p = C.c_void_p()
+        check(hip.jsgrad_hip_malloc(0, C.byref(p)))
+
+
+def test_generic_program_launch(hip):
+    """The reference's device smoke test (cli/devices.ts:4-24): [1,2,3]*2 == [2,4,6] through Compiler + Program."""
+    from denograd_amd.device import Device
+    dev = Device.get("HIP").init()
+    src = 'extern "C" __global__ void E_3(float* data0, const float* data1, const int n) { int i = blockIdx.x*blockDim.x+threadIdx.x; if (i < n) data0[i] = data1[i]*2.0f; }'
+    prg = dev.runtime("E_3", dev.compiler.compile_cached(src))
+    a = Tensor(np.float32([1, 2, 3]))
+    out = Tensor.empty((3,), "float32")
+    secs = prg.call([out.ptr, a.ptr], global_size=(1, 1, 1), local_size=(64, 1, 1), vals=(3,), wait=True)
+    assert np.array_equal(out.numpy(), np.float32([2, 4, 6])) and secs is not None and 0 <= secs < 1.0
+
+
+@pytest.mark.parametrize("dt", ["float32", "float16"])
+def test_rope_table_bit_exact(hip, dt):
+    for hd, end in ((64, 2 * 1024), (128, 2 * 300), (4, 164)):
+        t = Tensor.empty((end, hd // 2, 2), dt)
+        check(hip.jsgrad_hip_rope_table(t.ptr, hd, end, 500000.0, act_code(dt)))
+        ref = orc.freqs_cis(hd, end, 500000.0).astype(NPDT[dt])
+        assert np.array_equal(t.numpy().view(np.uint16 if dt == "float16" else np.uint32), ref.view(np.uint16 if dt == "float16" else np.uint32))
+
+
+def test_int8_quantize_dequant_bit_exact(hip):
+    for dt in ("float16", "float32"):
+        w = (RNG.standard_normal((96, 512)) * 0.02).astype(NPDT[dt])
+        w[7] = 0
+        codes, scale, tw = Tensor.empty(w.shape, "int8"), Tensor.empty((96,), "float16"), Tensor(w)
+        check(hip.jsgrad_hip_int8_quantize(tw.ptr, 96, 512, codes.ptr, scale.ptr, act_code(dt)))
+        q_ref, s_ref = orc.int8_quantize(w.astype(np.float32))
+        assert np.array_equal(codes.numpy(), q_ref) and np.array_equal(scale.numpy().view(np.uint16), s_ref.view(np.uint16))
+    # dequantisation over every code value and awkward scales
+    q = np.tile(np.arange(-128, 128, dtype=np.int8), (64, 2))
+    s = np.concatenate([np.abs(RNG.standard_normal(60)) * 1e-3, [0.0, 6.1e-5, 5.96e-8, 1.0]]).astype(np.float16)
+    out, tq, ts = Tensor.empty(q.shape, "float16"), Tensor(q), Tensor(s)
+    check(hip.jsgrad_hip_int8_dequant(tq.ptr, ts.ptr, 64, 512, out.ptr))
+    assert np.array_equal(out.numpy().view(np.uint16), orc.int8_dequant(q, s).view(np.uint16))
+
+
+def test_nf4_quantize_dequant_bit_exact(hip):
+    for dt in ("float16", "float32"):
+        w = (RNG.standard_normal((32, 256)) * 0.02).astype(NPDT[dt])
+        packed, scale, tw = Tensor.empty((w.size // 2,), "uint8"), Tensor.empty((w.size // 64, 1), "float16"), Tensor(w)
+        check(hip.jsgrad_hip_nf4_quantize(tw.ptr, w.size, packed.ptr, scale.ptr, act_code(dt)))
+        p_ref, s_ref = orc.nf4_quantize(w.astype(np.float32))
+        assert np.array_equal(packed.numpy(), p_ref) and np.array_equal(scale.numpy().view(np.uint16), s_ref.view(np.uint16))
+    allb = np.tile(np.arange(256, dtype=np.uint8), 8)
+    s = np.concatenate([np.abs(RNG.standard_normal(62)) * 0.05, [1.0, 0.0]]).astype(np.float16).reshape(-1, 1)
+    out, tb, ts = Tensor.empty((allb.size * 2,), "float16"), Tensor(allb), Tensor(s)
+    check(hip.jsgrad_hip_nf4_dequant(tb.ptr, ts.ptr, allb.size * 2, out.ptr))
+    assert np.array_equal(out.numpy().view(np.uint16), orc.nf4_dequant(allb, s).view(np.uint16))
+
+
+def make_weight(kind, out_f, in_f, dt):
+    w = (RNG.standard_normal((out_f, in_f)) * 0.05).astype(np.float32)
+    if kind == "f32": return w, None, ffi.W_F32
+    if kind == "f16": return w.astype(np.float16), None, ffi.W_F16
+    if kind == "i8":
+        q, s = orc.int8_quantize(w)
+        return q, s, ffi.W_I8
+    q, s = orc.nf4_quantize(w.astype(np.float16).astype(np.float32))
+    return q, s, ffi.W_NF4
+
+
+LINEAR_CASES = [("f32", "float32", 40, 256), ("f32", "float32", 1024, 768), ("f16", "float16", 72, 512), ("f16", "float16", 2048, 2048), ("f16", "float32", 64, 512),
+                ("i8", "float16", 100, 1024), ("i8", "float16", 4096, 4096), ("i8", "float16", 96, 14336), ("i8", "float32", 64, 256),
+                ("nf4", "float16", 64, 2048), ("nf4", "float16", 130, 4096), ("nf4", "float16", 48, 64)]
+
+
+@pytest.mark.parametrize("kind,dt,out_f,in_f", LINEAR_CASES)
+def test_linear_against_oracle(hip, kind, dt, out_f, in_f):
+    """y = x.W^T (+ fused RMSNorm, + residual).  Tolerance: 1e-2 relative to the output scale for fp16 activations
+    (north star), 1e-4 for float32; in practice the two differ only in float summation order."""
+    w, s, code = make_weight(kind, out_f, in_f, dt)
+    act16 = dt == "float16"
+    x = RNG.standard_normal(in_f).astype(NPDT[dt])
+    res = RNG.standard_normal(out_f).astype(NPDT[dt])
+    nw = (1 + 0.1 * RNG.standard_normal(in_f)).astype(NPDT[dt])
+    tw, ts, tx, tr, tn = Tensor(w), (Tensor(s) if s is not None else None), Tensor(x), Tensor(res), Tensor(nw)
+    y = Tensor.empty((out_f,), dt)
+    tol = 1e-2 if act16 else 1e-4
+    for use_norm in (False, True):
+        for use_res in (False, True):
+            check(hip.jsgrad_hip_linear(code, tw.ptr, ts.ptr if ts else None, out_f, in_f, tx.ptr, y.ptr, tn.ptr if use_norm else None, 1e-5, tr.ptr if use_res else None, act_code(dt)))
+            xin = x.astype(np.float32)
+            if use_norm: xin = orc.rmsnorm(xin, nw.astype(np.float32), 1e-5, act16)
+            ref = orc.linear(w, s, xin, out_f, in_f, act16)[0]
+            if use_res:
+                ref = ref + res.astype(np.float32)
+                if act16: ref = ref.astype(np.float16).astype(np.float32)
+            assert_close(f32(y), ref, act16, (use_norm, use_res), composed=use_norm)
+
+
+def test_linear_rejects_bad_shapes(hip):
+    x, y, w = Tensor.zeros((100,), "float16"), Tensor.zeros((8,), "float16"), Tensor.zeros((8, 100), "int8")
+    with pytest.raises(ffi.HipError, match="multiple of 16"):
+        check(hip.jsgrad_hip_linear(ffi.W_I8, w.ptr, y.ptr, 8, 100, x.ptr, y.ptr, None, 0.0, None, ffi.F16))
+    with pytest.raises(ffi.HipError, match="needs a scale"):
+        check(hip.jsgrad_hip_linear(ffi.W_I8, w.ptr, None, 8, 96, x.ptr, y.ptr, None, 0.0, None, ffi.F16))
+
+
+@pytest.mark.parametrize("dt", ["float32", "float16"])
+def test_rmsnorm_against_oracle(hip, dt):
+    for d in (256, 2048, 3072, 4096):
+        x = (RNG.standard_normal(d) * 2).astype(NPDT[dt])
+        w = (1 + 0.1 * RNG.standard_normal(d)).astype(NPDT[dt])
+        y, tx, tw = Tensor.empty((d,), dt), Tensor(x), Tensor(w)
+        check(hip.jsgrad_hip_rmsnorm(tx.ptr, tw.ptr, y.ptr, d, 1e-5, act_code(dt)))
+        ref = orc.rmsnorm(x.astype(np.float32), w.astype(np.float32), 1e-5, dt == "float16")
+        tol = 1e-2 if dt == "float16" else 1e-5
+        assert np.max(np.abs(f32(y) - ref)) <= tol * np.abs(ref).max()
+        if dt == "float16": assert np.mean(f32(y) == ref) > 0.99
+
+
+@pytest.mark.parametrize("kind", ["f32", "f16", "i8"])
+def test_embedding_gather_bit_exact(hip, kind):
+    V, d = 1000, 256
+    dt = "float32" if kind == "f32" else "float16"
+    w, s, code = make_weight(kind, V, d, dt)
+    tw, ts = Tensor(w), (Tensor(s) if s is not None else None)
+    out = Tensor.empty((d,), dt)
+    for tok in (0, 17, V - 1):
+        st = Tensor(np.int32([tok, 3]))
+        check(hip.jsgrad_hip_embed(code, tw.ptr, ts.ptr if ts else None, st.ptr, out.ptr, d, V, act_code(dt)))
+        if kind == "i8": ref = (w[tok].astype(np.float64) * float(s[tok])).astype(np.float16)
+        else: ref = w[tok]
+        assert np.array_equal(out.numpy().view(np.uint16 if dt == "float16" else np.uint32), ref.view(np.uint16 if dt == "float16" else np.uint32))
+
+
+@pytest.mark.parametrize("dt", ["float32", "float16"])
+def test_argmax_lowest_index_and_state_update(hip, dt):
+    toks = Tensor.zeros((64,), "int32")
+    for n, vals in ((5, [1, 5, 5, 2, 5]), (3, [3, 3, 3]), (3, [-np.inf, -1, -1])):
+        st = Tensor(np.int32([0, 7]))
+        tv = Tensor(np.array(vals, NPDT[dt]))
+        check(hip.jsgrad_hip_argmax(tv.ptr, n, st.ptr, toks.ptr, 1, act_code(dt)))
+        assert list(st.numpy()) == [orc.argmax(vals), 8] and toks.numpy()[7] == orc.argmax(vals)
+    x = RNG.standard_normal(128256).astype(np.float16).astype(NPDT[dt])
+    x[[100000, 2000, 77777]] = x.max() + 1            # three-way tie, lowest index wins
+    st, tx = Tensor(np.int32([0, 0])), Tensor(x)
+    check(hip.jsgrad_hip_argmax(tx.ptr, x.size, st.ptr, None, 0, act_code(dt)))
+    assert list(st.numpy()) == [2000, 0]
+
+
+QKV_CASES = [("f32", "float32", 256, 4, 2, 64), ("f16", "float16", 2048, 32, 8, 64), ("i8", "float16", 1024, 8, 2, 128), ("nf4", "float16", 1024, 8, 8, 128),
+             ("i8", "float16", 768, 6, 2, 128)]
+
+
+@pytest.mark.parametrize("kind,dt,dim,H,KV,hd", QKV_CASES)
+def test_qkv_rope_cache_write(hip, kind, dt, dim, H, KV, hd):
+    """attention_norm + wq/wk/wv + rotary + cache assign (models/llama.ts:61-87) at a non-zero position."""
+    act16, ctx, pos = dt == "float16", 48, 37
+    (wq, sq, code), (wk, sk, _), (wv, sv, _) = make_weight(kind, H * hd, dim, dt), make_weight(kind, KV * hd, dim, dt), make_weight(kind, KV * hd, dim, dt)
+    x = RNG.standard_normal(dim).astype(NPDT[dt])
+    nw = (1 + 0.1 * RNG.standard_normal(dim)).astype(NPDT[dt])
+    table = Tensor.empty((2 * ctx, hd // 2, 2), dt)
+    check(hip.jsgrad_hip_rope_table(table.ptr, hd, 2 * ctx, 500000.0, act_code(dt)))
+    ck, cv = Tensor.zeros((ctx, KV, hd), dt), Tensor.zeros((ctx, KV, hd), dt)
+    q = Tensor.empty((H * hd,), dt)
+    T = lambda a: Tensor(a) if a is not None else None
+    tq, tk, tv, tsq, tsk, tsv = T(wq), T(wk), T(wv), T(sq), T(sk), T(sv)
+    p = lambda t: t.ptr if t is not None else None
+    st, tx, tnw = Tensor(np.int32([0, pos])), Tensor(x), Tensor(nw)
+    check(hip.jsgrad_hip_qkv_rope(code, tq.ptr, p(tsq), tk.ptr, p(tsk), tv.ptr, p(tsv), tx.ptr, tnw.ptr, 1e-5, table.ptr, st.ptr,
+                                  q.ptr, ck.ptr, cv.ptr, dim, H, KV, hd, ctx, act_code(dt)))
+    xn = orc.rmsnorm(x.astype(np.float32), nw.astype(np.float32), 1e-5, act16)
+    fc = orc.freqs_cis(hd, 2 * ctx, 500000.0)[pos].astype(NPDT[dt]).astype(np.float32)
+    q_ref = orc.rope(orc.linear(wq, sq, xn, H * hd, dim, act16)[0], H, hd, fc, act16)
+    k_ref = orc.rope(orc.linear(wk, sk, xn, KV * hd, dim, act16)[0], KV, hd, fc, act16)
+    v_ref = orc.linear(wv, sv, xn, KV * hd, dim, act16)[0]
+    for got, ref in ((f32(q), q_ref), (f32(ck)[pos].reshape(-1), k_ref), (f32(cv)[pos].reshape(-1), v_ref)):
+        assert_close(got, ref, act16, composed=True)
+    rows = np.arange(ctx) != pos
+    assert np.all(f32(ck)[rows] == 0) and np.all(f32(cv)[rows] == 0)      # only row `pos` is written
+    # a position outside the cache must not write anything (and must not fault)
+    st2 = Tensor(np.int32([0, ctx]))
+    before = ck.numpy().copy()
+    check(hip.jsgrad_hip_qkv_rope(code, tq.ptr, p(tsq), tk.ptr, p(tsk), tv.ptr, p(tsv), tx.ptr, tnw.ptr, 1e-5, table.ptr, st2.ptr,
+                                  q.ptr, ck.ptr, cv.ptr, dim, H, KV, hd, ctx, act_code(dt)))
+    assert np.array_equal(ck.numpy(), before)
+
+
+@pytest.mark.parametrize("kind,dt,dim,F", [("f32", "float32", 256, 768), ("f16", "float16", 2048, 8192), ("i8", "float16", 1024, 2816), ("nf4", "float16", 1024, 1000)])
+def test_ffn_gate_swiglu(hip, kind, dt, dim, F):
+    act16 = dt == "float16"
+    (w1, s1, code), (w3, s3, _) = make_weight(kind, F, dim, dt), make_weight(kind, F, dim, dt)
+    x = (RNG.standard_normal(dim) * 3).astype(NPDT[dt])
+    nw = (1 + 0.1 * RNG.standard_normal(dim)).astype(NPDT[dt])
+    T = lambda a: Tensor(a) if a is not None else None
+    t1, t3, ts1, ts3 = T(w1), T(w3), T(s1), T(s3)
+    p = lambda t: t.ptr if t is not None else None
+    g, tx, tnw = Tensor.empty((F,), dt), Tensor(x), Tensor(nw)
+    check(hip.jsgrad_hip_ffn_gate(code, t1.ptr, p(ts1), t3.ptr, p(ts3), tx.ptr, tnw.ptr, 1e-5, g.ptr, dim, F, act_code(dt)))
+    xn = orc.rmsnorm(x.astype(np.float32), nw.astype(np.float32), 1e-5, act16)
+    a, u = orc.linear(w1, s1, xn, F, dim, act16)[0], orc.linear(w3, s3, xn, F, dim, act16)[0]
+    ref = orc.silu(a, act16) * u
+    if act16: ref = ref.astype(np.float16).astype(np.float32)
+    assert_close(f32(g), ref, act16, composed=True)
+
+
+def attn_oracle(q, K, V, H, KV, hd, T, act16):
+    """scores -> softmax -> P.V with the oracle's exp and rounding points, written with numpy around orc.xexp2f."""
+    out = np.empty(H * hd, np.float32)
+    scale = np.float32(1.0 / np.sqrt(hd))
+    for h in range(H):
+        g = h // (H // KV)
+        s = np.array([np.float32(np.dot(q[h * hd:(h + 1) * hd].astype(np.float64), K[t, g].astype(np.float64))) for t in range(T)], np.float32) * scale
+        e = orc.xexp2f(((s - s.max()) * np.float32(1.4426950408889634)).astype(np.float32))
+        p = (e * (np.float32(1) / e.astype(np.float32).sum(dtype=np.float32))).astype(np.float32)
+        if act16: p = p.astype(np.float16).astype(np.float32)
+        o = (p[:, None].astype(np.float64) * V[:T, g].astype(np.float64)).sum(0).astype(np.float32)
+        out[h * hd:(h + 1) * hd] = o.astype(np.float16).astype(np.float32) if act16 else o
+    return out
+
+
+@pytest.mark.parametrize("dt,H,KV,hd,ctx", [("float32", 4, 2, 64, 64), ("float16", 32, 8, 64, 1024), ("float16", 24, 8, 128, 600), ("float16", 8, 8, 128, 300),
+                                             ("float16", 8, 1, 64, 2100), ("float32", 6, 2, 128, 96)])
+def test_attention_decode(hip, dt, H, KV, hd, ctx):
+    """GQA decode attention over the cache for several T, including T=1, chunk boundaries and the full cache;
+    repeated launches share one workspace (the merging block must leave the counters at zero)."""
+    act16 = dt == "float16"
+    K = (RNG.standard_normal((ctx, KV, hd)) * 0.7).astype(NPDT[dt])
+    V = RNG.standard_normal((ctx, KV, hd)).astype(NPDT[dt])
+    q = (RNG.standard_normal(H * hd) * 0.7).astype(NPDT[dt])
+    tK, tV, tq = Tensor(K), Tensor(V), Tensor(q)
+    out = Tensor.empty((H * hd,), dt)
+    ws = Tensor.zeros((hip.jsgrad_hip_attn_workspace_bytes(H, KV, hd),), "uint8")
+    for T in sorted(t for t in {1, 2, 31, 32, 33, 65, ctx // 2 + 1, ctx - 1, ctx} if t <= ctx):
+        st = Tensor(np.int32([0, T - 1]))
+        check(hip.jsgrad_hip_attn_decode(tq.ptr, tK.ptr, tV.ptr, st.ptr, out.ptr, ws.ptr, H, KV, hd, ctx, act_code(dt)))
+        ref = attn_oracle(q.astype(np.float32), K.astype(np.float32), V.astype(np.float32), H, KV, hd, T, act16)
+        tol = 1e-2 if act16 else 1e-4
+        assert np.max(np.abs(f32(out) - ref)) <= tol * max(1.0, np.abs(ref).max()), f"T={T}"
+        assert np.mean(np.abs(f32(out) - ref) <= np.abs(ref) * (2.0 ** -8 if act16 else 2.0 ** -16) + 2e-4) > 0.99, f"T={T}"
+    assert np.all(ws.numpy()[:256] == 0)
