@@ -1,0 +1,243 @@
+#!/usr/bin/env python3
+"""Decode benchmark of the HIP Llama-3 path on one MI355X.
+
+A "step" is one greedy decode step (one token, batch 1) of a seeded random-init model whose weights are
+resident in HBM: the embedding gather, five launches per layer, the lm_head and the argmax, replayed as one
+captured HIP graph with the token fed back on the device.  The primary workload is BASELINE config 2
+(Llama-3.2-1B-shaped, fp16, 512-token prompt, 256 decoded tokens); the north-star shape (Llama-3.1-8B-shaped,
+int8 weight-only, batch 1) is measured in the same run and reported under "secondary".
+
+Prints ONE JSON line.  `roofline` is for the dominant kernel family (the one-row linear kernel behind wo, w2 and
+the lm_head): algorithmic bytes of those launches / their event-timed duration, measured in a separate eager pass
+of the same step with an event pair around every launch.  `step_roofline` is the whole-token figure
+(algorithmic bytes per token x tokens/s / 8 TB/s).  `cpu_baseline` times the CPU oracle (single thread, the way the
+reference's CLANG device runs) on a bounded sample of the same weights and cross-checks its tokens against the GPU.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def linear_bytes(cfg, out_f, in_f):
+    """weight (+ scale) bytes one one-row linear must stream"""
+    q = cfg["quantize"]
+    if q == "int8":
+        return out_f * in_f + out_f * 2
+    if q == "nf4":
+        return out_f * in_f // 2 + (out_f * in_f // 64) * 2
+    return out_f * in_f * 2
+
+
+def kernel_bytes(cfg, T):
+    """algorithmic HBM bytes per decode step of each kernel family at T visible positions"""
+    from denograd_amd import synthetic
+    d, V, L = cfg["dim"], cfg["vocab_size"], cfg["n_layers"]
+    shp = synthetic.linear_shapes(cfg)
+    lb = lambda name: linear_bytes(cfg, *shp[name])
+    head_q = "int8" if cfg["quantize"] == "int8" else None
+    head = (V * d + V * 2) if head_q == "int8" else V * d * 2
+    act = 2
+    return {
+        "qkv_rope": L * (lb("attention.wq") + lb("attention.wk") + lb("attention.wv") + d * act),
+        "attn_decode": synthetic.kv_bytes_per_position(cfg) * T,
+        "linear": L * (lb("attention.wo") + lb("feed_forward.w2")) + head + d * act,
+        "ffn_gate": L * (lb("feed_forward.w1") + lb("feed_forward.w3") + d * act),
+    }
+
+
+def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=True):
+    from denograd_amd import ffi, synthetic
+    from denograd_amd.ffi import check
+    from denograd_amd.llama3 import Llama3
+
+    lib = ffi.load()
+    ctx = prompt_len + warmup + steps + profile_steps + 8
+    cfg = synthetic.config(name, max_context=ctx)
+    t0 = time.perf_counter()
+    llm = Llama3.from_config(cfg).random_init(seed=0, tied=cfg["tied"])
+    if not use_graph:
+        llm.model.forward_jit = None     # the same kernels, launched one by one instead of replayed as a graph
+    check(lib.jsgrad_hip_sync())
+    log(f"[{name}] weights on device in {time.perf_counter() - t0:.1f}s")
+    prompt = [int(t) for t in synthetic.random_prompt(cfg, prompt_len, seed=0)]
+    t0 = time.perf_counter()
+    llm._prefill(prompt[:-1])
+    llm._call(prompt[-1])
+    llm.start_pos += 1
+    log(f"[{name}] token-serial prefill of {prompt_len} tokens in {time.perf_counter() - t0:.2f}s")
+
+    m = llm.model
+    m.generate(warmup)
+    llm.start_pos += warmup
+    check(lib.jsgrad_hip_sync())
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    check(lib.jsgrad_hip_event_create(C.byref(e0)))
+    check(lib.jsgrad_hip_event_create(C.byref(e1)))
+    t_first = llm.start_pos + 1
+    w0 = time.perf_counter()
+    check(lib.jsgrad_hip_event_record(e0))
+    m.generate(steps)
+    check(lib.jsgrad_hip_event_record(e1))
+    check(lib.jsgrad_hip_sync())
+    wall = time.perf_counter() - w0
+    llm.start_pos += steps
+    ms = C.c_float()
+    check(lib.jsgrad_hip_event_elapsed_ms(e0, e1, C.byref(ms)))
+    t_avg = t_first + (steps - 1) / 2.0          # mean number of visible positions over the timed steps
+    tok_s = steps / wall
+
+    # per-kernel durations: the same step, eager, one event pair per launch
+    check(lib.jsgrad_hip_profile(1))
+    for _ in range(profile_steps):
+        m._step()
+    kinds = {}
+    for kname, kid in ffi.PROF_KINDS.items():
+        n, tot = C.c_int(), C.c_double()
+        check(lib.jsgrad_hip_profile_read(kid, C.byref(n), C.byref(tot)))
+        if n.value:
+            kinds[kname] = {"launches_per_step": n.value // profile_steps, "ms_per_step": tot.value / profile_steps}
+    check(lib.jsgrad_hip_profile(0))
+    llm.start_pos += profile_steps
+    kb = kernel_bytes(cfg, llm.start_pos)
+    for kname, b in kb.items():
+        k = kinds[kname]
+        k["bytes_per_step"] = int(b)
+        k["avg_us_per_launch"] = 1e3 * k["ms_per_step"] / k["launches_per_step"]
+        k["GBps"] = b / (k["ms_per_step"] * 1e-3) / 1e9
+    dom = max(kb, key=lambda n: kinds[n]["ms_per_step"])
+    achieved = kinds[dom]["GBps"]
+    bytes_tok = synthetic.weight_bytes_per_token(cfg) + synthetic.kv_bytes_per_position(cfg) * t_avg
+    res = {
+        "name": name, "tok_s": tok_s, "ms_per_step": 1e3 * wall / steps, "event_ms_per_step": ms.value / steps,
+        "roofline": {"bound": "hbm", "kernel": f"gemv_kernel ({dom})", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "bytes_per_launch": int(kb[dom] / kinds[dom]["launches_per_step"]), "avg_us_per_launch": round(kinds[dom]["avg_us_per_launch"], 2)},
+        "step_roofline": {"bytes_per_token": int(bytes_tok), "achieved": round(bytes_tok * tok_s / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": round(bytes_tok * tok_s / 1e9 / HBM_PEAK_GBS, 4)},
+        "kernels": {k: {kk: (round(vv, 3) if isinstance(vv, float) else vv) for kk, vv in v.items()} for k, v in kinds.items()},
+        "config": {"workload": f"Llama-3 decode bs=1, {name}-shaped random init ({cfg['quantize']}), {prompt_len}-token prompt, {steps} greedy tokens",
+                   "prompt": prompt_len, "decode": steps, "avg_visible_positions": t_avg, "max_context": ctx},
+    }
+    return llm, cfg, res
+
+
+def cpu_baseline(llm, cfg, budget_s=15.0):
+    """Time the oracle on the host (1 thread) on the same weights and check its tokens against the GPU's."""
+    import oracle as orc
+    from denograd_amd import synthetic
+    from denograd_amd.state import get_state_dict
+
+    t0 = time.perf_counter()
+    sd = {k: v.numpy() for k, v in get_state_dict(llm.model).items()}
+    log(f"[cpu] weights copied to host in {time.perf_counter() - t0:.1f}s")
+    ocfg = dict(cfg, max_context=64)
+    cpu = orc.OracleModel(ocfg, sd)
+    prompt = [int(t) for t in synthetic.random_prompt(cfg, 4, seed=7)]
+    t0 = time.perf_counter()
+    cpu.forward([prompt[0]], 0, want_logits=False)
+    per = time.perf_counter() - t0
+    n_new = int(max(2, min(28, budget_s / per - len(prompt))))
+    cpu.reset()
+    t0 = time.perf_counter()
+    toks_c = list(cpu.generate(prompt, n_new))
+    dt = time.perf_counter() - t0
+    n_fwd = len(prompt) + n_new - 1
+    # the GPU on the same prompt from position 0 (stale cache rows past the current position are never read)
+    llm.start_pos, llm.last_seen_toks = 0, []
+    toks_g = llm.chat_tokens(prompt, n_new)["tokens"]
+    same = sum(int(a == b) for a, b in zip(toks_g, toks_c))
+    return {"value": round(n_fwd / dt, 4), "unit": "tok/s", "cores": 1, "kind": "port",
+            "sample": f"{n_fwd} single-token forwards ({len(prompt)}-token prompt + {n_new} greedy tokens from position 0) of the same {cfg['name']} weights, "
+                      f"C oracle (gcc -O2, fp16 storage, float accumulate), 1 thread of {os.cpu_count()} host cpus",
+            "tokens_identical_to_gpu": f"{same}/{n_new}"}
+
+
+def traffic_probe(name):
+    from denograd_amd import ffi, synthetic
+    from denograd_amd.ffi import check
+    from denograd_amd.llama3 import Llama3
+    from denograd_amd.tensor import Tensor
+    lib = ffi.load()
+    n = 512 << 20
+    src, dst = Tensor.zeros((n,), "uint8"), Tensor.empty((n,), "uint8")
+    check(lib.jsgrad_hip_sync())
+    check(lib.jsgrad_hip_copy(dst.ptr, src.ptr, n))      # reads 512 MiB, writes 512 MiB
+    check(lib.jsgrad_hip_sync())
+    cfg = synthetic.config(name, max_context=64)
+    llm = Llama3.from_config(cfg).random_init(seed=0, tied=cfg["tied"])
+    llm.model.forward_jit = None
+    for t in (1, 2, 3, 4):
+        llm._call(t)
+        llm.start_pos += 1
+    check(lib.jsgrad_hip_sync())
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--prompt", type=int, default=512)
+    ap.add_argument("--workload", default="1B", help="primary synthetic config (denograd_amd/synthetic.py)")
+    ap.add_argument("--secondary", default="8B-int8", help="second workload measured in the same run ('' to skip)")
+    ap.add_argument("--secondary-steps", type=int, default=128)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle baseline")
+    ap.add_argument("--traffic-probe", action="store_true", help="for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: one 512 MiB device-to-device copy "
+                    "(a plain copy kernel of known size, to scale the counters) followed by 4 eager decode steps of --workload; prints nothing")
+    ap.add_argument("--no-graph", action="store_true", help="launch every kernel eagerly instead of replaying a captured HIP graph "
+                    "(rocprofv3 --kernel-trace on this image crashes inside hipGraphLaunch, so profiles are taken this way)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py: this build runs on ONE GPU (no collectives, no sharding); --gpus must be 1")
+        sys.exit(2)
+
+    from denograd_amd import ffi
+    from denograd_amd.device import Device
+    dev = Device.get("HIP").init()
+    log(f"device: {dev.name}, {dev.cu_count} CUs")
+
+    if args.traffic_probe:
+        traffic_probe(args.workload)
+        return
+    llm, cfg, res = run_workload(args.workload, args.prompt, args.steps, args.warmup, use_graph=not args.no_graph)
+    cpu = None if args.no_cpu else cpu_baseline(llm, cfg)
+    del llm
+    secondary = None
+    if args.secondary:
+        llm2, cfg2, secondary = run_workload(args.secondary, args.prompt, args.secondary_steps, args.warmup, use_graph=not args.no_graph)
+        del llm2
+
+    out = {
+        "metric": "decode tok/s bs=1 + % HBM roofline, Llama-3.2-1B fp16 & 8B int8",
+        "value": round(res["tok_s"], 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(res["ms_per_step"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic", "config": res["config"],
+        "roofline": res["roofline"], "cpu_baseline": cpu,
+        "step_roofline": res["step_roofline"], "kernels": res["kernels"], "event_ms_per_step": round(res["event_ms_per_step"], 4),
+        "launch_mode": "eager" if args.no_graph else "hip_graph",
+    }
+    if secondary:
+        out["secondary"] = {"value": round(secondary["tok_s"], 2), "unit": "tok/s", "steps": args.secondary_steps, "ms_per_step": round(secondary["ms_per_step"], 4),
+                            "dtype": "i8 weights, f16 activations", "config": secondary["config"], "roofline": secondary["roofline"],
+                            "step_roofline": secondary["step_roofline"], "kernels": secondary["kernels"]}
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -207,24 +207,36 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_decode_kernel(AttnArgs a) {
   __syncthreads();
   if (!is_last) return;
   __threadfence();
+  // merge: one wavefront per query head turns the per-chunk (m, l) into weights exp(m_s - M) and 1/L ...
   const float *base = a.partial + (size_t)g * a.nsplit * NREP * (HD + 2);
+  for (int j = wave; j < NREP; j += NW) {
+    float M = -INFINITY;
+    for (int s = lane; s < n_active; s += 64) M = fmaxf(M, __builtin_nontemporal_load(base + ((size_t)s * NREP + j) * (HD + 2) + HD));
+    M = wave_max(M);
+    float L = 0.0f;
+    for (int s = lane; s < n_active; s += 64) {
+      const float *ps = base + ((size_t)s * NREP + j) * (HD + 2);
+      const float w = exp_f32(__builtin_nontemporal_load(ps + HD) - M);
+      sc[j][s] = w;  // n_active <= nsplit <= ATT_CHUNK_MAX
+      L = fmaf(__builtin_nontemporal_load(ps + HD + 1), w, L);
+    }
+    L = wave_sum(L);
+    if (lane == 0) l_sh[j] = 1.0f / L;  // softmax normalisation is e * (1/sum) (tensor.ts:2211-2214)
+  }
+  __syncthreads();
+  // ... then every thread sums its output elements over the chunks; the loads are independent, so they pipeline
   for (int i = tid; i < NREP * HD; i += ATT_THREADS) {
     const int j = i / HD, d = i % HD;
-    float M = -INFINITY;
-    for (int s = 0; s < n_active; s++) M = fmaxf(M, __builtin_nontemporal_load(base + ((size_t)s * NREP + j) * (HD + 2) + HD));
-    float L = 0.0f, O = 0.0f;
-    for (int s = 0; s < n_active; s++) {
-      const float *ps = base + ((size_t)s * NREP + j) * (HD + 2);
-      const float w = exp_f32(__fsub_rn(__builtin_nontemporal_load(ps + HD), M));
-      L = fmaf(__builtin_nontemporal_load(ps + HD + 1), w, L);
-      O = fmaf(__builtin_nontemporal_load(ps + d), w, O);
-    }
-    // softmax normalisation e * (1/sum) (tensor.ts:2211-2214), then the cast of the P.V result
-    ((AT *)a.out)[(size_t)(g * NREP + j) * HD + d] = (AT)Act<AT>::rn(__fmul_rn(O, __fdiv_rn(1.0f, L)));
+    const float *po = base + (size_t)j * (HD + 2) + d;
+    float O = 0.0f;
+#pragma unroll 8
+    for (int s = 0; s < n_active; s++) O = fmaf(__builtin_nontemporal_load(po + (size_t)s * NREP * (HD + 2)), sc[j][s], O);
+    ((AT *)a.out)[(size_t)(g * NREP + j) * HD + d] = (AT)Act<AT>::rn(O * l_sh[j]);  // the cast of the P.V result
   }
   if (tid == 0) __hip_atomic_store(&a.counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// splits: enough that a chunk fits the LDS score buffer, and no more than the merge can index there
 static int nsplit_for(int max_context) {
   int by_lds = (max_context + ATT_CHUNK_MAX - 1) / ATT_CHUNK_MAX;
   int wanted = (max_context + 31) / 32;
@@ -274,6 +286,7 @@ int jsgrad_hip_attn_decode(const void *q, const void *cache_k, const void *cache
   a.n_kv_heads = n_kv_heads; a.nsplit = nsplit_for(max_context); a.max_context = max_context;
   a.scale = (float)(1.0 / sqrt((double)head_dim));
   const int n_rep = n_heads / n_kv_heads;
+  ProfScope prof(PROF_ATTN);
   if (act == JSGRAD_F16) return head_dim == 64 ? launch_attn<_Float16, 64>(a, n_rep) : launch_attn<_Float16, 128>(a, n_rep);
   return head_dim == 64 ? launch_attn<float, 64>(a, n_rep) : launch_attn<float, 128>(a, n_rep);
 }

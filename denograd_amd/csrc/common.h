@@ -21,6 +21,14 @@ State &state();
 int fail(const char *fmt, ...);
 int fail_hip(hipError_t e, const char *what);
 
+// per-kernel timing with HIP events on the library stream (off unless jsgrad_hip_profile(1))
+enum { PROF_EMBED = 0, PROF_RMSNORM, PROF_LINEAR, PROF_QKV_ROPE, PROF_ATTN, PROF_FFN_GATE, PROF_ARGMAX, PROF_KINDS };
+struct ProfScope {
+  int slot;
+  explicit ProfScope(int kind);
+  ~ProfScope();
+};
+
 #define JSG_HIP(call)                                   \
   do {                                                  \
     hipError_t e_ = (call);                             \

@@ -46,33 +46,57 @@ template <typename AT> __global__ __launch_bounds__(1024) void rmsnorm_kernel(co
   }
 }
 
-// ---------------------------------------------------------------- greedy argmax (one block)
-// Tensor.argmax (tensor.ts:2314-2320): the lowest index among the maxima.
-template <typename AT> __global__ __launch_bounds__(1024) void argmax_kernel(const AT *x, int n, int32_t *st, int32_t *tokens_out, int advance) {
-  __shared__ float vmax[16];
-  __shared__ int imax[16];
+// ---------------------------------------------------------------- greedy argmax
+// Tensor.argmax (tensor.ts:2314-2320): the lowest index among the maxima.  ARGMAX_BLOCKS blocks each reduce a
+// slice; the last one to finish (agent-scope counter) reduces the per-block winners and updates the state words.
+constexpr int ARGMAX_BLOCKS = 128, ARGMAX_THREADS = 256;
+__device__ float g_argmax_val[ARGMAX_BLOCKS];
+__device__ int g_argmax_idx[ARGMAX_BLOCKS];
+__device__ int g_argmax_count;  // zero between launches: the finishing block resets it
+
+__device__ __forceinline__ void argmax_merge(float &best, int &bi, float ov, int oi) {
+  if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+}
+template <typename AT> __global__ __launch_bounds__(ARGMAX_THREADS) void argmax_kernel(const AT *x, int n, int32_t *st, int32_t *tokens_out, int tokens_cap, int advance) {
+  __shared__ float vmax[ARGMAX_THREADS / 64];
+  __shared__ int imax[ARGMAX_THREADS / 64];
+  __shared__ int is_last;
+  const int tid = threadIdx.x;
   float best = -INFINITY;
   int bi = 0x7fffffff;
-  for (int i = threadIdx.x; i < n; i += blockDim.x) {
-    float v = (float)x[i];
-    if (v > best || (v == best && i < bi)) { best = v; bi = i; }
+  for (int i = blockIdx.x * ARGMAX_THREADS + tid; i < n; i += gridDim.x * ARGMAX_THREADS) argmax_merge(best, bi, (float)x[i], i);
+  auto block_reduce = [&]() {
+    for (int off = 32; off > 0; off >>= 1) argmax_merge(best, bi, __shfl_xor(best, off), __shfl_xor(bi, off));
+    if ((tid & 63) == 0) { vmax[tid >> 6] = best; imax[tid >> 6] = bi; }
+    __syncthreads();
+    if (tid == 0)
+      for (int w = 1; w < ARGMAX_THREADS / 64; w++) argmax_merge(best, bi, vmax[w], imax[w]);
+  };
+  block_reduce();
+  if (tid == 0) {
+    g_argmax_val[blockIdx.x] = best;
+    g_argmax_idx[blockIdx.x] = bi;
+    __threadfence();
+    is_last = __hip_atomic_fetch_add(&g_argmax_count, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == (int)gridDim.x - 1;
   }
-  // wavefront reduction keeping the lower index on ties
-  for (int off = 32; off > 0; off >>= 1) {
-    float ov = __shfl_xor(best, off);
-    int oi = __shfl_xor(bi, off);
-    if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
-  }
-  if ((threadIdx.x & 63) == 0) { vmax[threadIdx.x >> 6] = best; imax[threadIdx.x >> 6] = bi; }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    for (int w = 1; w < (int)(blockDim.x >> 6); w++)
-      if (vmax[w] > best || (vmax[w] == best && imax[w] < bi)) { best = vmax[w]; bi = imax[w]; }
+  if (!is_last) return;
+  __threadfence();
+  best = -INFINITY;
+  bi = 0x7fffffff;
+  if (tid < (int)gridDim.x) {
+    best = __builtin_nontemporal_load(&g_argmax_val[tid]);
+    bi = __builtin_nontemporal_load(&g_argmax_idx[tid]);
+  }
+  __syncthreads();  // vmax / imax are reused
+  block_reduce();
+  if (tid == 0) {
     if (bi == 0x7fffffff) bi = n;  // all-NaN input: the reference's formula yields n
     const int pos = st[1];
-    if (tokens_out && pos >= 0) tokens_out[pos] = bi;
+    if (tokens_out && pos >= 0 && pos < tokens_cap) tokens_out[pos] = bi;
     st[0] = bi;
     if (advance) st[1] = pos + 1;
+    __hip_atomic_store(&g_argmax_count, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
 
@@ -282,6 +306,7 @@ int jsgrad_hip_embed(int kind, const void *table, const void *scale, const int32
   JSG_REQUIRE(kind == JSGRAD_W_F32 || kind == JSGRAD_W_F16 || kind == JSGRAD_W_I8, "jsgrad_hip_embed: table kind %d", kind);
   JSG_REQUIRE(kind != JSGRAD_W_I8 || scale, "jsgrad_hip_embed: int8 table needs row scales");
   dim3 grid((dim + 255) / 256), block(256);
+  ProfScope prof(PROF_EMBED);
   if (act == JSGRAD_F16) hipLaunchKernelGGL(embed_kernel<_Float16>, grid, block, 0, state().stream, kind, table, (const _Float16 *)scale, st, (_Float16 *)out, dim, vocab);
   else if (act == JSGRAD_F32) hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, state().stream, kind, table, (const _Float16 *)scale, st, (float *)out, dim, vocab);
   else return fail("jsgrad_hip_embed: unknown activation dtype %d", act);
@@ -293,6 +318,7 @@ int jsgrad_hip_rmsnorm(const void *x, const void *weight, void *y, int dim, floa
   JSG_READY();
   JSG_REQUIRE(x && weight && y && dim > 0, "jsgrad_hip_rmsnorm: bad argument");
   const float inv_d = (float)(1.0 / (double)dim);
+  ProfScope prof(PROF_RMSNORM);
   if (act == JSGRAD_F16) hipLaunchKernelGGL(rmsnorm_kernel<_Float16>, dim3(1), dim3(1024), 0, state().stream, (const _Float16 *)x, (const _Float16 *)weight, (_Float16 *)y, dim, eps, inv_d);
   else if (act == JSGRAD_F32) hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(1), dim3(1024), 0, state().stream, (const float *)x, (const float *)weight, (float *)y, dim, eps, inv_d);
   else return fail("jsgrad_hip_rmsnorm: unknown activation dtype %d", act);
@@ -300,11 +326,13 @@ int jsgrad_hip_rmsnorm(const void *x, const void *weight, void *y, int dim, floa
   return 0;
 }
 
-int jsgrad_hip_argmax(const void *logits, int n, int32_t *st, int32_t *tokens_out, int advance, int act) {
+int jsgrad_hip_argmax(const void *logits, int n, int32_t *st, int32_t *tokens_out, int tokens_cap, int advance, int act) {
   JSG_READY();
   JSG_REQUIRE(logits && st && n > 0, "jsgrad_hip_argmax: bad argument");
-  if (act == JSGRAD_F16) hipLaunchKernelGGL(argmax_kernel<_Float16>, dim3(1), dim3(1024), 0, state().stream, (const _Float16 *)logits, n, st, tokens_out, advance);
-  else if (act == JSGRAD_F32) hipLaunchKernelGGL(argmax_kernel<float>, dim3(1), dim3(1024), 0, state().stream, (const float *)logits, n, st, tokens_out, advance);
+  const int nb = n >= ARGMAX_BLOCKS * ARGMAX_THREADS ? ARGMAX_BLOCKS : (n + ARGMAX_THREADS - 1) / ARGMAX_THREADS;
+  ProfScope prof(PROF_ARGMAX);
+  if (act == JSGRAD_F16) hipLaunchKernelGGL(argmax_kernel<_Float16>, dim3(nb), dim3(ARGMAX_THREADS), 0, state().stream, (const _Float16 *)logits, n, st, tokens_out, tokens_cap, advance);
+  else if (act == JSGRAD_F32) hipLaunchKernelGGL(argmax_kernel<float>, dim3(nb), dim3(ARGMAX_THREADS), 0, state().stream, (const float *)logits, n, st, tokens_out, tokens_cap, advance);
   else return fail("jsgrad_hip_argmax: unknown activation dtype %d", act);
   JSG_LAUNCHED();
   return 0;

@@ -153,21 +153,45 @@ template <int KIND> __device__ __forceinline__ u4_t load_w(const void *w, size_t
   return __builtin_nontemporal_load((const u4_t *)p);
 }
 
-// stage x (optionally RMSNorm'ed) into LDS in the activation dtype
+// Stage x (optionally RMSNorm'ed) into LDS in the activation dtype.  Every thread moves 16-byte chunks; with a
+// norm the chunks stay in registers between the sum of squares and the scaling, so x is read from memory once and
+// the whole prologue costs one round of global loads and two barriers.
 template <typename AT> __device__ __forceinline__ void stage_x(const GemvArgs &a, AT *xs, float *red) {
-  const AT *x = (const AT *)a.x;
+  constexpr int EPC = 16 / sizeof(AT);  // elements per 16-byte chunk
+  constexpr int MAXCH = 4;              // chunks a thread keeps in registers on the norm path
   const int n = a.in_f, tid = threadIdx.x, nt = blockDim.x;
+  const int nchunks = n / EPC;          // in_f is a multiple of EPC (checked on the host)
+  const u4_t *xg = (const u4_t *)a.x;
+  u4_t *xl = (u4_t *)xs;
   if (a.norm_w == nullptr) {
-    for (int i = tid; i < n; i += nt) xs[i] = x[i];
+    for (int c = tid; c < nchunks; c += nt) xl[c] = xg[c];
     __syncthreads();
     return;
   }
+  const u4_t *wg = (const u4_t *)a.norm_w;
+  u4_t xr[MAXCH], wr[MAXCH];
   float ss = 0.0f;
-  for (int i = tid; i < n; i += nt) {
-    AT v = x[i];
-    xs[i] = v;
-    float f = (float)v;
-    ss = fmaf(f, f, ss);
+#pragma unroll
+  for (int i = 0; i < MAXCH; i++) {
+    const int c = tid + i * nt;
+    if (c < nchunks) { xr[i] = xg[c]; wr[i] = wg[c]; }
+  }
+#pragma unroll
+  for (int i = 0; i < MAXCH; i++) {
+    const int c = tid + i * nt;
+    if (c < nchunks) {
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        if constexpr (sizeof(AT) == 2) {
+          h2_t h = as_h2(xr[i][e]);
+          ss = fmaf((float)h[0], (float)h[0], ss);
+          ss = fmaf((float)h[1], (float)h[1], ss);
+        } else {
+          float f = __uint_as_float(xr[i][e]);
+          ss = fmaf(f, f, ss);
+        }
+      }
+    }
   }
   ss = wave_sum(ss);
   const int wave = tid >> 6, nw = nt >> 6;
@@ -177,142 +201,216 @@ template <typename AT> __device__ __forceinline__ void stage_x(const GemvArgs &a
   for (int i = 0; i < nw; i++) tot += red[i];
   // sqrt(1 / (mean + eps)), mean = sum * float(1/d)  (nn/index.ts:586, tensor.ts:2944-2946)
   const float r = __fsqrt_rn(__fdiv_rn(1.0f, __fadd_rn(__fmul_rn(tot, a.inv_d), a.eps)));
-  const AT *nw_ = (const AT *)a.norm_w;
-  for (int i = tid; i < n; i += nt) {
-    float v = Act<AT>::rn(__fmul_rn((float)xs[i], r));       // .cast(x.dtype) before the weight multiply
-    xs[i] = (AT)Act<AT>::rn(__fmul_rn(v, (float)nw_[i]));
+#pragma unroll
+  for (int i = 0; i < MAXCH; i++) {
+    const int c = tid + i * nt;
+    if (c < nchunks) {
+      u4_t o;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        if constexpr (sizeof(AT) == 2) {
+          h2_t h = as_h2(xr[i][e]), w = as_h2(wr[i][e]), y;
+          // .cast(x.dtype) before the weight multiply (nn/index.ts:588)
+          y[0] = (_Float16)((float)(_Float16)((float)h[0] * r) * (float)w[0]);
+          y[1] = (_Float16)((float)(_Float16)((float)h[1] * r) * (float)w[1]);
+          o[e] = __builtin_bit_cast(uint32_t, y);
+        } else {
+          o[e] = __float_as_uint((__uint_as_float(xr[i][e]) * r) * __uint_as_float(wr[i][e]));
+        }
+      }
+      xl[c] = o;
+    }
   }
   __syncthreads();
 }
 
-template <int KIND, typename AT, int EPI, int ROWS>
+// A block stages x once and then its wavefronts walk row groups (ROWS consecutive output rows of the NM matrices
+// that share x) grid-stride.  A wavefront's work is the flat sequence of (row group, k-batch) items; the weight
+// loads of item i+1 are issued into a second register buffer before item i is consumed, and the first item is
+// requested before x is staged, so a wavefront always has a batch of 128-bit loads in flight.
+template <int KIND, typename AT, int EPI, int ROWS, int UNROLL>
 __global__ __launch_bounds__(256) void gemv_kernel(GemvArgs a) {
   constexpr int VEC = WFmt<KIND>::VEC;
+  constexpr int BITS = KIND == JSGRAD_W_F32 ? 32 : KIND == JSGRAD_W_F16 ? 16 : KIND == JSGRAD_W_I8 ? 8 : 4;
+  constexpr int STEP = 64 * VEC;                 // elements one wavefront covers per k-step
   constexpr int NM = EPI == EPI_SWIGLU ? 2 : 1;  // matrices a wavefront evaluates on the same rows
+  static_assert(ROWS % 2 == 0 || EPI != EPI_ROPE_KV, "rotary pairs need an even row group");
   extern __shared__ __align__(16) unsigned char smem[];
   AT *xs = (AT *)smem;
   __shared__ float red[8];
   __shared__ float lut[16];
   if (KIND == JSGRAD_W_NF4 && threadIdx.x < 16) lut[threadIdx.x] = NF4_CODE[threadIdx.x];
-  stage_x<AT>(a, xs, red);  // ends with a barrier, which also publishes lut
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const int in_f = a.in_f;
   const int total = EPI == EPI_SWIGLU ? a.rows[0] : a.rows[0] + a.rows[1] + a.rows[2];
-  const int g0 = (blockIdx.x * nw + wave) * ROWS;  // first row of this wavefront in the combined row space
-  if (g0 >= total) return;
+  const int ngroups = (total + ROWS - 1) / ROWS;
+  const int gstride = gridDim.x * nw;
+  const int nsteps = (in_f + STEP - 1) / STEP;
+  const int nbatch = (nsteps + UNROLL - 1) / UNROLL;
+  typedef u4_t Buf[UNROLL][NM][ROWS];
+  // read the position now, not in the epilogue: the load then overlaps the weight stream instead of ending the kernel
+  const int pos = EPI == EPI_ROPE_KV ? a.st[1] : 0;
 
-  // which matrix the group lies in (EPI_ROPE_KV stacks wq, wk, wv; group boundaries are multiples of ROWS)
-  int m = 0, r0 = g0;
-  if (EPI == EPI_ROPE_KV) {
-    if (r0 >= a.rows[0]) { r0 -= a.rows[0]; m = 1; }
-    if (m == 1 && r0 >= a.rows[1]) { r0 -= a.rows[1]; m = 2; }
-  }
-  const int mrows = a.rows[m];
-  const void *wp[NM];
-  const void *sp[NM];
-  wp[0] = a.w[m]; sp[0] = a.s[m];
-  if (NM == 2) { wp[1] = a.w[1]; sp[1] = a.s[1]; }
+  // rows of a group: matrix m (EPI_ROPE_KV stacks wq, wk, wv; boundaries are multiples of ROWS), first row r0
+  struct Where { int m, r0, mrows; };
+  auto locate = [&](int grp) {
+    Where w = {0, grp * ROWS, 0};
+    if (EPI == EPI_ROPE_KV) {
+      if (w.r0 >= a.rows[0]) { w.r0 -= a.rows[0]; w.m = 1; }
+      if (w.m == 1 && w.r0 >= a.rows[1]) { w.r0 -= a.rows[1]; w.m = 2; }
+    }
+    // selects, not a.rows[m]: indexing the argument struct with a run-time m would copy it to scratch memory
+    w.mrows = w.m == 0 ? a.rows[0] : (w.m == 1 ? a.rows[1] : a.rows[2]);
+    return w;
+  };
+  auto wbase = [&](int m, int j) -> const void * { return NM == 2 ? (j == 0 ? a.w[0] : a.w[1]) : (m == 0 ? a.w[0] : (m == 1 ? a.w[1] : a.w[2])); };
+  auto sbase = [&](int m, int j) -> const void * { return NM == 2 ? (j == 0 ? a.s[0] : a.s[1]) : (m == 0 ? a.s[0] : (m == 1 ? a.s[1] : a.s[2])); };
+
+  auto load_item = [&](Buf &buf, int grp, int b) {
+    const Where w = locate(grp);
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+      const int k = (b * UNROLL + u) * STEP + lane * VEC;
+      if (k < in_f) {
+#pragma unroll
+        for (int j = 0; j < NM; j++)
+#pragma unroll
+          for (int r = 0; r < ROWS; r++) {
+            const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;  // tail rows reload the last row, never stored
+            const char *p = (const char *)wbase(w.m, j) + (((size_t)row * in_f + (size_t)k) * BITS) / 8;
+            buf[u][j][r] = __builtin_nontemporal_load((const u4_t *)p);
+          }
+      }
+    }
+  };
 
   float acc[NM][ROWS];
+  auto use_item = [&](const Buf &buf, int grp, int b) {
+    const Where w = locate(grp);
+    if (b == 0) {
 #pragma unroll
-  for (int j = 0; j < NM; j++)
+      for (int j = 0; j < NM; j++)
 #pragma unroll
-    for (int r = 0; r < ROWS; r++) acc[j][r] = 0.0f;
-
-  const int in_f = a.in_f;
-  for (int k = lane * VEC; k < in_f; k += 64 * VEC) {
-    u4_t wv[NM][ROWS];
-#pragma unroll
-    for (int j = 0; j < NM; j++)
-#pragma unroll
-      for (int r = 0; r < ROWS; r++) {
-        int row = r0 + r < mrows ? r0 + r : mrows - 1;  // clamp: tail rows reload the last row, never stored
-        wv[j][r] = load_w<KIND>(wp[j], (size_t)row, in_f, k);
-      }
-    XFrag<AT, VEC> xf;
-    xf.load(xs + k);
-#pragma unroll
-    for (int j = 0; j < NM; j++)
-#pragma unroll
-      for (int r = 0; r < ROWS; r++) {
-        float bs = 1.0f;
-        if constexpr (KIND == JSGRAD_W_NF4) {
-          int row = r0 + r < mrows ? r0 + r : mrows - 1;
-          bs = (float)((const _Float16 *)sp[j])[((size_t)row * in_f + k) >> 6];
-        }
-        acc[j][r] = Dot<KIND, AT>::run(wv[j][r], xf, acc[j][r], bs, lut);
-      }
-  }
-#pragma unroll
-  for (int j = 0; j < NM; j++)
-#pragma unroll
-    for (int r = 0; r < ROWS; r++) acc[j][r] = wave_sum(acc[j][r]);
-
-  // per-row results in the activation dtype: RN_act(sum [* scale])
-  float val[NM][ROWS];
-#pragma unroll
-  for (int j = 0; j < NM; j++)
-#pragma unroll
-    for (int r = 0; r < ROWS; r++) {
-      float v = acc[j][r];
-      if constexpr (KIND == JSGRAD_W_I8) {
-        int row = r0 + r < mrows ? r0 + r : mrows - 1;
-        v = __fmul_rn(v, (float)((const _Float16 *)sp[j])[row]);
-      }
-      val[j][r] = Act<AT>::rn(v);
+        for (int r = 0; r < ROWS; r++) acc[j][r] = 0.0f;
     }
-
-  if constexpr (EPI == EPI_STORE) {
-    AT *y = (AT *)a.y;
-    const AT *res = (const AT *)a.residual;
 #pragma unroll
-    for (int r = 0; r < ROWS; r++)
-      if (lane == r && r0 + r < mrows) {
-        float v = val[0][r];
-        if (res) v = Act<AT>::rn(__fadd_rn((float)res[r0 + r], v));
-        y[r0 + r] = (AT)v;
+    for (int u = 0; u < UNROLL; u++) {
+      const int k = (b * UNROLL + u) * STEP + lane * VEC;
+      if (k < in_f) {
+        XFrag<AT, VEC> xf;
+        xf.load(xs + k);
+#pragma unroll
+        for (int j = 0; j < NM; j++)
+#pragma unroll
+          for (int r = 0; r < ROWS; r++) {
+            float bs = 1.0f;
+            if constexpr (KIND == JSGRAD_W_NF4) {
+              const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;
+              bs = (float)((const _Float16 *)sbase(w.m, j))[((size_t)row * in_f + k) >> 6];
+            }
+            acc[j][r] = Dot<KIND, AT>::run(buf[u][j][r], xf, acc[j][r], bs, lut);
+          }
       }
-  } else if constexpr (EPI == EPI_SWIGLU) {
-    AT *g = (AT *)a.y;
+    }
+    if (b != nbatch - 1) return;
+
+    // ---- the group is complete: cross-lane sum, scale, cast, epilogue
+    float val[NM][ROWS];
 #pragma unroll
-    for (int r = 0; r < ROWS; r++)
-      if (lane == r && r0 + r < mrows) g[r0 + r] = (AT)Act<AT>::rn(__fmul_rn(silu_act<AT>(val[0][r]), val[1][r]));
-  } else {
-    static_assert(ROWS % 2 == 0 || EPI != EPI_ROPE_KV, "rotary pairs need an even row group");
-    const int pos = a.st[1];
-    if (pos < 0 || pos >= a.max_context) return;  // never write outside the cache
-    const int hd = a.head_dim;
-    if (m == 2) {  // value rows: plain copy into the cache row
-      AT *cv = (AT *)a.cache_v + (size_t)pos * a.rows[2];
+    for (int j = 0; j < NM; j++)
+#pragma unroll
+      for (int r = 0; r < ROWS; r++) {
+        float v = wave_sum(acc[j][r]);
+        if constexpr (KIND == JSGRAD_W_I8) {
+          const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;
+          v = v * (float)((const _Float16 *)sbase(w.m, j))[row];
+        }
+        val[j][r] = Act<AT>::rn(v);
+      }
+    const int r0 = w.r0, mrows = w.mrows;
+    if constexpr (EPI == EPI_STORE) {
+      AT *y = (AT *)a.y;
+      const AT *res = (const AT *)a.residual;
 #pragma unroll
       for (int r = 0; r < ROWS; r++)
-        if (lane == r && r0 + r < mrows) cv[r0 + r] = (AT)val[0][r];
-    } else {       // query / key rows: rotate interleaved pairs (llama.ts:17-32)
-      const AT *tab = (const AT *)a.rope_table + (size_t)pos * hd;
-      AT *dst = m == 0 ? (AT *)a.y : (AT *)a.cache_k + (size_t)pos * a.rows[1];
-#pragma unroll
-      for (int r = 0; r < ROWS; r += 2)
-        if (lane == r && r0 + r + 1 < mrows) {
-          const int i = ((r0 + r) % hd) >> 1;
-          const float c = (float)tab[2 * i], d = (float)tab[2 * i + 1];
-          const float av = val[0][r], bv = val[0][r + 1];
-          dst[r0 + r] = (AT)Act<AT>::rn(__fsub_rn(__fmul_rn(av, c), __fmul_rn(bv, d)));
-          dst[r0 + r + 1] = (AT)Act<AT>::rn(__fadd_rn(__fmul_rn(av, d), __fmul_rn(bv, c)));
+        if (lane == r && r0 + r < mrows) {
+          float v = val[0][r];
+          if (res) v = Act<AT>::rn((float)res[r0 + r] + v);
+          y[r0 + r] = (AT)v;
         }
+    } else if constexpr (EPI == EPI_SWIGLU) {
+      AT *g = (AT *)a.y;
+#pragma unroll
+      for (int r = 0; r < ROWS; r++)
+        if (lane == r && r0 + r < mrows) g[r0 + r] = (AT)Act<AT>::rn(silu_act<AT>(val[0][r]) * val[1][r]);
+    } else {
+      if (pos < 0 || pos >= a.max_context) return;  // never write outside the cache
+      const int hd = a.head_dim;
+      if (w.m == 2) {  // value rows: plain copy into the cache row
+        AT *cv = (AT *)a.cache_v + (size_t)pos * a.rows[2];
+#pragma unroll
+        for (int r = 0; r < ROWS; r++)
+          if (lane == r && r0 + r < mrows) cv[r0 + r] = (AT)val[0][r];
+      } else {         // query / key rows: rotate interleaved pairs (llama.ts:17-32)
+        const AT *tab = (const AT *)a.rope_table + (size_t)pos * hd;
+        AT *dst = w.m == 0 ? (AT *)a.y : (AT *)a.cache_k + (size_t)pos * a.rows[1];
+#pragma unroll
+        for (int r = 0; r < ROWS; r += 2)
+          if (lane == r && r0 + r + 1 < mrows) {
+            const int i = ((r0 + r) % hd) >> 1;
+            const float c = (float)tab[2 * i], d = (float)tab[2 * i + 1];
+            const float av = val[0][r], bv = val[0][r + 1];
+            dst[r0 + r] = (AT)Act<AT>::rn(av * c - bv * d);  // the build keeps a*b+c unfused: two roundings as in plain C
+            dst[r0 + r + 1] = (AT)Act<AT>::rn(av * d + bv * c);
+          }
+      }
     }
+  };
+
+  // flat item sequence of this wavefront: (grp, b) -> next
+  int grp = blockIdx.x * nw + wave, b = 0;
+  auto advance = [&](int &g, int &bb) {
+    if (++bb == nbatch) { bb = 0; g += gstride; }
+  };
+  Buf bufA, bufB;
+  if (grp < ngroups) load_item(bufA, grp, 0);
+
+  stage_x<AT>(a, xs, red);  // block-wide, ends with a barrier (which also publishes lut)
+
+  while (grp < ngroups) {
+    int g1 = grp, b1 = b;
+    advance(g1, b1);
+    if (g1 < ngroups) load_item(bufB, g1, b1);
+    use_item(bufA, grp, b);
+    if (g1 >= ngroups) break;
+    grp = g1; b = b1;
+    advance(g1, b1);
+    if (g1 < ngroups) load_item(bufA, g1, b1);
+    use_item(bufB, grp, b);
+    grp = g1; b = b1;
   }
 }
 
 // ---- host-side dispatch ------------------------------------------------------------------------
 
-template <int KIND, typename AT, int EPI> static int launch_rows(const GemvArgs &a, int total_rows) {
-  constexpr int ROWS = 4, NW = 4;
-  const int rows_per_block = ROWS * NW;
-  dim3 grid((total_rows + rows_per_block - 1) / rows_per_block), block(NW * 64);
+template <int KIND, typename AT, int EPI, int ROWS, int UNROLL> static int launch_cfg(const GemvArgs &a, int total_rows) {
+  constexpr int NW = 4;
+  const int ngroups = (total_rows + ROWS - 1) / ROWS;
+  const int need = (ngroups + NW - 1) / NW;      // one group per wavefront
+  const int cap = state().cu_count * 4;          // 16 resident wavefronts per CU; more rows than that are walked grid-stride
+  dim3 grid(need < cap ? need : cap), block(NW * 64);
   size_t lds = (size_t)a.in_f * sizeof(AT);
-  hipLaunchKernelGGL((gemv_kernel<KIND, AT, EPI, ROWS>), grid, block, lds, state().stream, a);
+  hipLaunchKernelGGL((gemv_kernel<KIND, AT, EPI, ROWS, UNROLL>), grid, block, lds, state().stream, a);
   JSG_LAUNCHED();
   return 0;
+}
+// Two register buffers of UNROLL x NM x ROWS 16-byte loads each: (2 rows, 4 steps) for one matrix, (2 rows, 2 steps)
+// for the SwiGLU pair, i.e. 8 loads = 8 KiB per wavefront per buffer either way.
+template <int KIND, typename AT, int EPI> static int launch_rows(const GemvArgs &a, int total_rows) {
+  if constexpr (EPI == EPI_SWIGLU) return launch_cfg<KIND, AT, EPI, 2, 2>(a, total_rows);
+  else
+  return launch_cfg<KIND, AT, EPI, 2, 4>(a, total_rows);
 }
 template <int EPI> static int dispatch(int kind, int act, const GemvArgs &a, int total_rows) {
 #define JSG_CASE(K)                                                          \
@@ -337,6 +435,12 @@ static int check_common(const char *who, int kind, int act, int in_f, const void
   JSG_REQUIRE((size_t)in_f * (act == JSGRAD_F16 ? 2 : 4) <= 64 * 1024, "%s: in_features %d does not fit the 64 KiB LDS staging buffer", who, in_f);
   return 0;
 }
+// the fused RMSNorm keeps 4 x 16 bytes of x per thread in registers (256 threads)
+static int check_norm(const char *who, const void *norm_weight, int act, int in_f) {
+  const int cap = 4 * 256 * (act == JSGRAD_F16 ? 8 : 4);
+  JSG_REQUIRE(norm_weight == nullptr || in_f <= cap, "%s: a fused RMSNorm handles at most %d features in this activation dtype, got %d", who, cap, in_f);
+  return 0;
+}
 
 }  // namespace jsg
 
@@ -351,9 +455,11 @@ int jsgrad_hip_linear(int kind, const void *w, const void *scale, int out_f, int
   JSG_REQUIRE(w && y && out_f > 0, "jsgrad_hip_linear: null weight/output or out_features %d", out_f);
   JSG_REQUIRE(kind < JSGRAD_W_I8 || scale, "jsgrad_hip_linear: quantised weight needs a scale");
   JSG_REQUIRE(y != x, "jsgrad_hip_linear: output must not alias the input");
+  if (int e = check_norm("jsgrad_hip_linear", norm_weight, act, in_f)) return e;
   GemvArgs a = {};
   a.w[0] = w; a.s[0] = scale; a.rows[0] = out_f; a.in_f = in_f; a.x = x; a.norm_w = norm_weight; a.eps = eps;
   a.inv_d = (float)(1.0 / (double)in_f); a.y = y; a.residual = residual;
+  ProfScope prof(PROF_LINEAR);
   return dispatch<EPI_STORE>(kind, act, a, out_f);
 }
 
@@ -363,9 +469,12 @@ int jsgrad_hip_ffn_gate(int kind, const void *w1, const void *s1, const void *w3
   if (int e = check_common("jsgrad_hip_ffn_gate", kind, act, dim, x)) return e;
   JSG_REQUIRE(w1 && w3 && g && hidden > 0, "jsgrad_hip_ffn_gate: null weight/output or hidden %d", hidden);
   JSG_REQUIRE(kind < JSGRAD_W_I8 || (s1 && s3), "jsgrad_hip_ffn_gate: quantised weights need scales");
+  JSG_REQUIRE(norm_weight, "jsgrad_hip_ffn_gate: null norm weight");
+  if (int e = check_norm("jsgrad_hip_ffn_gate", norm_weight, act, dim)) return e;
   GemvArgs a = {};
   a.w[0] = w1; a.s[0] = s1; a.w[1] = w3; a.s[1] = s3; a.rows[0] = hidden; a.rows[1] = hidden; a.in_f = dim; a.x = x;
   a.norm_w = norm_weight; a.eps = eps; a.inv_d = (float)(1.0 / (double)dim); a.y = g;
+  ProfScope prof(PROF_FFN_GATE);
   return dispatch<EPI_SWIGLU>(kind, act, a, hidden);
 }
 
@@ -379,11 +488,14 @@ int jsgrad_hip_qkv_rope(int kind, const void *wq, const void *sq, const void *wk
   JSG_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0, "jsgrad_hip_qkv_rope: n_heads %d must be a multiple of n_kv_heads %d", n_heads, n_kv_heads);
   JSG_REQUIRE(head_dim > 0 && head_dim % 4 == 0, "jsgrad_hip_qkv_rope: head_dim %d must be a multiple of 4", head_dim);
   JSG_REQUIRE(max_context > 0, "jsgrad_hip_qkv_rope: max_context %d", max_context);
+  JSG_REQUIRE(norm_weight, "jsgrad_hip_qkv_rope: null norm weight");
+  if (int e = check_norm("jsgrad_hip_qkv_rope", norm_weight, act, dim)) return e;
   GemvArgs a = {};
   a.w[0] = wq; a.s[0] = sq; a.w[1] = wk; a.s[1] = sk; a.w[2] = wv; a.s[2] = sv;
   a.rows[0] = n_heads * head_dim; a.rows[1] = n_kv_heads * head_dim; a.rows[2] = n_kv_heads * head_dim;
   a.in_f = dim; a.x = x; a.norm_w = norm_weight; a.eps = eps; a.inv_d = (float)(1.0 / (double)dim); a.y = q_out;
   a.rope_table = rope_table; a.st = st; a.cache_k = cache_k; a.cache_v = cache_v; a.head_dim = head_dim; a.max_context = max_context;
+  ProfScope prof(PROF_QKV_ROPE);
   return dispatch<EPI_ROPE_KV>(kind, act, a, a.rows[0] + a.rows[1] + a.rows[2]);
 }
 

@@ -28,6 +28,27 @@ int fail_hip(hipError_t e, const char *what) {
   return (int)e ? (int)e : 1;
 }
 
+
+// ---- profiling: one event pair per launch, summed per kernel kind when read back
+struct ProfState {
+  bool on = false;
+  std::vector<hipEvent_t> ev;  // 2 per slot
+  std::vector<int> kind;
+  size_t used = 0;
+};
+static ProfState g_prof;
+static constexpr size_t PROF_SLOTS = 16384;
+
+ProfScope::ProfScope(int k) : slot(-1) {
+  if (!g_prof.on || state().capturing || g_prof.used >= PROF_SLOTS) return;
+  slot = (int)g_prof.used++;
+  g_prof.kind[slot] = k;
+  (void)hipEventRecord(g_prof.ev[2 * slot], state().stream);
+}
+ProfScope::~ProfScope() {
+  if (slot >= 0) (void)hipEventRecord(g_prof.ev[2 * slot + 1], state().stream);
+}
+
 }  // namespace jsg
 
 using jsg::state;
@@ -191,6 +212,39 @@ int jsgrad_hip_event_elapsed_ms(void *start, void *stop, float *host_out_ms) {
 int jsgrad_hip_event_destroy(void *event) {
   JSG_READY();
   JSG_HIP(hipEventDestroy((hipEvent_t)event));
+  return 0;
+}
+
+int jsgrad_hip_profile(int enable) {
+  JSG_READY();
+  JSG_REQUIRE(!state().capturing, "jsgrad_hip_profile during graph capture");
+  jsg::ProfState &p = jsg::g_prof;
+  if (enable && p.ev.empty()) {
+    p.ev.resize(2 * jsg::PROF_SLOTS);
+    p.kind.resize(jsg::PROF_SLOTS);
+    for (auto &e : p.ev) JSG_HIP(hipEventCreate(&e));
+  }
+  JSG_HIP(hipStreamSynchronize(state().stream));
+  p.on = enable != 0;
+  p.used = 0;
+  return 0;
+}
+int jsgrad_hip_profile_read(int kind, int *host_out_count, double *host_out_total_ms) {
+  JSG_READY();
+  JSG_REQUIRE(kind >= 0 && kind < jsg::PROF_KINDS, "jsgrad_hip_profile_read: kind %d out of range", kind);
+  JSG_HIP(hipStreamSynchronize(state().stream));
+  jsg::ProfState &p = jsg::g_prof;
+  int n = 0;
+  double tot = 0.0;
+  for (size_t i = 0; i < p.used; i++) {
+    if (p.kind[i] != kind) continue;
+    float ms = 0.0f;
+    JSG_HIP(hipEventElapsedTime(&ms, p.ev[2 * i], p.ev[2 * i + 1]));
+    tot += ms;
+    n++;
+  }
+  *host_out_count = n;
+  *host_out_total_ms = tot;
   return 0;
 }
 

@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libjsgrad_hip.so")
 
 F32, F16 = 0, 1
 W_F32, W_F16, W_I8, W_NF4 = 0, 1, 2, 3
+PROF_KINDS = {"embed": 0, "rmsnorm": 1, "linear": 2, "qkv_rope": 3, "attn_decode": 4, "ffn_gate": 5, "argmax": 6}
 
 
 class HipError(RuntimeError):
@@ -44,6 +45,8 @@ SIGNATURES: dict[str, tuple[list, object]] = {
     "jsgrad_hip_event_record": ([_vp], _i32),
     "jsgrad_hip_event_elapsed_ms": ([_vp, _vp, C.POINTER(_f32)], _i32),
     "jsgrad_hip_event_destroy": ([_vp], _i32),
+    "jsgrad_hip_profile": ([_i32], _i32),
+    "jsgrad_hip_profile_read": ([_i32, C.POINTER(_i32), C.POINTER(C.c_double)], _i32),
     "jsgrad_hip_graph_begin": ([], _i32),
     "jsgrad_hip_graph_end": ([_pp], _i32),
     "jsgrad_hip_graph_launch": ([_vp], _i32),
@@ -56,7 +59,7 @@ SIGNATURES: dict[str, tuple[list, object]] = {
     "jsgrad_hip_attn_workspace_bytes": ([_i32, _i32, _i32], _sz),
     "jsgrad_hip_attn_decode": ([_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32], _i32),
     "jsgrad_hip_ffn_gate": ([_i32, _vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _i32, _i32, _i32], _i32),
-    "jsgrad_hip_argmax": ([_vp, _i32, _vp, _vp, _i32, _i32], _i32),
+    "jsgrad_hip_argmax": ([_vp, _i32, _vp, _vp, _i32, _i32, _i32], _i32),
     "jsgrad_hip_int8_quantize": ([_vp, _i32, _i32, _vp, _vp, _i32], _i32),
     "jsgrad_hip_int8_dequant": ([_vp, _vp, _i32, _i32, _vp], _i32),
     "jsgrad_hip_nf4_quantize": ([_vp, _sz, _vp, _vp, _i32], _i32),

@@ -181,7 +181,7 @@ class Transformer:
         for layer in self.layers:
             h = layer.call(h, self.state, self.freqs_cis, ctx)
         self.output.call(h, out=ctx.logits, norm=self.norm)
-        check(ffi.load().jsgrad_hip_argmax(ctx.logits.ptr, self.vocab_size, self.state.ptr, self.tokens_out.ptr, 1, act_code(self.dtype)))
+        check(ffi.load().jsgrad_hip_argmax(ctx.logits.ptr, self.vocab_size, self.state.ptr, self.tokens_out.ptr, self.max_context, 1, act_code(self.dtype)))
         return Tensor(buffer=self.state.lazydata.view(1, "int32", 0), shape=(), dtype="int32", device=self.device)
 
     def _advance_host_pos(self) -> None:

@@ -76,6 +76,13 @@ int jsgrad_hip_event_record(void *event);
 int jsgrad_hip_event_elapsed_ms(void *start, void *stop, float *host_out_ms); /* waits for `stop` */
 int jsgrad_hip_event_destroy(void *event);
 
+/* Per-kernel statistics (DEBUG>=2 of engine/realize.ts:168-178; ProfileRangeEvent, runtime/allocator.ts:147-151):
+ * while enabled, every Llama kernel launched outside a graph capture is bracketed by an event pair.  `read` waits
+ * for the stream and returns launch count and summed milliseconds of one kind since profiling was enabled. */
+enum { JSGRAD_PROF_EMBED = 0, JSGRAD_PROF_RMSNORM, JSGRAD_PROF_LINEAR, JSGRAD_PROF_QKV_ROPE, JSGRAD_PROF_ATTN, JSGRAD_PROF_FFN_GATE, JSGRAD_PROF_ARGMAX };
+int jsgrad_hip_profile(int enable);
+int jsgrad_hip_profile_read(int kind, int *host_out_count, double *host_out_total_ms);
+
 /* TinyJit capture / replay as a device graph (engine/jit.ts:14-69 apply_graph_to_jit, :71 GraphRunner,
  * `Compiled.graph` allocator.ts:176): everything queued between begin and end becomes one HIP graph. */
 int jsgrad_hip_graph_begin(void);
@@ -130,8 +137,9 @@ int jsgrad_hip_ffn_gate(int kind, const void *w1, const void *s1, const void *w3
 
 /* sample() at temperature 0 (models/llama.ts:137 -> Tensor.argmax tensor.ts:2314-2320): lowest index among
  * the maxima of logits[n] (activation dtype).  Writes the token to state[0] and, when advance != 0,
- * increments state[1]; tokens_out != NULL also receives the token at tokens_out[old start_pos]. */
-int jsgrad_hip_argmax(const void *logits, int n, int32_t *state, int32_t *tokens_out, int advance, int act);
+ * increments state[1]; tokens_out != NULL (an int32[tokens_cap] history) also receives the token at
+ * tokens_out[old start_pos] when that index is inside it. */
+int jsgrad_hip_argmax(const void *logits, int n, int32_t *state, int32_t *tokens_out, int tokens_cap, int advance, int act);
 
 /* ---------------------------------------------------------------------------------
  * Load-time kernels
