@@ -190,35 +190,33 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_decode_kernel(AttnArgs a) {
     float v = 0.0f;
 #pragma unroll
     for (int w = 0; w < NW; w++) v += o_part[w][j][d];
-    mine[j * (HD + 2) + d] = v;
+    st_coherent(&mine[j * (HD + 2) + d], v);
   }
   if (tid < NREP) {
-    mine[tid * (HD + 2) + HD] = m_sh[tid];
-    mine[tid * (HD + 2) + HD + 1] = l_sh[tid];
+    st_coherent(&mine[tid * (HD + 2) + HD], m_sh[tid]);
+    st_coherent(&mine[tid * (HD + 2) + HD + 1], l_sh[tid]);
   }
 
   // ---- publish, and let the last chunk of this kv head merge
-  __threadfence();
-  __syncthreads();
+  __syncthreads();  // every coherent store of the block has been acknowledged
   if (tid == 0) {
-    int old = __hip_atomic_fetch_add(&a.counters[g], 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    int old = __hip_atomic_fetch_add(&a.counters[g], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     is_last = (old == n_active - 1);
   }
   __syncthreads();
   if (!is_last) return;
-  __threadfence();
   // merge: one wavefront per query head turns the per-chunk (m, l) into weights exp(m_s - M) and 1/L ...
   const float *base = a.partial + (size_t)g * a.nsplit * NREP * (HD + 2);
   for (int j = wave; j < NREP; j += NW) {
     float M = -INFINITY;
-    for (int s = lane; s < n_active; s += 64) M = fmaxf(M, __builtin_nontemporal_load(base + ((size_t)s * NREP + j) * (HD + 2) + HD));
+    for (int s = lane; s < n_active; s += 64) M = fmaxf(M, ld_coherent(base + ((size_t)s * NREP + j) * (HD + 2) + HD));
     M = wave_max(M);
     float L = 0.0f;
     for (int s = lane; s < n_active; s += 64) {
       const float *ps = base + ((size_t)s * NREP + j) * (HD + 2);
-      const float w = exp_f32(__builtin_nontemporal_load(ps + HD) - M);
+      const float w = exp_f32(ld_coherent(ps + HD) - M);
       sc[j][s] = w;  // n_active <= nsplit <= ATT_CHUNK_MAX
-      L = fmaf(__builtin_nontemporal_load(ps + HD + 1), w, L);
+      L = fmaf(ld_coherent(ps + HD + 1), w, L);
     }
     L = wave_sum(L);
     if (lane == 0) l_sh[j] = 1.0f / L;  // softmax normalisation is e * (1/sum) (tensor.ts:2211-2214)
@@ -230,7 +228,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_decode_kernel(AttnArgs a) {
     const float *po = base + (size_t)j * (HD + 2) + d;
     float O = 0.0f;
 #pragma unroll 8
-    for (int s = 0; s < n_active; s++) O = fmaf(__builtin_nontemporal_load(po + (size_t)s * NREP * (HD + 2)), sc[j][s], O);
+    for (int s = 0; s < n_active; s++) O = fmaf(ld_coherent(po + (size_t)s * NREP * (HD + 2)), sc[j][s], O);
     ((AT *)a.out)[(size_t)(g * NREP + j) * HD + d] = (AT)Act<AT>::rn(O * l_sh[j]);  // the cast of the P.V result
   }
   if (tid == 0) __hip_atomic_store(&a.counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -248,14 +246,13 @@ template <typename AT, int HD> static int launch_attn(const AttnArgs &a, int n_r
   dim3 grid(a.n_kv_heads, a.nsplit), block(ATT_THREADS);
 #define JSG_REP(N)                                                                                   \
   case N:                                                                                            \
-    hipLaunchKernelGGL((attn_decode_kernel<AT, HD, N>), grid, block, 0, state().stream, a);            \
+    JSG_LAUNCH(PROF_ATTN, (attn_decode_kernel<AT, HD, N>), grid, block, 0, a);                         \
     break;
   switch (n_rep) {
     JSG_REP(1) JSG_REP(2) JSG_REP(3) JSG_REP(4) JSG_REP(8)
     default: return fail("jsgrad_hip_attn_decode: n_heads/n_kv_heads = %d is not one of 1,2,3,4,8", n_rep);
   }
 #undef JSG_REP
-  JSG_LAUNCHED();
   return 0;
 }
 
@@ -286,7 +283,6 @@ int jsgrad_hip_attn_decode(const void *q, const void *cache_k, const void *cache
   a.n_kv_heads = n_kv_heads; a.nsplit = nsplit_for(max_context); a.max_context = max_context;
   a.scale = (float)(1.0 / sqrt((double)head_dim));
   const int n_rep = n_heads / n_kv_heads;
-  ProfScope prof(PROF_ATTN);
   if (act == JSGRAD_F16) return head_dim == 64 ? launch_attn<_Float16, 64>(a, n_rep) : launch_attn<_Float16, 128>(a, n_rep);
   return head_dim == 64 ? launch_attn<float, 64>(a, n_rep) : launch_attn<float, 128>(a, n_rep);
 }

@@ -1,6 +1,7 @@
 // Shared device/host helpers for libjsgrad_hip.so (gfx950 only).
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -23,11 +24,19 @@ int fail_hip(hipError_t e, const char *what);
 
 // per-kernel timing with HIP events on the library stream (off unless jsgrad_hip_profile(1))
 enum { PROF_EMBED = 0, PROF_RMSNORM, PROF_LINEAR, PROF_QKV_ROPE, PROF_ATTN, PROF_FFN_GATE, PROF_ARGMAX, PROF_KINDS };
-struct ProfScope {
-  int slot;
-  explicit ProfScope(int kind);
-  ~ProfScope();
-};
+// Event pair for the next launch of `kind`, or false when profiling is off (or capturing, or out of slots).  The pair
+// is handed to hipExtLaunchKernelGGL, which stamps it with the dispatch's own begin/end times, so the elapsed time is
+// the kernel alone: no marker packets, no launch latency.
+bool prof_events(int kind, hipEvent_t *start, hipEvent_t *stop);
+
+// Launch on the library stream, timed when profiling is on.
+#define JSG_LAUNCH(kind, kernel, grid, block, lds, ...)                                                                  \
+  do {                                                                                                                   \
+    hipEvent_t ps_, pe_;                                                                                                 \
+    if (jsg::prof_events(kind, &ps_, &pe_)) hipExtLaunchKernelGGL(kernel, grid, block, lds, jsg::state().stream, ps_, pe_, 0, __VA_ARGS__); \
+    else hipLaunchKernelGGL(kernel, grid, block, lds, jsg::state().stream, __VA_ARGS__);                                 \
+    JSG_LAUNCHED();                                                                                                      \
+  } while (0)
 
 #define JSG_HIP(call)                                   \
   do {                                                  \
@@ -76,6 +85,16 @@ template <> struct Act<_Float16> {
   __device__ static __forceinline__ float ld(const _Float16 *p) { return (float)*p; }
   __device__ static __forceinline__ void st(_Float16 *p, float f) { *p = (_Float16)f; }
 };
+
+// Cross-block hand-off without cache-wide fences.  Data that another block will read in the same launch is written
+// with agent-scope (write-through) stores and read with agent-scope loads, which are served at the device-wide
+// coherence point rather than from a per-XCD L2 copy.  A block publishes by: coherent stores -> __syncthreads (which
+// waits for the stores to be acknowledged) -> one relaxed agent-scope atomic on a counter.  A full release/acquire
+// fence would write back and invalidate the whole L2 of the XCD once per block, which costs far more than the kernel.
+__device__ __forceinline__ void st_coherent(float *p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void st_coherent(int *p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ float ld_coherent(const float *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ int ld_coherent(const int *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
 // DPP cross-lane moves inside a 64-lane wavefront
 template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {

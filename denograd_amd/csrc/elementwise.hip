@@ -74,19 +74,18 @@ template <typename AT> __global__ __launch_bounds__(ARGMAX_THREADS) void argmax_
   };
   block_reduce();
   if (tid == 0) {
-    g_argmax_val[blockIdx.x] = best;
-    g_argmax_idx[blockIdx.x] = bi;
-    __threadfence();
-    is_last = __hip_atomic_fetch_add(&g_argmax_count, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == (int)gridDim.x - 1;
+    st_coherent(&g_argmax_val[blockIdx.x], best);
+    st_coherent(&g_argmax_idx[blockIdx.x], bi);
+    __builtin_amdgcn_s_waitcnt(0);  // both stores acknowledged before the counter moves
+    is_last = __hip_atomic_fetch_add(&g_argmax_count, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (int)gridDim.x - 1;
   }
   __syncthreads();
   if (!is_last) return;
-  __threadfence();
   best = -INFINITY;
   bi = 0x7fffffff;
   if (tid < (int)gridDim.x) {
-    best = __builtin_nontemporal_load(&g_argmax_val[tid]);
-    bi = __builtin_nontemporal_load(&g_argmax_idx[tid]);
+    best = ld_coherent(&g_argmax_val[tid]);
+    bi = ld_coherent(&g_argmax_idx[tid]);
   }
   __syncthreads();  // vmax / imax are reused
   block_reduce();
@@ -306,9 +305,8 @@ int jsgrad_hip_embed(int kind, const void *table, const void *scale, const int32
   JSG_REQUIRE(kind == JSGRAD_W_F32 || kind == JSGRAD_W_F16 || kind == JSGRAD_W_I8, "jsgrad_hip_embed: table kind %d", kind);
   JSG_REQUIRE(kind != JSGRAD_W_I8 || scale, "jsgrad_hip_embed: int8 table needs row scales");
   dim3 grid((dim + 255) / 256), block(256);
-  ProfScope prof(PROF_EMBED);
-  if (act == JSGRAD_F16) hipLaunchKernelGGL(embed_kernel<_Float16>, grid, block, 0, state().stream, kind, table, (const _Float16 *)scale, st, (_Float16 *)out, dim, vocab);
-  else if (act == JSGRAD_F32) hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, state().stream, kind, table, (const _Float16 *)scale, st, (float *)out, dim, vocab);
+  if (act == JSGRAD_F16) JSG_LAUNCH(PROF_EMBED, (embed_kernel<_Float16>), grid, block, 0, kind, table, (const _Float16 *)scale, st, (_Float16 *)out, dim, vocab);
+  else if (act == JSGRAD_F32) JSG_LAUNCH(PROF_EMBED, (embed_kernel<float>), grid, block, 0, kind, table, (const _Float16 *)scale, st, (float *)out, dim, vocab);
   else return fail("jsgrad_hip_embed: unknown activation dtype %d", act);
   JSG_LAUNCHED();
   return 0;
@@ -318,9 +316,8 @@ int jsgrad_hip_rmsnorm(const void *x, const void *weight, void *y, int dim, floa
   JSG_READY();
   JSG_REQUIRE(x && weight && y && dim > 0, "jsgrad_hip_rmsnorm: bad argument");
   const float inv_d = (float)(1.0 / (double)dim);
-  ProfScope prof(PROF_RMSNORM);
-  if (act == JSGRAD_F16) hipLaunchKernelGGL(rmsnorm_kernel<_Float16>, dim3(1), dim3(1024), 0, state().stream, (const _Float16 *)x, (const _Float16 *)weight, (_Float16 *)y, dim, eps, inv_d);
-  else if (act == JSGRAD_F32) hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(1), dim3(1024), 0, state().stream, (const float *)x, (const float *)weight, (float *)y, dim, eps, inv_d);
+  if (act == JSGRAD_F16) JSG_LAUNCH(PROF_RMSNORM, (rmsnorm_kernel<_Float16>), dim3(1), dim3(1024), 0, (const _Float16 *)x, (const _Float16 *)weight, (_Float16 *)y, dim, eps, inv_d);
+  else if (act == JSGRAD_F32) JSG_LAUNCH(PROF_RMSNORM, (rmsnorm_kernel<float>), dim3(1), dim3(1024), 0, (const float *)x, (const float *)weight, (float *)y, dim, eps, inv_d);
   else return fail("jsgrad_hip_rmsnorm: unknown activation dtype %d", act);
   JSG_LAUNCHED();
   return 0;
@@ -330,9 +327,8 @@ int jsgrad_hip_argmax(const void *logits, int n, int32_t *st, int32_t *tokens_ou
   JSG_READY();
   JSG_REQUIRE(logits && st && n > 0, "jsgrad_hip_argmax: bad argument");
   const int nb = n >= ARGMAX_BLOCKS * ARGMAX_THREADS ? ARGMAX_BLOCKS : (n + ARGMAX_THREADS - 1) / ARGMAX_THREADS;
-  ProfScope prof(PROF_ARGMAX);
-  if (act == JSGRAD_F16) hipLaunchKernelGGL(argmax_kernel<_Float16>, dim3(nb), dim3(ARGMAX_THREADS), 0, state().stream, (const _Float16 *)logits, n, st, tokens_out, tokens_cap, advance);
-  else if (act == JSGRAD_F32) hipLaunchKernelGGL(argmax_kernel<float>, dim3(nb), dim3(ARGMAX_THREADS), 0, state().stream, (const float *)logits, n, st, tokens_out, tokens_cap, advance);
+  if (act == JSGRAD_F16) JSG_LAUNCH(PROF_ARGMAX, (argmax_kernel<_Float16>), dim3(nb), dim3(ARGMAX_THREADS), 0, (const _Float16 *)logits, n, st, tokens_out, tokens_cap, advance);
+  else if (act == JSGRAD_F32) JSG_LAUNCH(PROF_ARGMAX, (argmax_kernel<float>), dim3(nb), dim3(ARGMAX_THREADS), 0, (const float *)logits, n, st, tokens_out, tokens_cap, advance);
   else return fail("jsgrad_hip_argmax: unknown activation dtype %d", act);
   JSG_LAUNCHED();
   return 0;

@@ -248,7 +248,13 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemvArgs a) {
   const int gstride = gridDim.x * nw;
   const int nsteps = (in_f + STEP - 1) / STEP;
   const int nbatch = (nsteps + UNROLL - 1) / UNROLL;
-  typedef u4_t Buf[UNROLL][NM][ROWS];
+  // One item's registers: the weight vectors plus, on the item that finishes a row group, the operands its epilogue
+  // will need (row scales, residual, rotary pair), fetched now so that no load latency is left at the end.
+  struct Buf {
+    u4_t w[UNROLL][NM][ROWS];
+    float scale[NM][ROWS];
+    float extra[ROWS];   // EPI_STORE: residual[row]; EPI_ROPE_KV: (cos, sin) of the pair in extra[r], extra[r+1]
+  };
   // read the position now, not in the epilogue: the load then overlaps the weight stream instead of ending the kernel
   const int pos = EPI == EPI_ROPE_KV ? a.st[1] : 0;
 
@@ -279,8 +285,25 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemvArgs a) {
           for (int r = 0; r < ROWS; r++) {
             const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;  // tail rows reload the last row, never stored
             const char *p = (const char *)wbase(w.m, j) + (((size_t)row * in_f + (size_t)k) * BITS) / 8;
-            buf[u][j][r] = __builtin_nontemporal_load((const u4_t *)p);
+            buf.w[u][j][r] = __builtin_nontemporal_load((const u4_t *)p);
           }
+      }
+    }
+    if (b != nbatch - 1) return;
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+      const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;
+      if constexpr (KIND == JSGRAD_W_I8) {
+#pragma unroll
+        for (int j = 0; j < NM; j++) buf.scale[j][r] = (float)((const _Float16 *)sbase(w.m, j))[row];
+      }
+      if constexpr (EPI == EPI_STORE) {
+        buf.extra[r] = a.residual ? (float)((const AT *)a.residual)[row] : 0.0f;
+      } else if constexpr (EPI == EPI_ROPE_KV) {
+        // table row `pos`, entry (cos, sin) of pair i = (row % head_dim) / 2: even r gets cos, odd r gets sin
+        const bool ok = pos >= 0 && pos < a.max_context;
+        const int i = (row % a.head_dim) >> 1;
+        buf.extra[r] = ok ? (float)((const AT *)a.rope_table)[(size_t)pos * a.head_dim + 2 * i + (r & 1)] : 0.0f;
       }
     }
   };
@@ -309,7 +332,7 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemvArgs a) {
               const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;
               bs = (float)((const _Float16 *)sbase(w.m, j))[((size_t)row * in_f + k) >> 6];
             }
-            acc[j][r] = Dot<KIND, AT>::run(buf[u][j][r], xf, acc[j][r], bs, lut);
+            acc[j][r] = Dot<KIND, AT>::run(buf.w[u][j][r], xf, acc[j][r], bs, lut);
           }
       }
     }
@@ -322,21 +345,18 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemvArgs a) {
 #pragma unroll
       for (int r = 0; r < ROWS; r++) {
         float v = wave_sum(acc[j][r]);
-        if constexpr (KIND == JSGRAD_W_I8) {
-          const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;
-          v = v * (float)((const _Float16 *)sbase(w.m, j))[row];
-        }
+        if constexpr (KIND == JSGRAD_W_I8) v = v * buf.scale[j][r];
         val[j][r] = Act<AT>::rn(v);
       }
     const int r0 = w.r0, mrows = w.mrows;
     if constexpr (EPI == EPI_STORE) {
       AT *y = (AT *)a.y;
-      const AT *res = (const AT *)a.residual;
+      const bool has_res = a.residual != nullptr;
 #pragma unroll
       for (int r = 0; r < ROWS; r++)
         if (lane == r && r0 + r < mrows) {
           float v = val[0][r];
-          if (res) v = Act<AT>::rn((float)res[r0 + r] + v);
+          if (has_res) v = Act<AT>::rn(buf.extra[r] + v);
           y[r0 + r] = (AT)v;
         }
     } else if constexpr (EPI == EPI_SWIGLU) {
@@ -346,20 +366,17 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemvArgs a) {
         if (lane == r && r0 + r < mrows) g[r0 + r] = (AT)Act<AT>::rn(silu_act<AT>(val[0][r]) * val[1][r]);
     } else {
       if (pos < 0 || pos >= a.max_context) return;  // never write outside the cache
-      const int hd = a.head_dim;
       if (w.m == 2) {  // value rows: plain copy into the cache row
         AT *cv = (AT *)a.cache_v + (size_t)pos * a.rows[2];
 #pragma unroll
         for (int r = 0; r < ROWS; r++)
           if (lane == r && r0 + r < mrows) cv[r0 + r] = (AT)val[0][r];
       } else {         // query / key rows: rotate interleaved pairs (llama.ts:17-32)
-        const AT *tab = (const AT *)a.rope_table + (size_t)pos * hd;
         AT *dst = w.m == 0 ? (AT *)a.y : (AT *)a.cache_k + (size_t)pos * a.rows[1];
 #pragma unroll
         for (int r = 0; r < ROWS; r += 2)
           if (lane == r && r0 + r + 1 < mrows) {
-            const int i = ((r0 + r) % hd) >> 1;
-            const float c = (float)tab[2 * i], d = (float)tab[2 * i + 1];
+            const float c = buf.extra[r], d = buf.extra[r + 1];
             const float av = val[0][r], bv = val[0][r + 1];
             dst[r0 + r] = (AT)Act<AT>::rn(av * c - bv * d);  // the build keeps a*b+c unfused: two roundings as in plain C
             dst[r0 + r + 1] = (AT)Act<AT>::rn(av * d + bv * c);
@@ -395,14 +412,14 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemvArgs a) {
 // ---- host-side dispatch ------------------------------------------------------------------------
 
 template <int KIND, typename AT, int EPI, int ROWS, int UNROLL> static int launch_cfg(const GemvArgs &a, int total_rows) {
+  constexpr int kind = EPI == EPI_STORE ? PROF_LINEAR : (EPI == EPI_SWIGLU ? PROF_FFN_GATE : PROF_QKV_ROPE);
   constexpr int NW = 4;
   const int ngroups = (total_rows + ROWS - 1) / ROWS;
   const int need = (ngroups + NW - 1) / NW;      // one group per wavefront
   const int cap = state().cu_count * 4;          // 16 resident wavefronts per CU; more rows than that are walked grid-stride
   dim3 grid(need < cap ? need : cap), block(NW * 64);
   size_t lds = (size_t)a.in_f * sizeof(AT);
-  hipLaunchKernelGGL((gemv_kernel<KIND, AT, EPI, ROWS, UNROLL>), grid, block, lds, state().stream, a);
-  JSG_LAUNCHED();
+  JSG_LAUNCH(kind, (gemv_kernel<KIND, AT, EPI, ROWS, UNROLL>), grid, block, lds, a);
   return 0;
 }
 // Two register buffers of UNROLL x NM x ROWS 16-byte loads each: (2 rows, 4 steps) for one matrix, (2 rows, 2 steps)
@@ -459,7 +476,6 @@ int jsgrad_hip_linear(int kind, const void *w, const void *scale, int out_f, int
   GemvArgs a = {};
   a.w[0] = w; a.s[0] = scale; a.rows[0] = out_f; a.in_f = in_f; a.x = x; a.norm_w = norm_weight; a.eps = eps;
   a.inv_d = (float)(1.0 / (double)in_f); a.y = y; a.residual = residual;
-  ProfScope prof(PROF_LINEAR);
   return dispatch<EPI_STORE>(kind, act, a, out_f);
 }
 
@@ -474,7 +490,6 @@ int jsgrad_hip_ffn_gate(int kind, const void *w1, const void *s1, const void *w3
   GemvArgs a = {};
   a.w[0] = w1; a.s[0] = s1; a.w[1] = w3; a.s[1] = s3; a.rows[0] = hidden; a.rows[1] = hidden; a.in_f = dim; a.x = x;
   a.norm_w = norm_weight; a.eps = eps; a.inv_d = (float)(1.0 / (double)dim); a.y = g;
-  ProfScope prof(PROF_FFN_GATE);
   return dispatch<EPI_SWIGLU>(kind, act, a, hidden);
 }
 
@@ -495,7 +510,6 @@ int jsgrad_hip_qkv_rope(int kind, const void *wq, const void *sq, const void *wk
   a.rows[0] = n_heads * head_dim; a.rows[1] = n_kv_heads * head_dim; a.rows[2] = n_kv_heads * head_dim;
   a.in_f = dim; a.x = x; a.norm_w = norm_weight; a.eps = eps; a.inv_d = (float)(1.0 / (double)dim); a.y = q_out;
   a.rope_table = rope_table; a.st = st; a.cache_k = cache_k; a.cache_v = cache_v; a.head_dim = head_dim; a.max_context = max_context;
-  ProfScope prof(PROF_QKV_ROPE);
   return dispatch<EPI_ROPE_KV>(kind, act, a, a.rows[0] + a.rows[1] + a.rows[2]);
 }
 

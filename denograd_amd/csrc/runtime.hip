@@ -39,14 +39,13 @@ struct ProfState {
 static ProfState g_prof;
 static constexpr size_t PROF_SLOTS = 16384;
 
-ProfScope::ProfScope(int k) : slot(-1) {
-  if (!g_prof.on || state().capturing || g_prof.used >= PROF_SLOTS) return;
-  slot = (int)g_prof.used++;
-  g_prof.kind[slot] = k;
-  (void)hipEventRecord(g_prof.ev[2 * slot], state().stream);
-}
-ProfScope::~ProfScope() {
-  if (slot >= 0) (void)hipEventRecord(g_prof.ev[2 * slot + 1], state().stream);
+bool prof_events(int kind, hipEvent_t *start, hipEvent_t *stop) {
+  if (!g_prof.on || state().capturing || g_prof.used >= PROF_SLOTS) return false;
+  const size_t slot = g_prof.used++;
+  g_prof.kind[slot] = kind;
+  *start = g_prof.ev[2 * slot];
+  *stop = g_prof.ev[2 * slot + 1];
+  return true;
 }
 
 }  // namespace jsg
