@@ -65,16 +65,16 @@ def kernel_bytes(cfg, T):
     }
 
 
-def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=True, blocker_steps=40):
+def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=True, blocker_steps=40, per_op_steps=64, fused_step=False):
     from denograd_amd import ffi, synthetic
     from denograd_amd.ffi import check
     from denograd_amd.llama3 import Llama3
 
     lib = ffi.load()
-    ctx = prompt_len + warmup + steps + profile_steps + blocker_steps + 8
+    ctx = prompt_len + warmup + steps + 2 * (profile_steps + blocker_steps) + per_op_steps + 16
     cfg = synthetic.config(name, max_context=ctx)
     t0 = time.perf_counter()
-    llm = Llama3.from_config(cfg).random_init(seed=0, tied=cfg["tied"])
+    llm = Llama3.from_config(cfg, fused_step=fused_step).random_init(seed=0, tied=cfg["tied"])
     if not use_graph:
         llm.model.forward_jit = None     # the same kernels, launched one by one instead of replayed as a graph
     check(lib.jsgrad_hip_sync())
@@ -109,40 +109,78 @@ def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=Tru
     # per-kernel durations: the same step, eager, with a start/stop event pair attached to every dispatch (the
     # dispatch's own begin/end stamps, as a kernel trace reports them).  Graph replays are queued first and not waited
     # for, so the eager launches run back to back like the replayed ones.
-    check(lib.jsgrad_hip_profile(1))
-    if use_graph:
-        m.generate(blocker_steps)
-        llm.start_pos += blocker_steps
-    for _ in range(profile_steps):
-        m._step()
-    kinds = {}
-    for kname, kid in ffi.PROF_KINDS.items():
-        n, tot = C.c_int(), C.c_double()
-        check(lib.jsgrad_hip_profile_read(kid, C.byref(n), C.byref(tot)))
-        if n.value:
-            kinds[kname] = {"launches_per_step": n.value // profile_steps, "ms_per_step": tot.value / profile_steps}
-    check(lib.jsgrad_hip_profile(0))
-    llm.start_pos += profile_steps
+    def profiled(n_steps):
+        check(lib.jsgrad_hip_profile(1))
+        if use_graph:
+            m.generate(blocker_steps)
+            llm.start_pos += blocker_steps
+        for _ in range(n_steps):
+            m._step()
+        kinds = {}
+        for kname, kid in ffi.PROF_KINDS.items():
+            n, tot = C.c_int(), C.c_double()
+            check(lib.jsgrad_hip_profile_read(kid, C.byref(n), C.byref(tot)))
+            if n.value:
+                kinds[kname] = {"launches_per_step": n.value // n_steps, "ms_per_step": tot.value / n_steps}
+        check(lib.jsgrad_hip_profile(0))
+        llm.start_pos += n_steps
+        return kinds
+
+    fused = m._fused is not None
+    kinds = profiled(profile_steps)
+    per_op = None
+    if fused:
+        # the same model through the one-launch-per-op path, for the per-family table and as a second data point
+        saved, m._fused = m._fused, None
+        if m.forward_jit is not None:
+            m.forward_jit.reset()
+        m._step(); m._step()
+        llm.start_pos += 2
+        check(lib.jsgrad_hip_sync())
+        w1 = time.perf_counter()
+        m.generate(per_op_steps)
+        check(lib.jsgrad_hip_sync())
+        per_op_ms = 1e3 * (time.perf_counter() - w1) / per_op_steps
+        llm.start_pos += per_op_steps
+        per_op = profiled(profile_steps)
+        m._fused = saved
+        if m.forward_jit is not None:
+            m.forward_jit.reset()
+    fam = per_op if fused else kinds
     kb = kernel_bytes(cfg, llm.start_pos)
-    for kname, b in kb.items():
-        k = kinds[kname]
-        k["bytes_per_step"] = int(b)
+    for kname, b_ in kb.items():
+        k = fam[kname]
+        k["bytes_per_step"] = int(b_)
         k["avg_us_per_launch"] = 1e3 * k["ms_per_step"] / k["launches_per_step"]
-        k["GBps"] = b / (k["ms_per_step"] * 1e-3) / 1e9
-    dom = "linear"   # wo, w2 and the lm_head: the weight-streaming family with the most launches and (with ffn_gate) the most time
-    achieved = kinds[dom]["GBps"]
+        k["GBps"] = b_ / (k["ms_per_step"] * 1e-3) / 1e9
     bytes_tok = synthetic.weight_bytes_per_token(cfg) + synthetic.kv_bytes_per_position(cfg) * t_avg
+    if fused:
+        # one launch = one token: the step kernel is the dominant (only) kernel
+        step_ms = kinds["decode_step"]["ms_per_step"]
+        bytes_now = synthetic.weight_bytes_per_token(cfg) + synthetic.kv_bytes_per_position(cfg) * llm.start_pos
+        achieved = bytes_now / (step_ms * 1e-3) / 1e9
+        roof = {"bound": "hbm", "kernel": "decode_step_kernel (whole token: embedding, 5 phases x layers, lm_head, argmax)", "achieved": round(achieved, 1),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get((name, "decode_step")),
+                "bytes_per_launch": int(bytes_now), "avg_us_per_launch": round(step_ms * 1e3, 2)}
+    else:
+        dom = "linear"   # wo, w2 and the lm_head: the weight-streaming family with the most launches and (with ffn_gate) the most time
+        achieved = fam[dom]["GBps"]
+        roof = {"bound": "hbm", "kernel": f"gemv_kernel ({dom})", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get((name, dom)),
+                "bytes_per_launch": int(kb[dom] / fam[dom]["launches_per_step"]), "avg_us_per_launch": round(fam[dom]["avg_us_per_launch"], 2)}
+    rnd = lambda d: {k: {kk: (round(vv, 3) if isinstance(vv, float) else vv) for kk, vv in v.items()} for k, v in d.items()}
     res = {
         "name": name, "tok_s": tok_s, "ms_per_step": 1e3 * wall / steps, "event_ms_per_step": ms.value / steps,
-        "roofline": {"bound": "hbm", "kernel": f"gemv_kernel ({dom})", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get((name, dom)),
-                     "bytes_per_launch": int(kb[dom] / kinds[dom]["launches_per_step"]), "avg_us_per_launch": round(kinds[dom]["avg_us_per_launch"], 2)},
+        "roofline": roof,
         "step_roofline": {"bytes_per_token": int(bytes_tok), "achieved": round(bytes_tok * tok_s / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                           "frac": round(bytes_tok * tok_s / 1e9 / HBM_PEAK_GBS, 4)},
-        "kernels": {k: {kk: (round(vv, 3) if isinstance(vv, float) else vv) for kk, vv in v.items()} for k, v in kinds.items()},
+        "kernels": rnd(kinds),
         "config": {"workload": f"Llama-3 decode bs=1, {name}-shaped random init ({cfg['quantize']}), {prompt_len}-token prompt, {steps} greedy tokens",
-                   "prompt": prompt_len, "decode": steps, "avg_visible_positions": t_avg, "max_context": ctx},
+                   "prompt": prompt_len, "decode": steps, "avg_visible_positions": t_avg, "max_context": ctx,
+                   "launch": ("one persistent kernel per token" if fused else "one launch per fused op") + (", replayed as a HIP graph" if use_graph else ", eager")},
     }
+    if per_op is not None:
+        res["per_op_path"] = {"tok_s": round(1e3 / per_op_ms, 2), "ms_per_step": round(per_op_ms, 4), "kernels": rnd(per_op)}
     return llm, cfg, res
 
 
@@ -209,6 +247,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle baseline")
     ap.add_argument("--traffic-probe", action="store_true", help="for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: one 512 MiB device-to-device copy "
                     "(a plain copy kernel of known size, to scale the counters) followed by 4 eager decode steps of --workload; prints nothing")
+    ap.add_argument("--fused-step", action="store_true", help="run each token as one persistent kernel (jsgrad_hip_decode_step) instead of one launch per fused op")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel eagerly instead of replaying a captured HIP graph "
                     "(rocprofv3 --kernel-trace on this image crashes inside hipGraphLaunch, so profiles are taken this way)")
     args = ap.parse_args()
@@ -224,12 +263,12 @@ def main():
     if args.traffic_probe:
         traffic_probe(args.workload)
         return
-    llm, cfg, res = run_workload(args.workload, args.prompt, args.steps, args.warmup, use_graph=not args.no_graph)
+    llm, cfg, res = run_workload(args.workload, args.prompt, args.steps, args.warmup, use_graph=not args.no_graph, fused_step=args.fused_step)
     cpu = None if args.no_cpu else cpu_baseline(llm, cfg)
     del llm
     secondary = None
     if args.secondary:
-        llm2, cfg2, secondary = run_workload(args.secondary, args.prompt, args.secondary_steps, args.warmup, use_graph=not args.no_graph)
+        llm2, cfg2, secondary = run_workload(args.secondary, args.prompt, args.secondary_steps, args.warmup, use_graph=not args.no_graph, fused_step=args.fused_step)
         del llm2
 
     out = {
@@ -239,12 +278,12 @@ def main():
         "dtype": "f16", "data": "synthetic", "config": res["config"],
         "roofline": res["roofline"], "cpu_baseline": cpu,
         "step_roofline": res["step_roofline"], "kernels": res["kernels"], "event_ms_per_step": round(res["event_ms_per_step"], 4),
-        "launch_mode": "eager" if args.no_graph else "hip_graph",
+        "launch_mode": "eager" if args.no_graph else "hip_graph", "per_op_path": res.get("per_op_path"),
     }
     if secondary:
         out["secondary"] = {"value": round(secondary["tok_s"], 2), "unit": "tok/s", "steps": args.secondary_steps, "ms_per_step": round(secondary["ms_per_step"], 4),
                             "dtype": "i8 weights, f16 activations", "config": secondary["config"], "roofline": secondary["roofline"],
-                            "step_roofline": secondary["step_roofline"], "kernels": secondary["kernels"]}
+                            "step_roofline": secondary["step_roofline"], "kernels": secondary["kernels"], "per_op_path": secondary.get("per_op_path")}
     print(json.dumps(out), flush=True)
 
 

@@ -1,50 +1,15 @@
-// Decode-time grouped-query attention over the HBM-resident KV cache for gfx950.
-//
-// One new query position against cache rows [0, T), T = start_pos + 1: repeat_kv +
-// scaled_dot_product_attention of the reference (/root/reference/jsgrad/models/llama.ts:89-95,
-// /root/reference/jsgrad/tensor.ts:3920-3934).  Scores, the softmax and the P.V sum are float32; the
-// exponential is the reference's polynomial exp2 (ops.ts:1650-1673).
-//
-// Mapping: grid (n_kv_heads, NSPLIT).  A block owns one kv head and one contiguous chunk of
-// positions, and serves all n_rep query heads of that kv head from a single read of K and V
-// (the GQA saving).  Inside the block a group of HD/EPL lanes covers one cache row with one 128-bit
-// load per lane.  Phase 1 writes the chunk's scores to LDS and finds the chunk maximum, phase 2
-// accumulates exp(s - m) and exp(s - m) * V.  Each block leaves (m, l, o) in the workspace; the last
-// block of a kv head to finish (agent-scope counter) merges the chunks and writes the output row.
-// The grid does not depend on T, so a captured graph replays unchanged while T grows.
-#include "common.h"
+// Stand-alone decode attention kernel: grid (n_kv_heads, NSPLIT), one work item per block (see attention_core.h).
+// NSPLIT is fixed from max_context, so the grid does not depend on T and a captured graph replays unchanged while T grows.
+#include "attention_core.h"
 
 namespace jsg {
 
 constexpr int ATT_THREADS = 256;
-constexpr int ATT_CHUNK_MAX = 256;  // positions per block held in LDS
-
-struct AttnArgs {
-  const void *q, *cache_k, *cache_v;
-  const int32_t *st;
-  void *out;
-  int *counters;   // [n_kv_heads], zero before the first launch; the merging block leaves them zero
-  float *partial;  // [n_kv_heads][nsplit][n_rep][HD + 2]
-  int n_kv_heads, nsplit, max_context;
-  float scale;     // float(1 / sqrt(head_dim)) (tensor.ts:3923 `.div(Math.sqrt(d))` = mul by the folded reciprocal)
-};
-
-template <int G> __device__ __forceinline__ float group_sum(float v) {
-  static_assert(G == 8 || G == 16 || G == 32, "lane group");
-  v += dpp_f<0xB1>(v);
-  v += dpp_f<0x4E>(v);
-  v += dpp_f<0x141>(v);
-  if (G >= 16) v += dpp_f<0x140>(v);
-  if (G == 32) v += __shfl_xor(v, 16);
-  return v;
-}
 
 template <typename AT, int HD, int NREP>
 __global__ __launch_bounds__(ATT_THREADS) void attn_decode_kernel(AttnArgs a) {
-  constexpr int EPL = 16 / sizeof(AT);  // elements per lane per 128-bit load
-  constexpr int G = HD / EPL;           // lanes per cache row
-  constexpr int RPI = 64 / G;           // rows per wavefront iteration
-  constexpr int NW = ATT_THREADS / 64;
+  typedef Attn<AT, HD, NREP, ATT_THREADS / 64, false> A;
+  __shared__ typename A::Smem sm;
   const int g = blockIdx.x, split = blockIdx.y;
   const int pos = a.st[1];
   if (pos < 0 || pos >= a.max_context) return;
@@ -52,186 +17,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_decode_kernel(AttnArgs a) {
   const int chunk = (T + a.nsplit - 1) / a.nsplit;  // <= ATT_CHUNK_MAX, checked on the host against max_context
   const int n_active = (T + chunk - 1) / chunk;
   if (split >= n_active) return;
-  const int t0 = split * chunk, t1 = min(T, t0 + chunk), CH = t1 - t0;
-
-  __shared__ float sc[NREP][ATT_CHUNK_MAX];
-  __shared__ float red[NREP][NW];
-  __shared__ float o_part[NW][NREP][HD];
-  __shared__ float m_sh[NREP], l_sh[NREP];
-  __shared__ int is_last;
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int sub = lane % G, grp = lane / G;
-  const size_t row_stride = (size_t)a.n_kv_heads * HD;
-  const AT *kbase = (const AT *)a.cache_k + (size_t)g * HD + (size_t)sub * EPL;
-  const AT *vbase = (const AT *)a.cache_v + (size_t)g * HD + (size_t)sub * EPL;
-
-  // this lane's slice of the n_rep query rows
-  float qf[NREP][EPL];
-#pragma unroll
-  for (int j = 0; j < NREP; j++) {
-    const AT *qp = (const AT *)a.q + (size_t)(g * NREP + j) * HD + sub * EPL;
-#pragma unroll
-    for (int e = 0; e < EPL; e++) qf[j][e] = (float)qp[e];
-  }
-
-  // ---- phase 1: scores of the chunk
-  for (int t = t0 + wave * RPI + grp; t < t1; t += NW * RPI) {
-    u4_t raw = *(const u4_t *)(kbase + (size_t)t * row_stride);
-    float kf[EPL];
-    if constexpr (sizeof(AT) == 2) {
-#pragma unroll
-      for (int e = 0; e < 4; e++) { h2_t h = as_h2(raw[e]); kf[2 * e] = (float)h[0]; kf[2 * e + 1] = (float)h[1]; }
-    } else {
-#pragma unroll
-      for (int e = 0; e < 4; e++) kf[e] = __uint_as_float(raw[e]);
-    }
-#pragma unroll
-    for (int j = 0; j < NREP; j++) {
-      float p = 0.0f;
-#pragma unroll
-      for (int e = 0; e < EPL; e++) p = fmaf(qf[j][e], kf[e], p);
-      p = group_sum<G>(p);
-      if (sub == 0) sc[j][t - t0] = __fmul_rn(p, a.scale);
-    }
-  }
-  __syncthreads();
-  // chunk maximum per head
-  {
-    float mx[NREP];
-#pragma unroll
-    for (int j = 0; j < NREP; j++) mx[j] = -INFINITY;
-    for (int i = tid; i < CH; i += ATT_THREADS)
-#pragma unroll
-      for (int j = 0; j < NREP; j++) mx[j] = fmaxf(mx[j], sc[j][i]);
-#pragma unroll
-    for (int j = 0; j < NREP; j++) {
-      float w = wave_max(mx[j]);
-      if (lane == 0) red[j][wave] = w;
-    }
-    __syncthreads();
-    if (tid < NREP) {
-      float w = red[tid][0];
-      for (int i = 1; i < NW; i++) w = fmaxf(w, red[tid][i]);
-      m_sh[tid] = w;
-    }
-    __syncthreads();
-  }
-  // scores -> exp(s - m) in place, and their sum
-  {
-    float ls[NREP];
-#pragma unroll
-    for (int j = 0; j < NREP; j++) ls[j] = 0.0f;
-    for (int i = tid; i < CH; i += ATT_THREADS)
-#pragma unroll
-      for (int j = 0; j < NREP; j++) {
-        float e = exp_f32(__fsub_rn(sc[j][i], m_sh[j]));
-        sc[j][i] = e;
-        ls[j] += e;
-      }
-#pragma unroll
-    for (int j = 0; j < NREP; j++) {
-      float w = wave_sum(ls[j]);
-      if (lane == 0) red[j][wave] = w;
-    }
-    __syncthreads();
-    if (tid < NREP) {
-      float w = 0.0f;
-      for (int i = 0; i < NW; i++) w += red[tid][i];
-      l_sh[tid] = w;
-    }
-    // the barrier below also orders the in-place exp writes before phase 2 reads them
-  }
-  __syncthreads();
-
-  // ---- phase 2: o[j][d] = sum_t p[j][t] * V[t][d]
-  float of[NREP][EPL];
-#pragma unroll
-  for (int j = 0; j < NREP; j++)
-#pragma unroll
-    for (int e = 0; e < EPL; e++) of[j][e] = 0.0f;
-  for (int t = t0 + wave * RPI + grp; t < t1; t += NW * RPI) {
-    u4_t raw = *(const u4_t *)(vbase + (size_t)t * row_stride);
-    float vf[EPL];
-    if constexpr (sizeof(AT) == 2) {
-#pragma unroll
-      for (int e = 0; e < 4; e++) { h2_t h = as_h2(raw[e]); vf[2 * e] = (float)h[0]; vf[2 * e + 1] = (float)h[1]; }
-    } else {
-#pragma unroll
-      for (int e = 0; e < 4; e++) vf[e] = __uint_as_float(raw[e]);
-    }
-#pragma unroll
-    for (int j = 0; j < NREP; j++) {
-      const float p = sc[j][t - t0];
-#pragma unroll
-      for (int e = 0; e < EPL; e++) of[j][e] = fmaf(p, vf[e], of[j][e]);
-    }
-  }
-  // lanes with the same `sub` hold different rows: fold the RPI groups of the wavefront together
-#pragma unroll
-  for (int j = 0; j < NREP; j++)
-#pragma unroll
-    for (int e = 0; e < EPL; e++) {
-      float v = of[j][e];
-#pragma unroll
-      for (int off = G; off < 64; off <<= 1) v += __shfl_xor(v, off);
-      of[j][e] = v;
-    }
-  if (grp == 0) {
-#pragma unroll
-    for (int j = 0; j < NREP; j++)
-#pragma unroll
-      for (int e = 0; e < EPL; e++) o_part[wave][j][sub * EPL + e] = of[j][e];
-  }
-  __syncthreads();
-  float *mine = a.partial + ((size_t)g * a.nsplit + split) * NREP * (HD + 2);
-  for (int i = tid; i < NREP * HD; i += ATT_THREADS) {
-    const int j = i / HD, d = i % HD;
-    float v = 0.0f;
-#pragma unroll
-    for (int w = 0; w < NW; w++) v += o_part[w][j][d];
-    st_coherent(&mine[j * (HD + 2) + d], v);
-  }
-  if (tid < NREP) {
-    st_coherent(&mine[tid * (HD + 2) + HD], m_sh[tid]);
-    st_coherent(&mine[tid * (HD + 2) + HD + 1], l_sh[tid]);
-  }
-
-  // ---- publish, and let the last chunk of this kv head merge
-  __syncthreads();  // every coherent store of the block has been acknowledged
-  if (tid == 0) {
-    int old = __hip_atomic_fetch_add(&a.counters[g], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    is_last = (old == n_active - 1);
-  }
-  __syncthreads();
-  if (!is_last) return;
-  // merge: one wavefront per query head turns the per-chunk (m, l) into weights exp(m_s - M) and 1/L ...
-  const float *base = a.partial + (size_t)g * a.nsplit * NREP * (HD + 2);
-  for (int j = wave; j < NREP; j += NW) {
-    float M = -INFINITY;
-    for (int s = lane; s < n_active; s += 64) M = fmaxf(M, ld_coherent(base + ((size_t)s * NREP + j) * (HD + 2) + HD));
-    M = wave_max(M);
-    float L = 0.0f;
-    for (int s = lane; s < n_active; s += 64) {
-      const float *ps = base + ((size_t)s * NREP + j) * (HD + 2);
-      const float w = exp_f32(ld_coherent(ps + HD) - M);
-      sc[j][s] = w;  // n_active <= nsplit <= ATT_CHUNK_MAX
-      L = fmaf(ld_coherent(ps + HD + 1), w, L);
-    }
-    L = wave_sum(L);
-    if (lane == 0) l_sh[j] = 1.0f / L;  // softmax normalisation is e * (1/sum) (tensor.ts:2211-2214)
-  }
-  __syncthreads();
-  // ... then every thread sums its output elements over the chunks; the loads are independent, so they pipeline
-  for (int i = tid; i < NREP * HD; i += ATT_THREADS) {
-    const int j = i / HD, d = i % HD;
-    const float *po = base + (size_t)j * (HD + 2) + d;
-    float O = 0.0f;
-#pragma unroll 8
-    for (int s = 0; s < n_active; s++) O = fmaf(ld_coherent(po + (size_t)s * NREP * (HD + 2)), sc[j][s], O);
-    ((AT *)a.out)[(size_t)(g * NREP + j) * HD + d] = (AT)Act<AT>::rn(O * l_sh[j]);  // the cast of the P.V result
-  }
-  if (tid == 0) __hip_atomic_store(&a.counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  A::item(a, sm, g, split, T, chunk, n_active);
 }
 
 // splits: enough that a chunk fits the LDS score buffer, and no more than the merge can index there

@@ -1,0 +1,245 @@
+// Device code of decode-time grouped-query attention over the HBM-resident KV cache for gfx950, shared by the
+// stand-alone kernel (attention.hip) and the whole-step kernel (decode_step.hip).
+//
+// One new query position against cache rows [0, T), T = start_pos + 1: repeat_kv + scaled_dot_product_attention of the
+// reference (/root/reference/jsgrad/models/llama.ts:89-95, /root/reference/jsgrad/tensor.ts:3920-3934).  Scores, the
+// softmax and the P.V sum are float32; the exponential is the reference's polynomial exp2 (ops.ts:1650-1673).
+//
+// A work item is (kv head g, chunk `split` of the positions).  The block that runs it serves all n_rep query heads of
+// the kv head from a single read of K and V (the GQA saving): a group of HD/EPL lanes covers one cache row with one
+// 128-bit load per lane.  Phase 1 writes the chunk's scores to LDS and finds the chunk maximum, phase 2 accumulates
+// exp(s - m) and exp(s - m) * V.  The item leaves (m, l, o) in the workspace; the last item of a kv head to finish
+// (agent-scope counter) merges the chunks and writes the output rows.
+#pragma once
+#include "common.h"
+
+namespace jsg {
+
+constexpr int ATT_CHUNK_MAX = 256;  // positions per item held in LDS; also the most chunks the merge can index
+
+struct AttnArgs {
+  const void *q, *cache_k, *cache_v;
+  const int32_t *st;
+  void *out;
+  int *counters;   // [n_kv_heads], zero before the first launch; the merging block leaves them zero
+  float *partial;  // [n_kv_heads][nsplit][n_rep][HD + 2]
+  int n_kv_heads, nsplit, max_context;
+  float scale;     // float(1 / sqrt(head_dim)) (tensor.ts:3923 `.div(Math.sqrt(d))` = mul by the folded reciprocal)
+};
+
+template <int G> __device__ __forceinline__ float group_sum(float v) {
+  static_assert(G == 8 || G == 16 || G == 32, "lane group");
+  v += dpp_f<0xB1>(v);
+  v += dpp_f<0x4E>(v);
+  v += dpp_f<0x141>(v);
+  if (G >= 16) v += dpp_f<0x140>(v);
+  if (G == 32) v += __shfl_xor(v, 16);
+  return v;
+}
+
+// NW wavefronts per block.  COHERENT: q and the output cross between blocks of the same launch.
+template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
+  static constexpr int EPL = 16 / sizeof(AT);  // elements per lane per 128-bit load
+  static constexpr int G = HD / EPL;           // lanes per cache row
+  static constexpr int RPI = 64 / G;           // rows per wavefront iteration
+  struct Smem {
+    float sc[NREP][ATT_CHUNK_MAX];
+    float red[NREP][NW];
+    float o_part[NW < 4 ? NW : 4][NREP][HD];   // wavefronts fold into four slots, then the slots are summed
+    float m_sh[NREP], l_sh[NREP];
+    int is_last;
+  };
+
+  // T visible positions cut into chunks of `chunk` rows (n_active of them); this call handles chunk `split` of kv head g.
+  // Must be called by every thread of the block (it contains barriers).
+  __device__ static void item(const AttnArgs &a, Smem &sm, int g, int split, int T, int chunk, int n_active) {
+    const int t0 = split * chunk, t1 = min(T, t0 + chunk), CH = t1 - t0;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = NW * 64;
+    const int sub = lane % G, grp = lane / G;
+    const size_t row_stride = (size_t)a.n_kv_heads * HD;
+    const AT *kbase = (const AT *)a.cache_k + (size_t)g * HD + (size_t)sub * EPL;
+    const AT *vbase = (const AT *)a.cache_v + (size_t)g * HD + (size_t)sub * EPL;
+
+    // this lane's slice of the n_rep query rows
+    float qf[NREP][EPL];
+#pragma unroll
+    for (int j = 0; j < NREP; j++) {
+      const AT *qp = (const AT *)a.q + (size_t)(g * NREP + j) * HD + sub * EPL;
+#pragma unroll
+      for (int e = 0; e < EPL; e++) {
+        if constexpr (COHERENT) qf[j][e] = (float)ld_coherent(qp + e);
+        else qf[j][e] = (float)qp[e];
+      }
+    }
+
+    // ---- phase 1: scores of the chunk
+    for (int t = t0 + wave * RPI + grp; t < t1; t += NW * RPI) {
+      u4_t raw = *(const u4_t *)(kbase + (size_t)t * row_stride);
+      float kf[EPL];
+      if constexpr (sizeof(AT) == 2) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) { h2_t h = as_h2(raw[e]); kf[2 * e] = (float)h[0]; kf[2 * e + 1] = (float)h[1]; }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) kf[e] = __uint_as_float(raw[e]);
+      }
+#pragma unroll
+      for (int j = 0; j < NREP; j++) {
+        float p = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPL; e++) p = fmaf(qf[j][e], kf[e], p);
+        p = group_sum<G>(p);
+        if (sub == 0) sm.sc[j][t - t0] = p * a.scale;
+      }
+    }
+    __syncthreads();
+    // chunk maximum per head
+    {
+      float mx[NREP];
+#pragma unroll
+      for (int j = 0; j < NREP; j++) mx[j] = -INFINITY;
+      for (int i = tid; i < CH; i += nthreads)
+#pragma unroll
+        for (int j = 0; j < NREP; j++) mx[j] = fmaxf(mx[j], sm.sc[j][i]);
+#pragma unroll
+      for (int j = 0; j < NREP; j++) {
+        float w = wave_max(mx[j]);
+        if (lane == 0) sm.red[j][wave] = w;
+      }
+      __syncthreads();
+      if (tid < NREP) {
+        float w = sm.red[tid][0];
+        for (int i = 1; i < NW; i++) w = fmaxf(w, sm.red[tid][i]);
+        sm.m_sh[tid] = w;
+      }
+      __syncthreads();
+    }
+    // scores -> exp(s - m) in place, and their sum
+    {
+      float ls[NREP];
+#pragma unroll
+      for (int j = 0; j < NREP; j++) ls[j] = 0.0f;
+      for (int i = tid; i < CH; i += nthreads)
+#pragma unroll
+        for (int j = 0; j < NREP; j++) {
+          float e = exp_f32(sm.sc[j][i] - sm.m_sh[j]);
+          sm.sc[j][i] = e;
+          ls[j] += e;
+        }
+#pragma unroll
+      for (int j = 0; j < NREP; j++) {
+        float w = wave_sum(ls[j]);
+        if (lane == 0) sm.red[j][wave] = w;
+      }
+      __syncthreads();
+      if (tid < NREP) {
+        float w = 0.0f;
+        for (int i = 0; i < NW; i++) w += sm.red[tid][i];
+        sm.l_sh[tid] = w;
+      }
+      // the barrier below also orders the in-place exp writes before phase 2 reads them
+    }
+    __syncthreads();
+
+    // ---- phase 2: o[j][d] = sum_t p[j][t] * V[t][d]
+    float of[NREP][EPL];
+#pragma unroll
+    for (int j = 0; j < NREP; j++)
+#pragma unroll
+      for (int e = 0; e < EPL; e++) of[j][e] = 0.0f;
+    for (int t = t0 + wave * RPI + grp; t < t1; t += NW * RPI) {
+      u4_t raw = *(const u4_t *)(vbase + (size_t)t * row_stride);
+      float vf[EPL];
+      if constexpr (sizeof(AT) == 2) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) { h2_t h = as_h2(raw[e]); vf[2 * e] = (float)h[0]; vf[2 * e + 1] = (float)h[1]; }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) vf[e] = __uint_as_float(raw[e]);
+      }
+#pragma unroll
+      for (int j = 0; j < NREP; j++) {
+        const float p = sm.sc[j][t - t0];
+#pragma unroll
+        for (int e = 0; e < EPL; e++) of[j][e] = fmaf(p, vf[e], of[j][e]);
+      }
+    }
+    // lanes with the same `sub` hold different rows: fold the RPI groups of the wavefront together
+#pragma unroll
+    for (int j = 0; j < NREP; j++)
+#pragma unroll
+      for (int e = 0; e < EPL; e++) {
+        float v = of[j][e];
+#pragma unroll
+        for (int off = G; off < 64; off <<= 1) v += __shfl_xor(v, off);
+        of[j][e] = v;
+      }
+    // wavefronts fold into (at most) four LDS slots, four at a time
+    constexpr int SLOTS = NW < 4 ? NW : 4;
+    for (int round = 0; round < NW / SLOTS; round++) {
+      if (grp == 0 && wave / SLOTS == round) {
+#pragma unroll
+        for (int j = 0; j < NREP; j++)
+#pragma unroll
+          for (int e = 0; e < EPL; e++) {
+            float *slot = &sm.o_part[wave % SLOTS][j][sub * EPL + e];
+            *slot = round == 0 ? of[j][e] : *slot + of[j][e];
+          }
+      }
+      __syncthreads();
+    }
+    float *mine = a.partial + ((size_t)g * a.nsplit + split) * NREP * (HD + 2);
+    for (int i = tid; i < NREP * HD; i += nthreads) {
+      const int j = i / HD, d = i % HD;
+      float v = 0.0f;
+#pragma unroll
+      for (int w = 0; w < SLOTS; w++) v += sm.o_part[w][j][d];
+      st_coherent(&mine[j * (HD + 2) + d], v);
+    }
+    if (tid < NREP) {
+      st_coherent(&mine[tid * (HD + 2) + HD], sm.m_sh[tid]);
+      st_coherent(&mine[tid * (HD + 2) + HD + 1], sm.l_sh[tid]);
+    }
+
+    // ---- publish, and let the last chunk of this kv head merge
+    __syncthreads();  // every coherent store of the block has been acknowledged
+    if (tid == 0) {
+      int old = __hip_atomic_fetch_add(&a.counters[g], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      sm.is_last = (old == n_active - 1);
+    }
+    __syncthreads();
+    if (!sm.is_last) return;
+    // merge: one wavefront per query head turns the per-chunk (m, l) into weights exp(m_s - M) and 1/L ...
+    const float *base = a.partial + (size_t)g * a.nsplit * NREP * (HD + 2);
+    for (int j = wave; j < NREP; j += NW) {
+      float M = -INFINITY;
+      for (int s = lane; s < n_active; s += 64) M = fmaxf(M, ld_coherent(base + ((size_t)s * NREP + j) * (HD + 2) + HD));
+      M = wave_max(M);
+      float L = 0.0f;
+      for (int s = lane; s < n_active; s += 64) {
+        const float *ps = base + ((size_t)s * NREP + j) * (HD + 2);
+        const float w = exp_f32(ld_coherent(ps + HD) - M);
+        sm.sc[j][s] = w;  // n_active <= nsplit <= ATT_CHUNK_MAX
+        L = fmaf(ld_coherent(ps + HD + 1), w, L);
+      }
+      L = wave_sum(L);
+      if (lane == 0) sm.l_sh[j] = 1.0f / L;  // softmax normalisation is e * (1/sum) (tensor.ts:2211-2214)
+    }
+    __syncthreads();
+    // ... then every thread sums its output elements over the chunks; the loads are independent, so they pipeline
+    for (int i = tid; i < NREP * HD; i += nthreads) {
+      const int j = i / HD, d = i % HD;
+      const float *po = base + (size_t)j * (HD + 2) + d;
+      float O = 0.0f;
+#pragma unroll 8
+      for (int s = 0; s < n_active; s++) O = fmaf(ld_coherent(po + (size_t)s * NREP * (HD + 2)), sm.sc[j][s], O);
+      AT *dst = (AT *)a.out + (size_t)(g * NREP + j) * HD + d;
+      const float r = Act<AT>::rn(O * sm.l_sh[j]);  // the cast of the P.V result
+      if constexpr (COHERENT) st_coherent(dst, (AT)r);
+      else *dst = (AT)r;
+    }
+    if (tid == 0) __hip_atomic_store(&a.counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+};
+
+}  // namespace jsg

@@ -23,7 +23,7 @@ int fail(const char *fmt, ...);
 int fail_hip(hipError_t e, const char *what);
 
 // per-kernel timing with HIP events on the library stream (off unless jsgrad_hip_profile(1))
-enum { PROF_EMBED = 0, PROF_RMSNORM, PROF_LINEAR, PROF_QKV_ROPE, PROF_ATTN, PROF_FFN_GATE, PROF_ARGMAX, PROF_KINDS };
+enum { PROF_EMBED = 0, PROF_RMSNORM, PROF_LINEAR, PROF_QKV_ROPE, PROF_ATTN, PROF_FFN_GATE, PROF_ARGMAX, PROF_STEP, PROF_KINDS };
 // Event pair for the next launch of `kind`, or false when profiling is off (or capturing, or out of slots).  The pair
 // is handed to hipExtLaunchKernelGGL, which stamps it with the dispatch's own begin/end times, so the elapsed time is
 // the kernel alone: no marker packets, no launch latency.
@@ -93,6 +93,12 @@ template <> struct Act<_Float16> {
 // fence would write back and invalidate the whole L2 of the XCD once per block, which costs far more than the kernel.
 __device__ __forceinline__ void st_coherent(float *p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void st_coherent(int *p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void st_coherent(_Float16 *p, _Float16 v) {
+  __hip_atomic_store((uint16_t *)p, __builtin_bit_cast(uint16_t, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ _Float16 ld_coherent(const _Float16 *p) {
+  return __builtin_bit_cast(_Float16, __hip_atomic_load((const uint16_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
 __device__ __forceinline__ float ld_coherent(const float *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ int ld_coherent(const int *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 

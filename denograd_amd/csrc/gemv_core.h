@@ -1,0 +1,437 @@
+// Device code of the one-row linear layers (GEMV) with in-register dequantisation for gfx950, shared by the
+// stand-alone kernels (gemv.hip) and the whole-step kernel (decode_step.hip).
+//
+// y[out] = x[in] . W^T for W stored as float32, float16, int8 (+ fp16 scale per output row) or NF4 (+ fp16 scale per
+// 64 elements): Linear.call / Int8Linear.call / NF4Linear.call of the reference
+// (/root/reference/jsgrad/nn/index.ts:411, /root/reference/jsgrad/models/llama3.ts:35,91-97) at batch 1, where the whole
+// cost is streaming W once from HBM.  Fused around it: RMSNorm of the input (nn/index.ts:586-588), and as epilogues a
+// plain store (+ residual), the rotary embedding with the KV-cache write (models/llama.ts:61-87), SwiGLU (llama.ts:108-110).
+#pragma once
+#include "common.h"
+
+namespace jsg {
+
+enum { EPI_STORE = 0, EPI_ROPE_KV = 1, EPI_SWIGLU = 2 };
+
+struct GemvArgs {
+  const void *w0, *w1, *w2;  // up to three matrices sharing the input row: (wq, wk, wv) or (w1, w3).  Separate fields,
+                             // not arrays: a run-time index into the argument struct would force it into scratch memory
+  const void *s0, *s1, *s2;  // their scales (int8: per row, nf4: per 64 elements)
+  int rows0, rows1, rows2;   // rows of each matrix (0 = unused)
+  int in_f;
+  const void *x;          // input row, activation dtype
+  const void *norm_w;     // RMSNorm weight or nullptr
+  float eps;
+  float inv_d;            // float(1/in_f), the constant the mean is multiplied with (tensor.ts:2113-2117)
+  void *y;                // EPI_STORE: y[rows0]; EPI_SWIGLU: g[rows0]; EPI_ROPE_KV: q_out[rows0]
+  const void *residual;   // EPI_STORE only, may be nullptr
+  const void *rope_table; // [2*max_context][hd/2][2], activation dtype
+  const int32_t *st;      // device {token, start_pos}
+  void *cache_k, *cache_v;
+  int head_dim, max_context;
+};
+
+// ---- weight formats: VEC elements per 16-byte load --------------------------------------------
+template <int KIND> struct WFmt;
+template <> struct WFmt<JSGRAD_W_F32> { static constexpr int VEC = 4; };
+template <> struct WFmt<JSGRAD_W_F16> { static constexpr int VEC = 8; };
+template <> struct WFmt<JSGRAD_W_I8> { static constexpr int VEC = 16; };
+template <> struct WFmt<JSGRAD_W_NF4> { static constexpr int VEC = 32; };
+
+// NF4 code book (llama3.ts:80-81); the CODE tensor is float16, so every literal is rounded to fp16 first
+#define JSG_C16(x) ((float)(_Float16)(x))
+static __device__ __constant__ float NF4_CODE[16] = {JSG_C16(-1.0f), JSG_C16(-0.6961928009986877f), JSG_C16(-0.5250730514526367f), JSG_C16(-0.39491748809814453f),
+                                              JSG_C16(-0.28444138169288635f), JSG_C16(-0.18477343022823334f), JSG_C16(-0.09105003625154495f), JSG_C16(0.0f),
+                                              JSG_C16(0.07958029955625534f), JSG_C16(0.16093020141124725f), JSG_C16(0.24611230194568634f), JSG_C16(0.33791524171829224f),
+                                              JSG_C16(0.44070982933044434f), JSG_C16(0.5626170039176941f), JSG_C16(0.7229568362236023f), JSG_C16(1.0f)};
+
+// x fragment of one lane for one step: VEC activations
+template <typename AT, int VEC> struct XFrag;
+template <int VEC> struct XFrag<_Float16, VEC> {
+  h2_t v[VEC / 2];
+  __device__ __forceinline__ void load(const _Float16 *xs) {
+    const u4_t *p = (const u4_t *)xs;
+#pragma unroll
+    for (int i = 0; i < VEC / 8; i++) {
+      u4_t t = p[i];
+#pragma unroll
+      for (int j = 0; j < 4; j++) v[i * 4 + j] = as_h2(t[j]);
+    }
+  }
+  __device__ __forceinline__ float get(int i) const { return (float)v[i >> 1][i & 1]; }
+};
+template <int VEC> struct XFrag<float, VEC> {
+  float v[VEC];
+  __device__ __forceinline__ void load(const float *xs) {
+    const f4_t *p = (const f4_t *)xs;
+#pragma unroll
+    for (int i = 0; i < VEC / 4; i++) {
+      f4_t t = p[i];
+#pragma unroll
+      for (int j = 0; j < 4; j++) v[i * 4 + j] = t[j];
+    }
+  }
+  __device__ __forceinline__ float get(int i) const { return v[i]; }
+};
+
+// dot of one 16-byte weight vector with the lane's x fragment, accumulated into acc
+template <int KIND, typename AT> struct Dot {
+  static constexpr int VEC = WFmt<KIND>::VEC;
+  // generic float path
+  __device__ static __forceinline__ float run(u4_t wv, const XFrag<AT, VEC> &xf, float acc, float blk_scale, const float *lut) {
+    if constexpr (KIND == JSGRAD_W_F32) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) acc = fmaf(xf.get(i), __uint_as_float(wv[i]), acc);
+    } else if constexpr (KIND == JSGRAD_W_F16) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        h2_t w2 = as_h2(wv[i]);
+        acc = fmaf(xf.get(2 * i), (float)w2[0], acc);
+        acc = fmaf(xf.get(2 * i + 1), (float)w2[1], acc);
+      }
+    } else if constexpr (KIND == JSGRAD_W_I8) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        int d = (int)wv[i];
+        acc = fmaf(xf.get(4 * i + 0), (float)((d << 24) >> 24), acc);
+        acc = fmaf(xf.get(4 * i + 1), (float)((d << 16) >> 24), acc);
+        acc = fmaf(xf.get(4 * i + 2), (float)((d << 8) >> 24), acc);
+        acc = fmaf(xf.get(4 * i + 3), (float)(d >> 24), acc);
+      }
+    } else {
+      // 32 codes; element 2j is the high nibble of byte j (llama3.ts:92-94,105). One scale per lane-step
+      // because 32 | 64 and k is a multiple of 32.  Each term is x * (code * scale) as the reference forms it:
+      // the inner product is exact in float (11 x 11 significant bits).
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        uint32_t d = wv[i];
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+          uint32_t byte = (d >> (8 * b)) & 0xffu;
+          acc = fmaf(xf.get(8 * i + 2 * b), lut[byte >> 4] * blk_scale, acc);
+          acc = fmaf(xf.get(8 * i + 2 * b + 1), lut[byte & 15u] * blk_scale, acc);
+        }
+      }
+    }
+    return acc;
+  }
+};
+// fp16 activations x fp16 weights: packed dot with float accumulation
+template <> struct Dot<JSGRAD_W_F16, _Float16> {
+  static constexpr int VEC = 8;
+  __device__ static __forceinline__ float run(u4_t wv, const XFrag<_Float16, 8> &xf, float acc, float, const float *) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) acc = __builtin_amdgcn_fdot2(as_h2(wv[i]), xf.v[i], acc, false);
+    return acc;
+  }
+};
+// fp16 activations x int8 weights: bytes -> exact fp16 integers through the 0x6400 exponent trick
+// (0x6400 | u is the half 1024 + u for u in 0..255), then the packed dot
+template <> struct Dot<JSGRAD_W_I8, _Float16> {
+  static constexpr int VEC = 16;
+  __device__ static __forceinline__ float run(u4_t wv, const XFrag<_Float16, 16> &xf, float acc, float, const float *) {
+    const h2_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};  // 1024 + 128
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      uint32_t u = wv[i] ^ 0x80808080u;  // signed byte w -> unsigned w + 128
+      h2_t lo = as_h2(__builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias;
+      h2_t hi = as_h2(__builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias;
+      acc = __builtin_amdgcn_fdot2(lo, xf.v[2 * i], acc, false);
+      acc = __builtin_amdgcn_fdot2(hi, xf.v[2 * i + 1], acc, false);
+    }
+    return acc;
+  }
+};
+
+// Stage x (optionally RMSNorm'ed) into LDS in the activation dtype.  Every thread moves 16-byte chunks; with a
+// norm the chunks stay in registers between the sum of squares and the scaling, so x is read from memory once and
+// the whole prologue costs one round of loads and two barriers.  Ends with a barrier.
+// COHERENT: x was written by other blocks of the same launch, so it is read at the device-wide coherence point.
+template <typename AT, bool COHERENT> __device__ __forceinline__ void stage_x(const GemvArgs &a, AT *xs, float *red) {
+  constexpr int EPC = 16 / sizeof(AT);  // elements per 16-byte chunk
+  constexpr int MAXCH = 4;              // chunks a thread keeps in registers on the norm path (host checks the size)
+  const int n = a.in_f, tid = threadIdx.x, nt = blockDim.x;
+  const int nchunks = n / EPC;          // in_f is a multiple of EPC (checked on the host)
+  const u4_t *xg = (const u4_t *)a.x;
+  u4_t *xl = (u4_t *)xs;
+  auto ldx = [&](int c) -> u4_t {
+    if constexpr (COHERENT) {
+      const uint32_t *p = (const uint32_t *)(xg + c);
+      u4_t v;
+#pragma unroll
+      for (int e = 0; e < 4; e++) v[e] = __hip_atomic_load(p + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return v;
+    } else {
+      return xg[c];
+    }
+  };
+  if (a.norm_w == nullptr) {
+    for (int c = tid; c < nchunks; c += nt) xl[c] = ldx(c);
+    __syncthreads();
+    return;
+  }
+  const u4_t *wg = (const u4_t *)a.norm_w;
+  u4_t xr[MAXCH], wr[MAXCH];
+  float ss = 0.0f;
+#pragma unroll
+  for (int i = 0; i < MAXCH; i++) {
+    const int c = tid + i * nt;
+    if (c < nchunks) { xr[i] = ldx(c); wr[i] = wg[c]; }
+  }
+#pragma unroll
+  for (int i = 0; i < MAXCH; i++) {
+    const int c = tid + i * nt;
+    if (c < nchunks) {
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        if constexpr (sizeof(AT) == 2) {
+          h2_t h = as_h2(xr[i][e]);
+          ss = fmaf((float)h[0], (float)h[0], ss);
+          ss = fmaf((float)h[1], (float)h[1], ss);
+        } else {
+          float f = __uint_as_float(xr[i][e]);
+          ss = fmaf(f, f, ss);
+        }
+      }
+    }
+  }
+  ss = wave_sum(ss);
+  const int wave = tid >> 6, nw = nt >> 6;
+  if ((tid & 63) == 0) red[wave] = ss;
+  __syncthreads();
+  float tot = 0.0f;
+  for (int i = 0; i < nw; i++) tot += red[i];
+  // sqrt(1 / (mean + eps)), mean = sum * float(1/d)  (nn/index.ts:586, tensor.ts:2944-2946)
+  const float r = __fsqrt_rn(__fdiv_rn(1.0f, __fadd_rn(__fmul_rn(tot, a.inv_d), a.eps)));
+#pragma unroll
+  for (int i = 0; i < MAXCH; i++) {
+    const int c = tid + i * nt;
+    if (c < nchunks) {
+      u4_t o;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        if constexpr (sizeof(AT) == 2) {
+          h2_t h = as_h2(xr[i][e]), w = as_h2(wr[i][e]), y;
+          // .cast(x.dtype) before the weight multiply (nn/index.ts:588)
+          y[0] = (_Float16)((float)(_Float16)((float)h[0] * r) * (float)w[0]);
+          y[1] = (_Float16)((float)(_Float16)((float)h[1] * r) * (float)w[1]);
+          o[e] = __builtin_bit_cast(uint32_t, y);
+        } else {
+          o[e] = __float_as_uint((__uint_as_float(xr[i][e]) * r) * __uint_as_float(wr[i][e]));
+        }
+      }
+      xl[c] = o;
+    }
+  }
+  __syncthreads();
+}
+
+// One item's registers: the weight vectors plus, on the item that finishes a row group, the operands its epilogue will
+// need (row scales, residual, rotary pair), fetched with the weights so that no load latency is left at the end.
+// Every configuration in use moves 8 x 16 bytes per lane and item (UNROLL x NM x ROWS = 8) and has ROWS = 2, so one
+// plain struct serves all of them; the whole-step kernel can then carry ONE prefetched buffer from phase to phase.
+struct GemvBuf {
+  u4_t w[8];       // [u][j][r] flattened
+  float scale[4];  // [j][r] flattened
+  float extra[2];  // EPI_STORE: residual[row]; EPI_ROPE_KV: (cos, sin) of the rotary pair
+};
+
+// The GEMV of one launch (or of one phase of the whole-step kernel).  A block stages x once, then its wavefronts walk
+// row groups (ROWS consecutive output rows of the NM matrices that share x) grid-stride.  A wavefront's work is the flat
+// sequence of (row group, k-batch) items; the loads of item i+1 go into a second register buffer before item i is
+// consumed, and the first item is requested before x is staged (or, with `preloaded`, before the caller even waited
+// for the previous phase), so a wavefront always has a batch of 128-bit loads in flight.
+// COHERENT: x, residual and outputs cross between blocks of the same launch.
+template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> struct Gemv {
+  static constexpr int VEC = WFmt<KIND>::VEC;
+  static constexpr int BITS = KIND == JSGRAD_W_F32 ? 32 : KIND == JSGRAD_W_F16 ? 16 : KIND == JSGRAD_W_I8 ? 8 : 4;
+  static constexpr int STEP = 64 * VEC;                 // elements one wavefront covers per k-step
+  static constexpr int NM = EPI == EPI_SWIGLU ? 2 : 1;  // matrices a wavefront evaluates on the same rows
+  typedef GemvBuf Buf;
+  static_assert(ROWS == 2 && UNROLL * NM * ROWS == 8, "GemvBuf holds 8 vectors for 2 rows");
+  __device__ static __forceinline__ constexpr int wi(int u, int j, int r) { return (u * NM + j) * ROWS + r; }
+  __device__ static __forceinline__ constexpr int si(int j, int r) { return j * ROWS + r; }
+
+  struct Where { int m, r0, mrows; };
+  // rows of a group: matrix m (EPI_ROPE_KV stacks wq, wk, wv; boundaries are multiples of ROWS), first row r0
+  __device__ static __forceinline__ Where locate(const GemvArgs &a, int grp) {
+    Where w = {0, grp * ROWS, 0};
+    if (EPI == EPI_ROPE_KV) {
+      if (w.r0 >= a.rows0) { w.r0 -= a.rows0; w.m = 1; }
+      if (w.m == 1 && w.r0 >= a.rows1) { w.r0 -= a.rows1; w.m = 2; }
+    }
+    w.mrows = a.rows0 * (w.m == 0) + a.rows1 * (w.m == 1) + a.rows2 * (w.m == 2);
+    return w;
+  }
+  // Pick one of three pointers by a run-time index with arithmetic, not `?:` or an array: the optimiser turns a
+  // select of loads from the argument struct into a load from a selected address, which forces the whole struct
+  // into scratch memory.
+  __device__ static __forceinline__ const void *pick(const void *p0, const void *p1, const void *p2, int m) {
+    return (const void *)((uintptr_t)p0 * (uintptr_t)(m == 0) + (uintptr_t)p1 * (uintptr_t)(m == 1) + (uintptr_t)p2 * (uintptr_t)(m == 2));
+  }
+  __device__ static __forceinline__ const void *wbase(const GemvArgs &a, int m, int j) { return NM == 2 ? pick(a.w0, a.w1, a.w2, j) : pick(a.w0, a.w1, a.w2, m); }
+  __device__ static __forceinline__ const void *sbase(const GemvArgs &a, int m, int j) { return NM == 2 ? pick(a.s0, a.s1, a.s2, j) : pick(a.s0, a.s1, a.s2, m); }
+  __device__ static __forceinline__ int ngroups(const GemvArgs &a) {
+    return ((EPI == EPI_SWIGLU ? a.rows0 : a.rows0 + a.rows1 + a.rows2) + ROWS - 1) / ROWS;
+  }
+  __device__ static __forceinline__ int nbatch(const GemvArgs &a) { return ((a.in_f + STEP - 1) / STEP + UNROLL - 1) / UNROLL; }
+
+  // issue the loads of item (grp, b)
+  __device__ static __forceinline__ void load_item(const GemvArgs &a, Buf &buf, int grp, int b, int pos) {
+    const int lane = threadIdx.x & 63, in_f = a.in_f;
+    const Where w = locate(a, grp);
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+      const int k = (b * UNROLL + u) * STEP + lane * VEC;
+      if (k < in_f) {
+#pragma unroll
+        for (int j = 0; j < NM; j++)
+#pragma unroll
+          for (int r = 0; r < ROWS; r++) {
+            const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;  // tail rows reload the last row, never stored
+            const char *p = (const char *)wbase(a, w.m, j) + (((size_t)row * in_f + (size_t)k) * BITS) / 8;
+            buf.w[wi(u, j, r)] = __builtin_nontemporal_load((const u4_t *)p);
+          }
+      }
+    }
+    if (b != nbatch(a) - 1) return;
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+      const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;
+      if constexpr (KIND == JSGRAD_W_I8) {
+#pragma unroll
+        for (int j = 0; j < NM; j++) buf.scale[si(j, r)] = (float)((const _Float16 *)sbase(a, w.m, j))[row];
+      }
+      if constexpr (EPI == EPI_STORE) {
+        const AT *res = (const AT *)a.residual;
+        if (res == nullptr) buf.extra[r] = 0.0f;
+        else if constexpr (COHERENT) buf.extra[r] = (float)ld_coherent(res + row);
+        else buf.extra[r] = (float)res[row];
+      } else if constexpr (EPI == EPI_ROPE_KV) {
+        // table row `pos`, entry (cos, sin) of pair i = (row % head_dim) / 2: even r gets cos, odd r gets sin
+        const bool ok = pos >= 0 && pos < a.max_context;
+        const int i = (row % a.head_dim) >> 1;
+        buf.extra[r] = ok ? (float)((const AT *)a.rope_table)[(size_t)pos * a.head_dim + 2 * i + (r & 1)] : 0.0f;
+      }
+    }
+  }
+
+  // the first item of this wavefront, requested ahead of run()
+  __device__ static __forceinline__ void prefetch(const GemvArgs &a, Buf &buf, int pos) {
+    const int grp = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (grp < ngroups(a)) load_item(a, buf, grp, 0, pos);
+  }
+
+  __device__ static __forceinline__ void store_out(AT *p, float v) {
+    if constexpr (COHERENT) st_coherent(p, (AT)v);
+    else *p = (AT)v;
+  }
+
+  // consume item (grp, b) from buf; on the last batch of the group: cross-lane sum, scale, cast, epilogue
+  __device__ static __forceinline__ void use_item(const GemvArgs &a, const Buf &buf, int grp, int b, float (&acc)[NM][ROWS], const AT *xs, const float *lut, int pos) {
+    const int lane = threadIdx.x & 63, in_f = a.in_f;
+    const Where w = locate(a, grp);
+    if (b == 0) {
+#pragma unroll
+      for (int j = 0; j < NM; j++)
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) acc[j][r] = 0.0f;
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+      const int k = (b * UNROLL + u) * STEP + lane * VEC;
+      if (k < in_f) {
+        XFrag<AT, VEC> xf;
+        xf.load(xs + k);
+#pragma unroll
+        for (int j = 0; j < NM; j++)
+#pragma unroll
+          for (int r = 0; r < ROWS; r++) {
+            float bs = 1.0f;
+            if constexpr (KIND == JSGRAD_W_NF4) {
+              const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;
+              bs = (float)((const _Float16 *)sbase(a, w.m, j))[((size_t)row * in_f + k) >> 6];
+            }
+            acc[j][r] = Dot<KIND, AT>::run(buf.w[wi(u, j, r)], xf, acc[j][r], bs, lut);
+          }
+      }
+    }
+    if (b != nbatch(a) - 1) return;
+
+    float val[NM][ROWS];
+#pragma unroll
+    for (int j = 0; j < NM; j++)
+#pragma unroll
+      for (int r = 0; r < ROWS; r++) {
+        float v = wave_sum(acc[j][r]);
+        if constexpr (KIND == JSGRAD_W_I8) v = v * buf.scale[si(j, r)];
+        val[j][r] = Act<AT>::rn(v);
+      }
+    const int r0 = w.r0, mrows = w.mrows;
+    if constexpr (EPI == EPI_STORE) {
+      AT *y = (AT *)a.y;
+      const bool has_res = a.residual != nullptr;
+#pragma unroll
+      for (int r = 0; r < ROWS; r++)
+        if (lane == r && r0 + r < mrows) {
+          float v = val[0][r];
+          if (has_res) v = Act<AT>::rn(buf.extra[r] + v);
+          store_out(y + r0 + r, v);
+        }
+    } else if constexpr (EPI == EPI_SWIGLU) {
+      AT *g = (AT *)a.y;
+#pragma unroll
+      for (int r = 0; r < ROWS; r++)
+        if (lane == r && r0 + r < mrows) store_out(g + r0 + r, Act<AT>::rn(silu_act<AT>(val[0][r]) * val[1][r]));
+    } else {
+      if (pos < 0 || pos >= a.max_context) return;  // never write outside the cache
+      if (w.m == 2) {  // value rows: plain copy into the cache row
+        AT *cv = (AT *)a.cache_v + (size_t)pos * a.rows2;
+#pragma unroll
+        for (int r = 0; r < ROWS; r++)
+          if (lane == r && r0 + r < mrows) store_out(cv + r0 + r, val[0][r]);
+      } else {         // query / key rows: rotate interleaved pairs (llama.ts:17-32)
+        AT *dst = w.m == 0 ? (AT *)a.y : (AT *)a.cache_k + (size_t)pos * a.rows1;
+#pragma unroll
+        for (int r = 0; r < ROWS; r += 2)
+          if (lane == r && r0 + r + 1 < mrows) {
+            const float c = buf.extra[r], d = buf.extra[r + 1];
+            const float av = val[0][r], bv = val[0][r + 1];
+            store_out(dst + r0 + r, Act<AT>::rn(av * c - bv * d));  // the build keeps a*b+c unfused: two roundings as in plain C
+            store_out(dst + r0 + r + 1, Act<AT>::rn(av * d + bv * c));
+          }
+      }
+    }
+  }
+
+  // xs: LDS for in_f activations; red: LDS float[blockDim/64]; lut: LDS float[16] (NF4 code book, written here)
+  __device__ static __forceinline__ void run(const GemvArgs &a, AT *xs, float *red, float *lut, Buf &bufA, bool preloaded, int pos) {
+    const int wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int ng = ngroups(a), nb = nbatch(a), gstride = gridDim.x * nw;
+    if (KIND == JSGRAD_W_NF4 && threadIdx.x < 16) lut[threadIdx.x] = NF4_CODE[threadIdx.x];
+    int grp = blockIdx.x * nw + wave, b = 0;
+    if (!preloaded && grp < ng) load_item(a, bufA, grp, 0, pos);
+
+    stage_x<AT, COHERENT>(a, xs, red);  // block-wide, ends with a barrier (which also publishes lut)
+
+    float acc[NM][ROWS];
+    Buf bufB;
+    auto advance = [&](int &g, int &bb) {
+      if (++bb == nb) { bb = 0; g += gstride; }
+    };
+    while (grp < ng) {
+      int g1 = grp, b1 = b;
+      advance(g1, b1);
+      if (g1 < ng) load_item(a, bufB, g1, b1, pos);
+      use_item(a, bufA, grp, b, acc, xs, lut, pos);
+      if (g1 >= ng) break;
+      grp = g1; b = b1;
+      advance(g1, b1);
+      if (g1 < ng) load_item(a, bufA, g1, b1, pos);
+      use_item(a, bufB, grp, b, acc, xs, lut, pos);
+      grp = g1; b = b1;
+    }
+  }
+};
+
+}  // namespace jsg

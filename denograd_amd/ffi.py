@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libjsgrad_hip.so")
 
 F32, F16 = 0, 1
 W_F32, W_F16, W_I8, W_NF4 = 0, 1, 2, 3
-PROF_KINDS = {"embed": 0, "rmsnorm": 1, "linear": 2, "qkv_rope": 3, "attn_decode": 4, "ffn_gate": 5, "argmax": 6}
+PROF_KINDS = {"embed": 0, "rmsnorm": 1, "linear": 2, "qkv_rope": 3, "attn_decode": 4, "ffn_gate": 5, "argmax": 6, "decode_step": 7}
 
 
 class HipError(RuntimeError):
@@ -60,6 +60,9 @@ SIGNATURES: dict[str, tuple[list, object]] = {
     "jsgrad_hip_attn_decode": ([_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32], _i32),
     "jsgrad_hip_ffn_gate": ([_i32, _vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _i32, _i32, _i32], _i32),
     "jsgrad_hip_argmax": ([_vp, _i32, _vp, _vp, _i32, _i32, _i32], _i32),
+    "jsgrad_hip_step_workspace_bytes": ([_i32, _i32, _i32], _sz),
+    "jsgrad_hip_decode_step": ([_vp], _i32),
+    "jsgrad_hip_step_status": ([_vp, C.POINTER(_i32)], _i32),
     "jsgrad_hip_int8_quantize": ([_vp, _i32, _i32, _vp, _vp, _i32], _i32),
     "jsgrad_hip_int8_dequant": ([_vp, _vp, _i32, _i32, _vp], _i32),
     "jsgrad_hip_nf4_quantize": ([_vp, _sz, _vp, _vp, _i32], _i32),
@@ -67,6 +70,22 @@ SIGNATURES: dict[str, tuple[list, object]] = {
     "jsgrad_hip_randn": ([_vp, _sz, _i32, _u64, _f32], _i32),
     "jsgrad_hip_fill": ([_vp, _sz, _i32, _f32], _i32),
 }
+
+
+
+class LayerDesc(C.Structure):
+    """jsgrad_hip_layer_t"""
+    _fields_ = [(n, C.c_void_p) for n in ("wq", "wk", "wv", "wo", "w1", "w2", "w3", "sq", "sk", "sv", "so", "s1", "s2", "s3",
+                                           "attention_norm", "ffn_norm", "cache_k", "cache_v")]
+
+
+class StepDesc(C.Structure):
+    """jsgrad_hip_step_t"""
+    _fields_ = ([("layers", C.c_void_p)] + [(n, C.c_int) for n in ("n_layers", "dim", "hidden", "n_heads", "n_kv_heads", "head_dim", "vocab", "max_context")]
+                + [("eps", C.c_float)] + [(n, C.c_int) for n in ("kind", "out_kind", "embed_kind", "act")]
+                + [(n, C.c_void_p) for n in ("tok_emb", "tok_scale", "out_w", "out_s", "final_norm", "rope_table", "state", "tokens_out")]
+                + [("tokens_cap", C.c_int)] + [(n, C.c_void_p) for n in ("h", "h2", "q", "attn", "g", "logits", "workspace", "trace")])
+
 
 _lib: C.CDLL | None = None
 

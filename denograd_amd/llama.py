@@ -103,6 +103,50 @@ class _Scratch:
         self.workspace = Tensor.zeros((nbytes,), "uint8", device)
 
 
+class _FusedStep:
+    """Descriptor of the single-kernel decode step (jsgrad_hip_decode_step): device array of per-layer tensors, the
+    activation rows and the workspace.  Built once per model; plays the role of the GraphRunner that replaces a captured
+    list of kernels by one device-side program (engine/jit.ts:71)."""
+
+    def __init__(self, model: "Transformer", ctx: "_Scratch"):
+        lib = ffi.load()
+        m = model
+        kinds = {l.kind for blk in m.layers for l in (blk.attention.wq, blk.attention.wk, blk.attention.wv, blk.attention.wo,
+                                                      blk.feed_forward.w1, blk.feed_forward.w2, blk.feed_forward.w3)}
+        if m.dtype != "float16" or len(kinds) != 1 or next(iter(kinds)) not in (ffi.W_F16, ffi.W_I8) or m.output.kind != next(iter(kinds)):
+            raise NotImplementedError("the single-kernel step is built for fp16 activations with fp16 or int8 layers and an lm_head stored the same way")
+        hd = m.dim // m.n_heads
+        if hd not in (64, 128) or m.n_heads // m.n_kv_heads not in (1, 2, 3, 4):
+            raise NotImplementedError("the single-kernel step is built for head_dim 64/128 and up to 4 query heads per kv head")
+        arr = (ffi.LayerDesc * len(m.layers))()
+        p = lambda t: t.ptr if t is not None else None
+        for i, blk in enumerate(m.layers):
+            a, f = blk.attention, blk.feed_forward
+            half = a.cache_kv.nbytes // 2
+            arr[i] = ffi.LayerDesc(a.wq.weight.ptr, a.wk.weight.ptr, a.wv.weight.ptr, a.wo.weight.ptr, f.w1.weight.ptr, f.w2.weight.ptr, f.w3.weight.ptr,
+                                   p(a.wq.scale), p(a.wk.scale), p(a.wv.scale), p(a.wo.scale), p(f.w1.scale), p(f.w2.scale), p(f.w3.scale),
+                                   blk.attention_norm.weight.ptr, blk.ffn_norm.weight.ptr, a.cache_kv.ptr, a.cache_kv.ptr + half)
+        raw = np.frombuffer(bytes(arr), np.uint8) if len(m.layers) else np.zeros(1, np.uint8)
+        self.layers = Tensor(raw.copy(), device=m.device)
+        nbytes = lib.jsgrad_hip_step_workspace_bytes(m.n_heads, m.n_kv_heads, hd)
+        self.workspace = Tensor.zeros((nbytes,), "uint8", m.device)
+        emb = m.tok_embeddings
+        from .nn import _KIND
+        self.desc = ffi.StepDesc(self.layers.ptr, len(m.layers), m.dim, m.hidden_dim, m.n_heads, m.n_kv_heads, hd, m.vocab_size, m.max_context,
+                                 m.norm.eps, next(iter(kinds)), m.output.kind, _KIND[emb.weight.dtype], ffi.F16,
+                                 emb.weight.ptr, p(emb.scale), m.output.weight.ptr, p(m.output.scale), m.norm.weight.ptr, m.freqs_cis.ptr,
+                                 m.state.ptr, m.tokens_out.ptr, m.max_context,
+                                 ctx.h.ptr, ctx.h2.ptr, ctx.q.ptr, ctx.attn.ptr, ctx.g.ptr, ctx.logits.ptr, self.workspace.ptr, None)
+
+    def launch(self) -> None:
+        check(ffi.load().jsgrad_hip_decode_step(C.byref(self.desc)))
+
+    def error(self) -> int:
+        e = C.c_int(0)
+        check(ffi.load().jsgrad_hip_step_status(self.workspace.ptr, C.byref(e)))
+        return e.value
+
+
 class TinyJit:
     """Capture-and-replay of one decode step (engine/jit.ts:236-352): call 0 runs eagerly, call 1 runs and is
     captured into a HIP graph, later calls replay the graph."""
@@ -139,7 +183,8 @@ class TinyJit:
 
 class Transformer:
     def __init__(self, dim: int, hidden_dim: int, n_heads: int, n_layers: int, norm_eps: float, vocab_size: int, linear=Linear, embedding=Embedding,
-                 n_kv_heads: int | None = None, rope_theta: float = 10000, max_context: int = 1024, jit: bool = True, feed_forward=FeedForward, device: str = "HIP"):
+                 n_kv_heads: int | None = None, rope_theta: float = 10000, max_context: int = 1024, jit: bool = True, feed_forward=FeedForward, device: str = "HIP",
+                 fused_step: bool = False):
         self.dim, self.hidden_dim, self.n_heads, self.vocab_size, self.max_context = dim, hidden_dim, n_heads, vocab_size, max_context
         self.n_kv_heads = n_kv_heads if n_kv_heads is not None else n_heads
         self.rope_theta, self.device = rope_theta, device
@@ -155,6 +200,9 @@ class Transformer:
         self.tokens_out = Tensor.zeros((max_context,), "int32", device)      # token produced at each start_pos
         self._ctx: _Scratch | None = None
         self._pos = 0                                                        # host mirror of state[1]
+        # False: one launch per fused op (the faster of the two today); True: the whole step as one persistent kernel
+        self.fused_step = fused_step
+        self._fused: _FusedStep | None = None
 
     # ---- plumbing
     @property
@@ -168,6 +216,8 @@ class Transformer:
             self.freqs_cis = precompute_freqs_cis(hd, self.max_context * 2, self.rope_theta, self.dtype, self.device)
             for layer in self.layers:
                 layer.attention._ensure_cache(self.dtype, self.device)
+            if self.fused_step:
+                self._fused = _FusedStep(self, self._ctx)      # raises NotImplementedError for models it was not built for
         return self._ctx
 
     def _step(self) -> Tensor:
@@ -177,6 +227,9 @@ class Transformer:
         if self._pos >= self.max_context:
             raise ValueError(f"KV cache of {self.max_context} positions is full")
         self._pos += 1
+        if self._fused is not None:
+            self._fused.launch()
+            return Tensor(buffer=self.state.lazydata.view(1, "int32", 0), shape=(), dtype="int32", device=self.device)
         h = self.tok_embeddings.call(self.state, out=ctx.h)
         for layer in self.layers:
             h = layer.call(h, self.state, self.freqs_cis, ctx)

@@ -114,23 +114,24 @@ class Llama3:
     explicit `args` dict), load a state dict, then `_prefill` / `_call` / `generate` token ids."""
 
     def __init__(self, size: str | None = None, quantize: str | None = None, device: str = "HIP", max_context: int = 8192, temperature: float = 0.0,
-                 top_k: int = 0, top_p: float = 0.0, alpha_f: float = 0.0, alpha_p: float = 0.0, args: dict | None = None):
+                 top_k: int = 0, top_p: float = 0.0, alpha_f: float = 0.0, alpha_p: float = 0.0, args: dict | None = None, fused_step: bool = False):
         self.size, self.quantize, self.device, self.max_context = size, quantize, device, max_context
         self.temperature, self.top_k, self.top_p, self.alpha_f, self.alpha_p = temperature, top_k, top_p, alpha_f, alpha_p
         self.linear, self.embedding, self.quantize_embeds = _classes(quantize)
         params = dict(MODEL_PARAMS[size]["args"]) if args is None else dict(args)
         self.params = params
         self.model = Transformer(params["dim"], params["hidden_dim"], params["n_heads"], params["n_layers"], params["norm_eps"], params["vocab_size"],
-                                 self.linear, self.embedding, params.get("n_kv_heads"), params["rope_theta"], self.max_context, True, device=device)
+                                 self.linear, self.embedding, params.get("n_kv_heads"), params["rope_theta"], self.max_context, True, device=device,
+                                 fused_step=fused_step)
         self.start_pos = 0
         self.last_seen_toks: list[int] = []
 
     # ---- loading
     @staticmethod
-    def from_config(cfg: dict, device: str = "HIP") -> "Llama3":
+    def from_config(cfg: dict, device: str = "HIP", fused_step: bool = False) -> "Llama3":
         args = {k: cfg[k] for k in ("dim", "hidden_dim", "n_heads", "n_kv_heads", "n_layers", "norm_eps", "rope_theta", "vocab_size")}
         q = cfg["quantize"] if cfg["quantize"] in ("int8", "nf4") else None
-        return Llama3(quantize=q, device=device, max_context=cfg["max_context"], args=args)
+        return Llama3(quantize=q, device=device, max_context=cfg["max_context"], args=args, fused_step=fused_step)
 
     def load_weights(self, weights: dict, quantized: bool = False) -> "Llama3":
         """llama3.ts:233-255: `weights` holds unquantised Meta-style tensors (host arrays or device Tensors) unless

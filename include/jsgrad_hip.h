@@ -79,7 +79,7 @@ int jsgrad_hip_event_destroy(void *event);
 /* Per-kernel statistics (DEBUG>=2 of engine/realize.ts:168-178; ProfileRangeEvent, runtime/allocator.ts:147-151):
  * while enabled, every Llama kernel launched outside a graph capture is bracketed by an event pair.  `read` waits
  * for the stream and returns launch count and summed milliseconds of one kind since profiling was enabled. */
-enum { JSGRAD_PROF_EMBED = 0, JSGRAD_PROF_RMSNORM, JSGRAD_PROF_LINEAR, JSGRAD_PROF_QKV_ROPE, JSGRAD_PROF_ATTN, JSGRAD_PROF_FFN_GATE, JSGRAD_PROF_ARGMAX };
+enum { JSGRAD_PROF_EMBED = 0, JSGRAD_PROF_RMSNORM, JSGRAD_PROF_LINEAR, JSGRAD_PROF_QKV_ROPE, JSGRAD_PROF_ATTN, JSGRAD_PROF_FFN_GATE, JSGRAD_PROF_ARGMAX, JSGRAD_PROF_STEP };
 int jsgrad_hip_profile(int enable);
 int jsgrad_hip_profile_read(int kind, int *host_out_count, double *host_out_total_ms);
 
@@ -140,6 +140,46 @@ int jsgrad_hip_ffn_gate(int kind, const void *w1, const void *s1, const void *w3
  * increments state[1]; tokens_out != NULL (an int32[tokens_cap] history) also receives the token at
  * tokens_out[old start_pos] when that index is inside it. */
 int jsgrad_hip_argmax(const void *logits, int n, int32_t *state, int32_t *tokens_out, int tokens_cap, int advance, int act);
+
+/* ---------------------------------------------------------------------------------
+ * The whole decode step as ONE kernel.
+ *
+ * What TinyJit + a device graph do in the reference - replay every kernel of Transformer.forward for one token as a
+ * single device-side program (engine/jit.ts:71 GraphRunner, :190-217 CapturedJit.call, models/llama.ts:201-220) - done
+ * here by a persistent kernel: one resident block per CU walks embedding, the five phases of every TransformerBlock,
+ * final norm + lm_head and the greedy argmax, with grid barriers in between and the next phase's weights already in
+ * flight.  Same arithmetic and results as the per-kernel entry points above.  fp16 activations; fp16 or int8 layers with
+ * an lm_head stored the same way.
+ * --------------------------------------------------------------------------------- */
+
+/* tensors of one TransformerBlock (models/llama.ts:112-128); scales are NULL for fp16 weights */
+typedef struct {
+  const void *wq, *wk, *wv, *wo, *w1, *w2, *w3;
+  const void *sq, *sk, *sv, *so, *s1, *s2, *s3;
+  const void *attention_norm, *ffn_norm;
+  void *cache_k, *cache_v; /* [max_context][n_kv_heads][head_dim] each */
+} jsgrad_hip_layer_t;
+
+/* host-side descriptor; `layers` is a DEVICE array of n_layers jsgrad_hip_layer_t */
+typedef struct {
+  const jsgrad_hip_layer_t *layers;
+  int n_layers, dim, hidden, n_heads, n_kv_heads, head_dim, vocab, max_context;
+  float eps;
+  int kind, out_kind, embed_kind, act; /* JSGRAD_W_* of the layers / lm_head / embedding table, JSGRAD_F16 */
+  const void *tok_emb, *tok_scale, *out_w, *out_s, *final_norm, *rope_table;
+  int32_t *state;      /* device {token, start_pos}: read at the start, advanced at the end */
+  int32_t *tokens_out; /* optional int32[tokens_cap] history, receives the token at [start_pos] */
+  int tokens_cap;
+  void *h, *h2, *q, *attn, *g, *logits; /* activation rows: dim, dim, n_heads*head_dim, n_heads*head_dim, hidden, vocab */
+  void *workspace;     /* jsgrad_hip_step_workspace_bytes(), zero-filled once before first use */
+  long long *trace;    /* optional device int64[2048]: block 0 stamps the 100 MHz device clock at every phase boundary */
+} jsgrad_hip_step_t;
+
+size_t jsgrad_hip_step_workspace_bytes(int n_heads, int n_kv_heads, int head_dim);
+int jsgrad_hip_decode_step(const jsgrad_hip_step_t *host_desc);
+/* Every wait inside the step kernel is bounded; *host_out_error becomes 1 if one ever ran out (the blocks were not all
+ * resident, e.g. another process held CUs) - the tokens of that step are then not to be trusted.  Waits for the stream. */
+int jsgrad_hip_step_status(const void *workspace, int *host_out_error);
 
 /* ---------------------------------------------------------------------------------
  * Load-time kernels

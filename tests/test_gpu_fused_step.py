@@ -1,0 +1,63 @@
+"""The single-kernel decode step (jsgrad_hip_decode_step) against the one-launch-per-op path and the oracle: same
+arithmetic, so the same tokens and (to summation order inside attention chunks) the same logits."""
+import numpy as np
+import pytest
+
+import oracle as orc
+from denograd_amd import synthetic
+from denograd_amd.llama3 import Llama3
+from tests.helpers import quantize_state
+from tests.test_gpu_model import CASES
+
+pytestmark = pytest.mark.gpu
+FUSABLE = ["tiny-f16", "small-int8", "small-f16-hd128"]
+
+
+@pytest.mark.parametrize("name", FUSABLE)
+def test_fused_step_equals_per_op_path_and_oracle(name):
+    cfg = CASES[name]
+    sd = quantize_state(cfg, synthetic.random_state_dict(cfg, seed=0, std=0.02))
+    fused = Llama3.from_config(cfg, fused_step=True).load_weights(sd, quantized=True)
+    plain = Llama3.from_config(cfg, fused_step=False).load_weights(sd, quantized=True)
+    cpu = orc.OracleModel(cfg, sd)
+    prompt = [int(t) for t in synthetic.random_prompt(cfg, 16, seed=1)]
+    a = fused.chat_tokens(prompt, 32)["tokens"]
+    b = plain.chat_tokens(prompt, 32)["tokens"]
+    assert fused.model._fused is not None and plain.model._fused is None
+    assert fused.model._fused.error() == 0, "a bounded wait inside the step kernel ran out"
+    assert a == b
+    assert a == list(cpu.generate(prompt, 32))
+    la, lb = fused.model.logits.numpy().astype(np.float32), plain.model.logits.numpy().astype(np.float32)
+    # attention is cut into different chunks on the two paths, so sums differ in their last bits and a few fp16 roundings flip
+    assert np.allclose(la, lb, rtol=2e-3, atol=2e-3)
+
+
+def test_fused_step_long_context_many_chunks():
+    """Several attention chunks per kv head and more items than blocks per head.  Both paths are fed the same tokens
+    (teacher forcing): over a thousand free-running steps on near-flat logits the two would part at the first sub-ulp tie."""
+    cfg = dict(CASES["tiny-f16"], max_context=1536, name="tiny-f16-long")
+    sd = synthetic.random_state_dict(cfg, seed=3, std=0.05)
+    fused = Llama3.from_config(cfg, fused_step=True).load_weights(sd, quantized=True)
+    plain = Llama3.from_config(cfg, fused_step=False).load_weights(sd, quantized=True)
+    toks = [int(t) for t in synthetic.random_prompt(cfg, 1300, seed=2)]
+    agree = 0
+    for pos, t in enumerate(toks):
+        ta = fused._call(t); fused.start_pos += 1
+        tb = plain._call(t); plain.start_pos += 1
+        agree += int(ta == tb)
+        if pos in (0, 63, 64, 65, 300, 777, 1299):
+            la, lb = fused.model.logits.numpy().astype(np.float32), plain.model.logits.numpy().astype(np.float32)
+            assert np.allclose(la, lb, rtol=2e-3, atol=2e-3), f"position {pos}"
+    assert fused.model._fused.error() == 0
+    assert agree >= 0.99 * len(toks)
+
+
+def test_fused_step_rejects_what_it_was_not_built_for():
+    cfg = CASES["small-nf4"]
+    sd = quantize_state(cfg, synthetic.random_state_dict(cfg, seed=0))
+    llm = Llama3.from_config(cfg, fused_step=True).load_weights(sd, quantized=True)
+    with pytest.raises(NotImplementedError):
+        llm._call(1)
+    auto = Llama3.from_config(cfg).load_weights(sd, quantized=True)      # default: falls back to one launch per op
+    auto._call(1)
+    assert auto.model._fused is None
