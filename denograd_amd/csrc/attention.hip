@@ -11,6 +11,14 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_decode_kernel(AttnArgs a) {
   typedef Attn<AT, HD, NREP, ATT_THREADS / 64, false> A;
   __shared__ typename A::Smem sm;
   const int g = blockIdx.x, split = blockIdx.y;
+  if (const int z = blockIdx.z) {   // sequence z of a batch: same position, its own rows of q / out / cache / workspace
+    a.q = (const char *)a.q + z * a.q_bstride;
+    a.out = (char *)a.out + z * a.q_bstride;
+    a.cache_k = (const char *)a.cache_k + z * a.cache_bstride;
+    a.cache_v = (const char *)a.cache_v + z * a.cache_bstride;
+    a.counters += z * a.n_kv_heads;
+    a.partial += z * a.partial_bstride;
+  }
   const int pos = a.st[1];
   if (pos < 0 || pos >= a.max_context) return;
   const int T = pos + 1;
@@ -28,8 +36,8 @@ static int nsplit_for(int max_context) {
   return by_lds > wanted ? by_lds : wanted;
 }
 
-template <typename AT, int HD> static int launch_attn(const AttnArgs &a, int n_rep) {
-  dim3 grid(a.n_kv_heads, a.nsplit), block(ATT_THREADS);
+template <typename AT, int HD> static int launch_attn(const AttnArgs &a, int n_rep, int batch = 1) {
+  dim3 grid(a.n_kv_heads, a.nsplit, batch), block(ATT_THREADS);
 #define JSG_REP(N)                                                                                   \
   case N:                                                                                            \
     JSG_LAUNCH(PROF_ATTN, (attn_decode_kernel<AT, HD, N>), grid, block, 0, a);                         \
@@ -52,6 +60,33 @@ size_t jsgrad_hip_attn_workspace_bytes(int n_heads, int n_kv_heads, int head_dim
   // counters + partials for the largest split count any max_context can ask for (256)
   (void)n_kv_heads;
   return 256 + (size_t)n_heads * 256 * (head_dim + 2) * sizeof(float);
+}
+
+size_t jsgrad_hip_attn_batch_workspace_bytes(int batch, int n_heads, int n_kv_heads, int head_dim) {
+  // per sequence: n_kv_heads counters, then the partials as above
+  return (size_t)batch * (((size_t)n_kv_heads * sizeof(int) + 255) / 256 * 256 + (size_t)n_heads * 256 * (head_dim + 2) * sizeof(float));
+}
+
+int jsgrad_hip_attn_decode_batch(const void *q, const void *cache_k, const void *cache_v, const int32_t *st, void *out, void *workspace, int batch,
+                                 int n_heads, int n_kv_heads, int head_dim, int max_context) {
+  JSG_READY();
+  JSG_REQUIRE(q && cache_k && cache_v && st && out && workspace, "jsgrad_hip_attn_decode_batch: null pointer argument");
+  JSG_REQUIRE(batch > 0 && batch <= 65535, "jsgrad_hip_attn_decode_batch: batch %d", batch);
+  JSG_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_kv_heads <= 64 && n_heads % n_kv_heads == 0, "jsgrad_hip_attn_decode_batch: n_heads %d / n_kv_heads %d", n_heads, n_kv_heads);
+  JSG_REQUIRE(head_dim == 64 || head_dim == 128, "jsgrad_hip_attn_decode_batch: head_dim %d (64 and 128 are built)", head_dim);
+  JSG_REQUIRE(max_context > 0 && max_context <= 256 * ATT_CHUNK_MAX, "jsgrad_hip_attn_decode_batch: max_context %d exceeds %d", max_context, 256 * ATT_CHUNK_MAX);
+  const size_t counter_bytes = ((size_t)n_kv_heads * sizeof(int) + 255) / 256 * 256;
+  AttnArgs a;
+  a.q = q; a.cache_k = cache_k; a.cache_v = cache_v; a.st = st; a.out = out;
+  a.counters = (int *)workspace;                                   // [batch][n_kv_heads], densely packed
+  a.partial = (float *)((char *)workspace + (size_t)batch * counter_bytes);
+  a.n_kv_heads = n_kv_heads; a.nsplit = nsplit_for(max_context); a.max_context = max_context;
+  a.scale = (float)(1.0 / sqrt((double)head_dim));
+  a.q_bstride = (size_t)n_heads * head_dim * sizeof(_Float16);
+  a.cache_bstride = (size_t)max_context * n_kv_heads * head_dim * sizeof(_Float16);
+  a.partial_bstride = (size_t)n_heads * 256 * (head_dim + 2);
+  const int n_rep = n_heads / n_kv_heads;
+  return head_dim == 64 ? launch_attn<_Float16, 64>(a, n_rep, batch) : launch_attn<_Float16, 128>(a, n_rep, batch);
 }
 
 int jsgrad_hip_attn_decode(const void *q, const void *cache_k, const void *cache_v, const int32_t *st, void *out, void *workspace, int n_heads,

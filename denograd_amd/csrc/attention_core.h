@@ -25,6 +25,9 @@ struct AttnArgs {
   float *partial;  // [n_kv_heads][nsplit][n_rep][HD + 2]
   int n_kv_heads, nsplit, max_context;
   float scale;     // float(1 / sqrt(head_dim)) (tensor.ts:3923 `.div(Math.sqrt(d))` = mul by the folded reciprocal)
+  // several sequences at the same position (grid z): distance between consecutive sequences, in bytes (q, out, caches)
+  // and in elements (counters, partial); zero for a single sequence
+  size_t q_bstride = 0, cache_bstride = 0, partial_bstride = 0;
 };
 
 template <int G> __device__ __forceinline__ float group_sum(float v) {

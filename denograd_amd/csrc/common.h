@@ -23,7 +23,7 @@ int fail(const char *fmt, ...);
 int fail_hip(hipError_t e, const char *what);
 
 // per-kernel timing with HIP events on the library stream (off unless jsgrad_hip_profile(1))
-enum { PROF_EMBED = 0, PROF_RMSNORM, PROF_LINEAR, PROF_QKV_ROPE, PROF_ATTN, PROF_FFN_GATE, PROF_ARGMAX, PROF_STEP, PROF_KINDS };
+enum { PROF_EMBED = 0, PROF_RMSNORM, PROF_LINEAR, PROF_QKV_ROPE, PROF_ATTN, PROF_FFN_GATE, PROF_ARGMAX, PROF_STEP, PROF_GEMM, PROF_ATTN_PREFILL, PROF_KINDS };
 // Event pair for the next launch of `kind`, or false when profiling is off (or capturing, or out of slots).  The pair
 // is handed to hipExtLaunchKernelGGL, which stamps it with the dispatch's own begin/end times, so the elapsed time is
 // the kernel alone: no marker packets, no launch latency.
@@ -185,6 +185,13 @@ __device__ __forceinline__ float xexp2h(float d) {
 }
 // Tensor.exp on float tensors (tensor.ts:147-154)
 __device__ __forceinline__ float exp_f32(float x) { return xexp2f(__fmul_rn(x, 1.4426950408889634f)); }
+
+// NF4 code book (llama3.ts:80-81); the CODE tensor is float16, so every literal is rounded to fp16 first
+#define JSG_C16(x) ((float)(_Float16)(x))
+static __device__ __constant__ float NF4_CODE[16] = {JSG_C16(-1.0f), JSG_C16(-0.6961928009986877f), JSG_C16(-0.5250730514526367f), JSG_C16(-0.39491748809814453f),
+                                              JSG_C16(-0.28444138169288635f), JSG_C16(-0.18477343022823334f), JSG_C16(-0.09105003625154495f), JSG_C16(0.0f),
+                                              JSG_C16(0.07958029955625534f), JSG_C16(0.16093020141124725f), JSG_C16(0.24611230194568634f), JSG_C16(0.33791524171829224f),
+                                              JSG_C16(0.44070982933044434f), JSG_C16(0.5626170039176941f), JSG_C16(0.7229568362236023f), JSG_C16(1.0f)};
 
 // silu(a) = a * 1/(1 + exp2(a * -1/ln2)) (tensor.ts:2909-2911, 3210-3226) in the activation dtype's arithmetic
 template <typename AT> __device__ __forceinline__ float silu_act(float a);

@@ -1,0 +1,371 @@
+// Several-row linear layers on the gfx950 matrix cores: y[M][N] = x[M][K] . W[N][K]^T for M > 1 rows of fp16
+// activations (batched prefill and batched decode), fp32 accumulate, fp16 out.
+//
+// What the reference computes (/root/reference/jsgrad/tensor.ts:2593-2605 `dot`, :3800 `linear`; Int8Linear.call
+// /root/reference/jsgrad/models/llama3.ts:35; NF4Linear.call :91-97): with more than one input row the weight operand is
+// expanded over the rows, so a quantised weight is first realised in fp16, W = RN16(code * scale), and the products of
+// two fp16 values are then summed in float.  The dequantised fp16 tile written to LDS here is exactly that realised
+// matrix; v_pk_mul_f16 of the exact fp16 code by the fp16 scale is the single rounding RN16(code * scale).
+//
+// Tiling: 256 threads = 4 wavefronts laid out WGM x WGN; a wavefront owns TM x TN tiles of 32x32 outputs and walks K in
+// steps of 16 with v_mfma_f32_32x32x16_f16.  Both operands are K-contiguous in memory (x rows, W rows), so a lane's
+// 8-element operand fragment is one 128-bit LDS read.  LDS rows are padded by 8 halves (144-byte stride), which
+// spreads the 32 rows of a fragment read over all banks.  One LDS buffer, register prefetch of the next K tile issued
+// before the MFMAs of the current one.  Tile ids are remapped so that the blocks resident on one XCD (round-robin by
+// block id) share operand tiles in that XCD's L2.
+#include "common.h"
+
+namespace jsg {
+
+typedef float f16_t __attribute__((ext_vector_type(16)));
+
+enum { GEPI_STORE = 0, GEPI_ROPE_KV = 1, GEPI_SWIGLU = 2 };
+
+constexpr int GEMM_BK = 64;           // K elements per LDS tile
+constexpr int GEMM_LDS_STRIDE = 72;   // halves per LDS row (64 + 8 padding)
+constexpr int GEMM_THREADS = 256;
+
+struct GemmArgs {
+  const void *w0, *w1, *w2;           // up to three weight matrices stacked along N (wq|wk|wv, or w1|w3)
+  const _Float16 *s0, *s1, *s2;       // their scales (int8: per row; nf4: per 64 elements)
+  int n0, n1, n2;                     // their row counts
+  int M, N, K;                        // N = columns of the output this launch produces
+  const _Float16 *x;                  // [M][K]
+  _Float16 *y;                        // [M][N]  (ROPE_KV: q rows [M][n0])
+  const _Float16 *residual;           // [M][N] or null
+  // ROPE_KV
+  const _Float16 *rope_table;         // [2*max_context][hd/2][2]
+  _Float16 *cache_k, *cache_v;        // [B][max_context][n1]
+  int seq_len, start_pos, head_dim, max_context;
+};
+
+__device__ __forceinline__ uint32_t pk_mul_h2(uint32_t a, h2_t s) {
+  h2_t r = as_h2(a) * s;
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+// 4 int8 codes (one dword) -> 4 exact fp16 values: byte | 0x6400 is 1024 + (code ^ 0x80), minus 1152 leaves the code
+__device__ __forceinline__ void i8x4_to_h2x2(uint32_t q, uint32_t &lo, uint32_t &hi) {
+  const uint32_t u = q ^ 0x80808080u;
+  const h2_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+  h2_t a = as_h2(__builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias;   // bytes 0,1
+  h2_t b = as_h2(__builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias;   // bytes 2,3
+  lo = __builtin_bit_cast(uint32_t, a);
+  hi = __builtin_bit_cast(uint32_t, b);
+}
+
+template <int KIND, int EPI, int WGM, int WGN, int TM, int TN>
+__global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(GemmArgs a) {
+  static_assert(WGM * WGN == 4, "four wavefronts");
+  static_assert(EPI != GEPI_SWIGLU || TN % 2 == 0, "a wavefront holds the w1 and the w3 tile of the same columns");
+  constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32, LS = GEMM_LDS_STRIDE;
+  constexpr int A_LOADS = BM / 32;                                                    // 16-byte loads per thread per K tile
+  constexpr int B_ROWS_PER_PASS = KIND == JSGRAD_W_F16 ? 32 : KIND == JSGRAD_W_I8 ? 64 : 128;
+  constexpr int B_CHUNKS = GEMM_THREADS / B_ROWS_PER_PASS;                             // 16-byte chunks per row of the K tile
+  constexpr int B_LOADS = BN / B_ROWS_PER_PASS;
+  static_assert(B_LOADS >= 1, "tile too narrow for this weight format");
+  __shared__ __align__(16) _Float16 As[BM * LS];
+  __shared__ __align__(16) _Float16 Bs[BN * LS];
+  __shared__ _Float16 lut[16];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WGN, wn = wave % WGN;
+  const int l32 = lane & 31, lg = lane >> 5;
+
+  if constexpr (KIND == JSGRAD_W_NF4) {
+    if (tid < 16) lut[tid] = (_Float16)NF4_CODE[tid];
+  }
+
+  // ---- tile id: XCD-contiguous, then grouped so that neighbouring ids share an x tile column-block
+  const int tiles_m = (a.M + BM - 1) / BM, tiles_n = a.N / (EPI == GEPI_SWIGLU ? BN / 2 : BN);
+  const int nblocks = tiles_m * tiles_n;
+  int bid = blockIdx.x;
+  {
+    const int per = nblocks / 8;
+    if (bid < per * 8) bid = (bid & 7) * per + (bid >> 3);
+  }
+  constexpr int GROUP = 8;
+  const int in_group = GROUP * tiles_n;
+  const int first_m = (bid / in_group) * GROUP;
+  const int gsz = min(tiles_m - first_m, GROUP);
+  const int tm_ = first_m + (bid % in_group) % gsz, tn_ = (bid % in_group) / gsz;
+  const int m0 = tm_ * BM;
+  const int n0_out = tn_ * (EPI == GEPI_SWIGLU ? BN / 2 : BN);   // first output column of this tile
+
+  // ---- B source of every row this thread loads: (matrix, row) is fixed over the K loop
+  const unsigned char *bsrc[B_LOADS];
+  h2_t bscale[B_LOADS];
+  const _Float16 *bscale_ptr[B_LOADS];
+  const int brow_t = tid / B_CHUNKS, bchunk = tid % B_CHUNKS;
+#pragma unroll
+  for (int i = 0; i < B_LOADS; i++) {
+    const int r = brow_t + i * B_ROWS_PER_PASS;      // row inside the B tile
+    const void *w; const _Float16 *s; int row;
+    if constexpr (EPI == GEPI_SWIGLU) {
+      const bool up = r >= BN / 2;
+      w = up ? a.w1 : a.w0; s = up ? a.s1 : a.s0; row = n0_out + (up ? r - BN / 2 : r);
+    } else if constexpr (EPI == GEPI_ROPE_KV) {
+      const int n = n0_out + r;
+      if (n < a.n0) { w = a.w0; s = a.s0; row = n; }
+      else if (n < a.n0 + a.n1) { w = a.w1; s = a.s1; row = n - a.n0; }
+      else { w = a.w2; s = a.s2; row = n - a.n0 - a.n1; }
+    } else { w = a.w0; s = a.s0; row = n0_out + r; }
+    const size_t e = (size_t)row * a.K;              // element offset of the row
+    if constexpr (KIND == JSGRAD_W_F16) bsrc[i] = (const unsigned char *)w + e * 2 + bchunk * 16;
+    else if constexpr (KIND == JSGRAD_W_I8) { bsrc[i] = (const unsigned char *)w + e + bchunk * 16; const _Float16 sv = s[row]; bscale[i] = h2_t{sv, sv}; }
+    else { bsrc[i] = (const unsigned char *)w + e / 2 + bchunk * 16; bscale_ptr[i] = s + e / 64; }
+  }
+  const unsigned char *asrc[A_LOADS];
+  const int arow_t = tid / 8, achunk = tid % 8;
+#pragma unroll
+  for (int i = 0; i < A_LOADS; i++) {
+    int m = m0 + arow_t + i * 32;
+    if (m >= a.M) m = a.M - 1;                        // rows past the end are computed and never stored
+    asrc[i] = (const unsigned char *)(a.x + (size_t)m * a.K) + achunk * 16;
+  }
+
+  f16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+  u4_t ga[A_LOADS], gb[B_LOADS];
+  _Float16 gs[B_LOADS];
+  auto issue = [&](int kt) {
+    const size_t ko = (size_t)kt * GEMM_BK;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; i++) ga[i] = *(const u4_t *)(asrc[i] + ko * 2);
+#pragma unroll
+    for (int i = 0; i < B_LOADS; i++) {
+      if constexpr (KIND == JSGRAD_W_F16) gb[i] = *(const u4_t *)(bsrc[i] + ko * 2);
+      else if constexpr (KIND == JSGRAD_W_I8) gb[i] = *(const u4_t *)(bsrc[i] + ko);
+      else { gb[i] = *(const u4_t *)(bsrc[i] + ko / 2); gs[i] = bscale_ptr[i][kt]; }
+    }
+  };
+  auto commit = [&]() {
+#pragma unroll
+    for (int i = 0; i < A_LOADS; i++) *(u4_t *)&As[(arow_t + i * 32) * LS + achunk * 8] = ga[i];
+#pragma unroll
+    for (int i = 0; i < B_LOADS; i++) {
+      _Float16 *dst = &Bs[(brow_t + i * B_ROWS_PER_PASS) * LS];
+      if constexpr (KIND == JSGRAD_W_F16) *(u4_t *)(dst + bchunk * 8) = gb[i];
+      else if constexpr (KIND == JSGRAD_W_I8) {
+        u4_t o0, o1;
+        uint32_t lo, hi;
+        i8x4_to_h2x2(gb[i].x, lo, hi); o0.x = pk_mul_h2(lo, bscale[i]); o0.y = pk_mul_h2(hi, bscale[i]);
+        i8x4_to_h2x2(gb[i].y, lo, hi); o0.z = pk_mul_h2(lo, bscale[i]); o0.w = pk_mul_h2(hi, bscale[i]);
+        i8x4_to_h2x2(gb[i].z, lo, hi); o1.x = pk_mul_h2(lo, bscale[i]); o1.y = pk_mul_h2(hi, bscale[i]);
+        i8x4_to_h2x2(gb[i].w, lo, hi); o1.z = pk_mul_h2(lo, bscale[i]); o1.w = pk_mul_h2(hi, bscale[i]);
+        *(u4_t *)(dst + bchunk * 16) = o0;
+        *(u4_t *)(dst + bchunk * 16 + 8) = o1;
+      } else {
+        // 16 bytes = 32 elements; the high nibble of a byte is the even element (llama3.ts:92-94)
+        const h2_t sv = {gs[i], gs[i]};
+        uint32_t wds[4] = {gb[i].x, gb[i].y, gb[i].z, gb[i].w};
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+          u4_t o;
+          uint32_t outw[4];
+#pragma unroll
+          for (int b = 0; b < 4; b++) {
+            const uint32_t byte = (wds[d] >> (8 * b)) & 0xffu;
+            const h2_t c = {lut[byte >> 4], lut[byte & 15]};
+            h2_t r = c * sv;
+            outw[b] = __builtin_bit_cast(uint32_t, r);
+          }
+          o.x = outw[0]; o.y = outw[1]; o.z = outw[2]; o.w = outw[3];
+          *(u4_t *)(dst + bchunk * 32 + d * 8) = o;
+        }
+      }
+    }
+  };
+
+  const int nk = a.K / GEMM_BK;
+  issue(0);
+  if constexpr (KIND == JSGRAD_W_NF4) __syncthreads();   // the code table is in LDS
+  for (int kt = 0; kt < nk; kt++) {
+    commit();
+    __syncthreads();
+    if (kt + 1 < nk) issue(kt + 1);
+#pragma unroll
+    for (int kk = 0; kk < GEMM_BK / 16; kk++) {
+      h8_t af[TM], bf[TN];
+#pragma unroll
+      for (int i = 0; i < TM; i++) af[i] = *(const h8_t *)&As[((wm * TM + i) * 32 + l32) * LS + kk * 16 + lg * 8];
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        int rbase;
+        if constexpr (EPI == GEPI_SWIGLU) rbase = j < TN / 2 ? (wn * (TN / 2) + j) * 32 : BN / 2 + (wn * (TN / 2) + j - TN / 2) * 32;
+        else rbase = (wn * TN + j) * 32;
+        bf[j] = *(const h8_t *)&Bs[(rbase + l32) * LS + kk * 16 + lg * 8];
+      }
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue.  Accumulator r of a lane is output row 8*(r/4) + 4*(lane/32) + r%4, column lane%32 of the 32x32 tile.
+#pragma unroll
+  for (int i = 0; i < TM; i++) {
+    const int mbase = m0 + (wm * TM + i) * 32 + lg * 4;
+    if constexpr (EPI == GEPI_SWIGLU) {
+#pragma unroll
+      for (int j = 0; j < TN / 2; j++) {
+        const int n = n0_out + (wn * (TN / 2) + j) * 32 + l32;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int m = mbase + 8 * (r / 4) + (r % 4);
+          if (m < a.M) {
+            // silu(w1 x) * (w3 x), each GEMM output and the product stored as fp16 (llama.ts:108-110)
+            const float g = rn16(acc[i][j][r]), u = rn16(acc[i][j + TN / 2][r]);
+            a.y[(size_t)m * a.N + n] = (_Float16)(silu_act<_Float16>(g) * u);
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        const int n = n0_out + (wn * TN + j) * 32 + l32;
+        if constexpr (EPI == GEPI_STORE) {
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int m = mbase + 8 * (r / 4) + (r % 4);
+            if (m < a.M) {
+              float v = rn16(acc[i][j][r]);
+              if (a.residual) v = (float)a.residual[(size_t)m * a.N + n] + v;
+              a.y[(size_t)m * a.N + n] = (_Float16)v;
+            }
+          }
+        } else {
+          // wq | wk | wv columns; q and k get the interleaved-pair rotation (llama.ts:17-32), k and v go to the cache rows
+          const int which = n < a.n0 ? 0 : (n < a.n0 + a.n1 ? 1 : 2);
+          const int nl = which == 0 ? n : (which == 1 ? n - a.n0 : n - a.n0 - a.n1);
+          const int pair = (nl % a.head_dim) >> 1;
+          const bool odd = nl & 1;
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int m = mbase + 8 * (r / 4) + (r % 4);
+            const float own = rn16(acc[i][j][r]);
+            const float other = dpp_f<0xB1>(own);              // the neighbouring column: the other half of the pair
+            if (m < a.M) {
+              const int b = m / a.seq_len, pos = a.start_pos + m % a.seq_len;
+              float v = own;
+              if (which < 2) {
+                const h2_t cs = *(const h2_t *)(a.rope_table + ((size_t)pos * (a.head_dim / 2) + pair) * 2);
+                const float c = (float)cs.x, d = (float)cs.y;
+                v = odd ? other * d + own * c : own * c - other * d;
+              }
+              if (which == 0) a.y[(size_t)m * a.n0 + nl] = (_Float16)v;
+              else {
+                _Float16 *cache = which == 1 ? a.cache_k : a.cache_v;
+                cache[((size_t)b * a.max_context + pos) * a.n1 + nl] = (_Float16)v;
+              }
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+// ---- host side ---------------------------------------------------------------------------------------------------
+
+template <int KIND, int EPI, int WGM, int WGN, int TM, int TN> static int launch_gemm(const GemmArgs &a, int prof_kind) {
+  constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
+  const int out_per_tile = EPI == GEPI_SWIGLU ? BN / 2 : BN;
+  const int tiles = ((a.M + BM - 1) / BM) * (a.N / out_per_tile);
+  JSG_LAUNCH(prof_kind, (gemm_kernel<KIND, EPI, WGM, WGN, TM, TN>), dim3(tiles), dim3(GEMM_THREADS), 0, a);
+  return 0;
+}
+
+template <int EPI> static int dispatch_gemm(int kind, const GemmArgs &a, int prof_kind) {
+  // tall inputs: 256x128 block tiles; short ones (batched decode): 32 rows x 128 columns per block
+  const bool tall = a.M > 64;
+#define JSG_CASE(K)                                                                                                    \
+  case K:                                                                                                              \
+    return tall ? launch_gemm<K, EPI, 2, 2, 4, 2>(a, prof_kind) : launch_gemm<K, EPI, 1, 4, 1, EPI == GEPI_SWIGLU ? 2 : 1>(a, prof_kind);
+  switch (kind) {
+    JSG_CASE(JSGRAD_W_F16)
+    JSG_CASE(JSGRAD_W_I8)
+    JSG_CASE(JSGRAD_W_NF4)
+  }
+#undef JSG_CASE
+  return fail("jsgrad_hip_gemm: weight kind %d is not built for several rows (fp16, int8 and nf4 are)", kind);
+}
+
+// largest column tile any configuration uses: output widths must be multiples of it
+constexpr int GEMM_N_ALIGN = 128;
+
+static int check_gemm(const char *who, int kind, int rows, int in_f) {
+  JSG_REQUIRE(kind == JSGRAD_W_F16 || kind == JSGRAD_W_I8 || kind == JSGRAD_W_NF4, "%s: weight kind %d is not built for several rows (fp16, int8 and nf4 are)", who, kind);
+  JSG_REQUIRE(rows > 0, "%s: %d rows", who, rows);
+  JSG_REQUIRE(in_f > 0 && in_f % GEMM_BK == 0, "%s: in_features %d must be a positive multiple of %d", who, in_f, GEMM_BK);
+  return 0;
+}
+
+}  // namespace jsg
+
+using namespace jsg;
+
+extern "C" {
+
+int jsgrad_hip_gemm(int kind, const void *w, const void *scale, int out_f, int in_f, const void *x, int rows, void *y, const void *residual) {
+  JSG_READY();
+  if (int rc = check_gemm("jsgrad_hip_gemm", kind, rows, in_f)) return rc;
+  JSG_REQUIRE(w && x && y, "jsgrad_hip_gemm: null pointer argument");
+  JSG_REQUIRE(kind == JSGRAD_W_F16 || scale, "jsgrad_hip_gemm: quantised weights need their scales");
+  JSG_REQUIRE(out_f > 0 && out_f % GEMM_N_ALIGN == 0, "jsgrad_hip_gemm: out_features %d must be a positive multiple of %d", out_f, GEMM_N_ALIGN);
+  GemmArgs a = {};
+  a.w0 = w; a.s0 = (const _Float16 *)scale; a.n0 = out_f;
+  a.M = rows; a.N = out_f; a.K = in_f;
+  a.x = (const _Float16 *)x; a.y = (_Float16 *)y; a.residual = (const _Float16 *)residual;
+  return dispatch_gemm<GEPI_STORE>(kind, a, PROF_GEMM);
+}
+
+int jsgrad_hip_gemm_qkv_rope(int kind, const void *wq, const void *sq, const void *wk, const void *sk, const void *wv, const void *sv, const void *x,
+                             int rows, int seq_len, int start_pos, const void *rope_table, void *q_out, void *cache_k, void *cache_v, int dim,
+                             int n_heads, int n_kv_heads, int head_dim, int max_context) {
+  JSG_READY();
+  if (int rc = check_gemm("jsgrad_hip_gemm_qkv_rope", kind, rows, dim)) return rc;
+  JSG_REQUIRE(wq && wk && wv && x && rope_table && q_out && cache_k && cache_v, "jsgrad_hip_gemm_qkv_rope: null pointer argument");
+  JSG_REQUIRE(kind == JSGRAD_W_F16 || (sq && sk && sv), "jsgrad_hip_gemm_qkv_rope: quantised weights need their scales");
+  JSG_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && n_heads > 0 && n_kv_heads > 0, "jsgrad_hip_gemm_qkv_rope: bad head geometry");
+  const int nq = n_heads * head_dim, nkv = n_kv_heads * head_dim;
+  JSG_REQUIRE(nq % GEMM_N_ALIGN == 0 && nkv % GEMM_N_ALIGN == 0, "jsgrad_hip_gemm_qkv_rope: n_heads*head_dim %d and n_kv_heads*head_dim %d must be multiples of %d", nq, nkv,
+              GEMM_N_ALIGN);
+  JSG_REQUIRE(seq_len > 0 && rows % seq_len == 0, "jsgrad_hip_gemm_qkv_rope: %d rows are not whole sequences of %d", rows, seq_len);
+  JSG_REQUIRE(start_pos >= 0 && start_pos + seq_len <= max_context, "jsgrad_hip_gemm_qkv_rope: positions [%d, %d) outside the cache of %d", start_pos,
+              start_pos + seq_len, max_context);
+  GemmArgs a = {};
+  a.w0 = wq; a.w1 = wk; a.w2 = wv;
+  a.s0 = (const _Float16 *)sq; a.s1 = (const _Float16 *)sk; a.s2 = (const _Float16 *)sv;
+  a.n0 = nq; a.n1 = nkv; a.n2 = nkv;
+  a.M = rows; a.N = nq + 2 * nkv; a.K = dim;
+  a.x = (const _Float16 *)x; a.y = (_Float16 *)q_out;
+  a.rope_table = (const _Float16 *)rope_table; a.cache_k = (_Float16 *)cache_k; a.cache_v = (_Float16 *)cache_v;
+  a.seq_len = seq_len; a.start_pos = start_pos; a.head_dim = head_dim; a.max_context = max_context;
+  return dispatch_gemm<GEPI_ROPE_KV>(kind, a, PROF_GEMM);
+}
+
+int jsgrad_hip_gemm_ffn_gate(int kind, const void *w1, const void *s1, const void *w3, const void *s3, const void *x, int rows, void *y, int dim,
+                             int hidden) {
+  JSG_READY();
+  if (int rc = check_gemm("jsgrad_hip_gemm_ffn_gate", kind, rows, dim)) return rc;
+  JSG_REQUIRE(w1 && w3 && x && y, "jsgrad_hip_gemm_ffn_gate: null pointer argument");
+  JSG_REQUIRE(kind == JSGRAD_W_F16 || (s1 && s3), "jsgrad_hip_gemm_ffn_gate: quantised weights need their scales");
+  JSG_REQUIRE(hidden > 0 && hidden % GEMM_N_ALIGN == 0, "jsgrad_hip_gemm_ffn_gate: hidden_dim %d must be a positive multiple of %d", hidden, GEMM_N_ALIGN);
+  GemmArgs a = {};
+  a.w0 = w1; a.w1 = w3; a.s0 = (const _Float16 *)s1; a.s1 = (const _Float16 *)s3;
+  a.n0 = hidden; a.n1 = hidden;
+  a.M = rows; a.N = hidden; a.K = dim;
+  a.x = (const _Float16 *)x; a.y = (_Float16 *)y;
+  return dispatch_gemm<GEPI_SWIGLU>(kind, a, PROF_GEMM);
+}
+
+}  // extern "C"

@@ -38,13 +38,6 @@ template <> struct WFmt<JSGRAD_W_F16> { static constexpr int VEC = 8; };
 template <> struct WFmt<JSGRAD_W_I8> { static constexpr int VEC = 16; };
 template <> struct WFmt<JSGRAD_W_NF4> { static constexpr int VEC = 32; };
 
-// NF4 code book (llama3.ts:80-81); the CODE tensor is float16, so every literal is rounded to fp16 first
-#define JSG_C16(x) ((float)(_Float16)(x))
-static __device__ __constant__ float NF4_CODE[16] = {JSG_C16(-1.0f), JSG_C16(-0.6961928009986877f), JSG_C16(-0.5250730514526367f), JSG_C16(-0.39491748809814453f),
-                                              JSG_C16(-0.28444138169288635f), JSG_C16(-0.18477343022823334f), JSG_C16(-0.09105003625154495f), JSG_C16(0.0f),
-                                              JSG_C16(0.07958029955625534f), JSG_C16(0.16093020141124725f), JSG_C16(0.24611230194568634f), JSG_C16(0.33791524171829224f),
-                                              JSG_C16(0.44070982933044434f), JSG_C16(0.5626170039176941f), JSG_C16(0.7229568362236023f), JSG_C16(1.0f)};
-
 // x fragment of one lane for one step: VEC activations
 template <typename AT, int VEC> struct XFrag;
 template <int VEC> struct XFrag<_Float16, VEC> {

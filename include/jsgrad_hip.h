@@ -79,7 +79,7 @@ int jsgrad_hip_event_destroy(void *event);
 /* Per-kernel statistics (DEBUG>=2 of engine/realize.ts:168-178; ProfileRangeEvent, runtime/allocator.ts:147-151):
  * while enabled, every Llama kernel launched outside a graph capture is bracketed by an event pair.  `read` waits
  * for the stream and returns launch count and summed milliseconds of one kind since profiling was enabled. */
-enum { JSGRAD_PROF_EMBED = 0, JSGRAD_PROF_RMSNORM, JSGRAD_PROF_LINEAR, JSGRAD_PROF_QKV_ROPE, JSGRAD_PROF_ATTN, JSGRAD_PROF_FFN_GATE, JSGRAD_PROF_ARGMAX, JSGRAD_PROF_STEP };
+enum { JSGRAD_PROF_EMBED = 0, JSGRAD_PROF_RMSNORM, JSGRAD_PROF_LINEAR, JSGRAD_PROF_QKV_ROPE, JSGRAD_PROF_ATTN, JSGRAD_PROF_FFN_GATE, JSGRAD_PROF_ARGMAX, JSGRAD_PROF_STEP, JSGRAD_PROF_GEMM, JSGRAD_PROF_ATTN_PREFILL };
 int jsgrad_hip_profile(int enable);
 int jsgrad_hip_profile_read(int kind, int *host_out_count, double *host_out_total_ms);
 
@@ -140,6 +140,53 @@ int jsgrad_hip_ffn_gate(int kind, const void *w1, const void *s1, const void *w3
  * increments state[1]; tokens_out != NULL (an int32[tokens_cap] history) also receives the token at
  * tokens_out[old start_pos] when that index is inside it. */
 int jsgrad_hip_argmax(const void *logits, int n, int32_t *state, int32_t *tokens_out, int tokens_cap, int advance, int act);
+
+/* ---------------------------------------------------------------------------------
+ * Several rows at once: batched prefill (S > 1 new positions) and batched decode (B > 1 sequences).
+ *
+ * Transformer.forward with tokens of shape [B, S] (models/llama.ts:201-213): the rows are the B*S positions, row
+ * m = b*S + s sits at position start_pos + s of sequence b.  fp16 activations; fp16, int8 or NF4 weights.  With more
+ * than one row the reference expands the weight over the rows, which realises a quantised weight in fp16 first
+ * (W = RN16(code * scale)); the kernels below reproduce that.  Linear layers run on the matrix cores (MFMA) with
+ * float accumulation.  Output widths must be multiples of 128, in_features multiples of 64.
+ * The KV cache of a layer is [B][max_context][n_kv_heads][head_dim] (models/llama.ts:78-80).
+ * --------------------------------------------------------------------------------- */
+
+/* Embedding.call / Int8Embedding.call (nn/index.ts:607-619, llama3.ts:71-77) for `rows` device token ids. */
+int jsgrad_hip_embed_rows(int kind, const void *table, const void *scale, const int32_t *tokens, int rows, void *out, int dim, int vocab);
+
+/* RMSNorm.call (nn/index.ts:586-588) on every row of x[rows][dim]. */
+int jsgrad_hip_rmsnorm_rows(const void *x, const void *weight, void *y, int rows, int dim, float eps);
+
+/* Linear.call / Int8Linear.call / NF4Linear.call (nn/index.ts:411, llama3.ts:35,91-97) on x[rows][in_f]:
+ * y[rows][out_f] = x . W^T (+ residual[rows][out_f] added after the cast, models/llama.ts:125-126). */
+int jsgrad_hip_gemm(int kind, const void *w, const void *scale, int out_f, int in_f, const void *x, int rows, void *y, const void *residual);
+
+/* wq/wk/wv + apply_rotary_emb + KV-cache assign (models/llama.ts:61-87) for rows = B * seq_len positions starting
+ * at start_pos: q_out[rows][n_heads*head_dim] gets the rotated queries, cache rows [start_pos, start_pos+seq_len) of
+ * every sequence get the rotated keys and the values.  x is the already normed input. */
+int jsgrad_hip_gemm_qkv_rope(int kind, const void *wq, const void *sq, const void *wk, const void *sk, const void *wv, const void *sv, const void *x,
+                             int rows, int seq_len, int start_pos, const void *rope_table, void *q_out, void *cache_k, void *cache_v, int dim,
+                             int n_heads, int n_kv_heads, int head_dim, int max_context);
+
+/* w1, w3 + SwiGLU (FeedForward.call, models/llama.ts:108-110) on the already normed x[rows][dim]:
+ * g[rows][hidden] = silu(w1 x) * (w3 x). */
+int jsgrad_hip_gemm_ffn_gate(int kind, const void *w1, const void *s1, const void *w3, const void *s3, const void *x, int rows, void *g, int dim,
+                             int hidden);
+
+/* repeat_kv + scaled_dot_product_attention with the causal mask triu(start_pos + 1) (models/llama.ts:89-95,208;
+ * tensor.ts:3920-3934): query row s of sequence b sees cache rows [0, start_pos + s].  q / out: [B*seq_len][n_heads*head_dim]. */
+int jsgrad_hip_attn_prefill(const void *q, const void *cache_k, const void *cache_v, void *out, int batch, int seq_len, int start_pos, int n_heads,
+                            int n_kv_heads, int head_dim, int max_context);
+
+/* jsgrad_hip_attn_decode for B sequences that sit at the same position state[1]: q / out are [B][n_heads*head_dim].
+ * workspace: jsgrad_hip_attn_batch_workspace_bytes() bytes, zero-filled once before first use. */
+size_t jsgrad_hip_attn_batch_workspace_bytes(int batch, int n_heads, int n_kv_heads, int head_dim);
+int jsgrad_hip_attn_decode_batch(const void *q, const void *cache_k, const void *cache_v, const int32_t *state, void *out, void *workspace, int batch,
+                                 int n_heads, int n_kv_heads, int head_dim, int max_context);
+
+/* Tensor.argmax (tensor.ts:2314-2320) of every row of logits[rows][n]: tokens_out[rows]. */
+int jsgrad_hip_argmax_rows(const void *logits, int rows, int n, int32_t *tokens_out);
 
 /* ---------------------------------------------------------------------------------
  * The whole decode step as ONE kernel.

@@ -456,6 +456,7 @@ typedef struct {
 
 typedef struct {
   int dim, hidden, n_heads, n_kv_heads, n_layers, vocab, max_context, head_dim, act16;
+  int batched;               /* the call carries several sequences: weights are expanded over the rows even when S == 1 */
   float norm_eps, rope_theta;
   int embed_kind;            /* OR_W_F32 / OR_W_F16 / OR_W_I8 */
   const void *tok_emb;
@@ -501,6 +502,10 @@ void or_model_set_norm(or_model_t *m, int layer, int which, const float *w) {
   if (layer < 0) { m->norm = w; return; }
   if (which == 0) m->layers[layer].attention_norm = w; else m->layers[layer].ffn_norm = w;
 }
+/* Several sequences per call (tokens [B, S], B > 1): every Linear sees more than one input row, so quantised weights
+ * are realised in fp16 first (see or_linear_ex) even for S == 1.  The sequences themselves are independent; the caller
+ * runs them one after the other through or_model_forward with this flag set. */
+void or_model_set_batched(or_model_t *m, int batched) { m->batched = batched; }
 void or_model_set_embedding(or_model_t *m, int kind, const void *table, const void *scale) {
   m->embed_kind = kind; m->tok_emb = table; m->tok_scale = (const uint16_t *)scale;
 }
@@ -529,6 +534,7 @@ static void attention(or_model_t *m, int layer, const float *xn, int S, int star
   const or_layer_t *l = &m->layers[layer];
   const int d = m->dim, H = m->n_heads, KV = m->n_kv_heads, hd = m->head_dim, n_rep = H / KV, act16 = m->act16;
   const int T = start_pos + S;
+  const int mat = S > 1 || m->batched;
   const float scale = (float)(1.0 / sqrt((double)hd));
   float *q = (float *)malloc(sizeof(float) * (size_t)H * hd);
   float *k = (float *)malloc(sizeof(float) * (size_t)KV * hd);
@@ -542,9 +548,9 @@ static void attention(or_model_t *m, int layer, const float *xn, int S, int star
   for (int s = 0; s < S; s++) {
     int pos = start_pos + s;
     for (int i = 0; i < hd; i++) fc[i] = rn_act(m->freqs[(size_t)pos * hd + i], act16); /* llama.ts:205 cast */
-    or_linear_ex(&l->wq, xn + (size_t)s * d, q, act16, S > 1);
-    or_linear_ex(&l->wk, xn + (size_t)s * d, k, act16, S > 1);
-    or_linear_ex(&l->wv, xn + (size_t)s * d, cv + (size_t)pos * KV * hd, act16, S > 1);
+    or_linear_ex(&l->wq, xn + (size_t)s * d, q, act16, mat);
+    or_linear_ex(&l->wk, xn + (size_t)s * d, k, act16, mat);
+    or_linear_ex(&l->wv, xn + (size_t)s * d, cv + (size_t)pos * KV * hd, act16, mat);
     rope_rows(q, H, hd, fc, act16);
     rope_rows(k, KV, hd, fc, act16);
     memcpy(qs + (size_t)s * H * hd, q, sizeof(float) * (size_t)H * hd);
@@ -577,7 +583,7 @@ static void attention(or_model_t *m, int layer, const float *xn, int S, int star
       }
     }
   }
-  for (int s = 0; s < S; s++) or_linear_ex(&l->wo, attn + (size_t)s * H * hd, out + (size_t)s * d, act16, S > 1);
+  for (int s = 0; s < S; s++) or_linear_ex(&l->wo, attn + (size_t)s * H * hd, out + (size_t)s * d, act16, mat);
   free(q); free(k); free(attn); free(qs); free(sc); free(fc);
 }
 
@@ -611,13 +617,14 @@ int or_model_forward(or_model_t *m, const int *tokens, int S, int start_pos, flo
     for (long i = 0; i < (long)S * d; i++) h[i] = rn_act(h[i] + t[i], act16);
     for (int s = 0; s < S; s++) {
       or_rmsnorm(h + (size_t)s * d, l->ffn_norm, d, m->norm_eps, act16, xn + (size_t)s * d);
-      feed_forward(m, l, xn + (size_t)s * d, t + (size_t)s * d, S > 1);
+      feed_forward(m, l, xn + (size_t)s * d, t + (size_t)s * d, S > 1 || m->batched);
     }
     for (long i = 0; i < (long)S * d; i++) h[i] = rn_act(h[i] + t[i], act16);
   }
   float *lg = logits ? logits : (float *)malloc(sizeof(float) * (size_t)m->vocab);
   or_rmsnorm(h + (size_t)(S - 1) * d, m->norm, d, m->norm_eps, act16, xn);
-  or_linear(&m->output, xn, lg, act16);
+  /* the lm_head runs on all S rows before the last one is selected (llama.ts:210), so it too sees several rows */
+  or_linear_ex(&m->output, xn, lg, act16, S > 1 || m->batched);
   int tok = or_argmax(lg, m->vocab);
   if (!logits) free(lg);
   free(h); free(xn); free(t);

@@ -55,7 +55,7 @@ def lib() -> C.CDLL:
             "or_rope": ([vp, i32, i32, vp, i32], None),
             "or_argmax": ([vp, i32], i32),
             "or_model_new": ([i32, i32, i32, i32, i32, i32, i32, f32, f32, i32], vp),
-            "or_model_free": ([vp], None), "or_model_reset_cache": ([vp], None),
+            "or_model_free": ([vp], None), "or_model_reset_cache": ([vp], None), "or_model_set_batched": ([vp, C.c_int], None),
             "or_model_set_linear": ([vp, i32, i32, i32, i32, i32, vp, vp], None),
             "or_model_set_norm": ([vp, i32, i32, vp], None),
             "or_model_set_embedding": ([vp, i32, vp, vp], None),
@@ -250,6 +250,10 @@ class OracleModel:
 
     def reset(self):
         lib().or_model_reset_cache(self._m)
+
+    def set_batched(self, batched: bool) -> None:
+        """Treat every forward as one sequence of a batch of several (weights expanded over rows even for S == 1)."""
+        lib().or_model_set_batched(self._m, int(batched))
 
     def forward(self, tokens, start_pos: int, want_logits: bool = True):
         """Transformer.forward on tokens [S] at start_pos -> (greedy token, float32 logits of the last position)."""

@@ -10,6 +10,7 @@ import oracle as orc
 from denograd_amd import ffi
 from denograd_amd.ffi import check
 from denograd_amd.tensor import Tensor
+from tests.helpers import assert_close
 
 pytestmark = pytest.mark.gpu
 RNG = np.random.default_rng(11)
@@ -18,25 +19,6 @@ NPDT = {"float32": np.float32, "float16": np.float16}
 
 def act_code(dt): return ffi.F16 if dt == "float16" else ffi.F32
 def f32(t): return t.numpy().astype(np.float32)
-
-
-def assert_close(got, ref, act16, what="", composed=False):
-    """Two layers: the north-star tolerance (1e-2 of the output scale for fp16 activations, 1e-4 for float32), and the
-    much tighter statement that the two paths differ only by float summation order: at most 2 ulp of the activation
-    dtype (plus float summation noise at the output scale, which matters for results that cancel) and mostly identical values."""
-    got, ref = np.asarray(got, np.float32), np.asarray(ref, np.float32)
-    scale = max(1.0, float(np.abs(ref).max()))
-    assert np.max(np.abs(got - ref)) <= (1e-2 if act16 else 1e-4) * scale, what
-    if act16:
-        ulp = np.spacing(np.abs(ref).astype(np.float16)).astype(np.float32)
-        if composed:   # a fused RMSNorm in front: a few inputs differ by one fp16 ulp, which moves every output a little
-            assert np.all(np.abs(got - ref) <= 4 * ulp + scale * 2.0 ** -11), what
-            assert np.mean(got == ref) > 0.5, what
-        else:
-            assert np.all(np.abs(got - ref) <= 2 * ulp + scale * 2.0 ** -18), what    # + float-sum noise for results that cancel to ~0
-            assert np.mean(got == ref) > 0.9, what
-    else:
-        assert np.all(np.abs(got - ref) <= scale * 2.0 ** (-15 if composed else -18)), what
 
 
 def test_device_is_gfx950(hip):
