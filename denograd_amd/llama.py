@@ -41,10 +41,29 @@ class Attention:
         self.wo = linear(self.n_heads * self.head_dim, dim, False)
         self.cache_kv: Tensor | None = None
 
-    def _ensure_cache(self, dtype: str, device: str) -> None:
-        # Tensor.zeros([2, bsz, max_context, n_kv_heads, head_dim]) (llama.ts:78-80), bsz = 1
-        if self.cache_kv is None:
-            self.cache_kv = Tensor.zeros((2, 1, self.max_context, self.n_kv_heads, self.head_dim), dtype, device)
+    def _ensure_cache(self, dtype: str, device: str, bsz: int = 1) -> None:
+        # Tensor.zeros([2, bsz, max_context, n_kv_heads, head_dim]) (llama.ts:78-80); created for the batch size of the
+        # first call, as in the reference, and recreated (empty) when a call arrives with another batch size
+        if self.cache_kv is None or self.cache_kv.shape[1] != bsz:
+            self.cache_kv = Tensor.zeros((2, bsz, self.max_context, self.n_kv_heads, self.head_dim), dtype, device)
+
+    def call_rows(self, xn: Tensor, bsz: int, seqlen: int, start_pos: int, state: Tensor, freqs_cis: Tensor, rows: "_RowScratch", residual: Tensor, out: Tensor) -> Tensor:
+        """Several positions and/or sequences: xn [bsz*seqlen, dim] is the normed input; out = residual + wo(attention)."""
+        lib = ffi.load()
+        half = self.cache_kv.nbytes // 2
+        ck, cv = self.cache_kv.ptr, self.cache_kv.ptr + half
+        n = bsz * seqlen
+        sp = lambda l: l.scale.ptr if l.scale is not None else None
+        check(lib.jsgrad_hip_gemm_qkv_rope(self.wq.kind, self.wq.weight.ptr, sp(self.wq), self.wk.weight.ptr, sp(self.wk), self.wv.weight.ptr, sp(self.wv),
+                                           xn.ptr, n, seqlen, start_pos, freqs_cis.ptr, rows.q.ptr, ck, cv,
+                                           self.dim, self.n_heads, self.n_kv_heads, self.head_dim, self.max_context))
+        if seqlen == 1:
+            check(lib.jsgrad_hip_attn_decode_batch(rows.q.ptr, ck, cv, state.ptr, rows.attn.ptr, rows.workspace.ptr, bsz,
+                                                   self.n_heads, self.n_kv_heads, self.head_dim, self.max_context))
+        else:
+            check(lib.jsgrad_hip_attn_prefill(rows.q.ptr, ck, cv, rows.attn.ptr, bsz, seqlen, start_pos, self.n_heads, self.n_kv_heads, self.head_dim, self.max_context))
+        check(lib.jsgrad_hip_gemm(self.wo.kind, self.wo.weight.ptr, sp(self.wo), self.dim, self.n_heads * self.head_dim, rows.attn.ptr, n, out.ptr, residual.ptr))
+        return out
 
     def call(self, x: Tensor, state: Tensor, freqs_cis: Tensor, norm: RMSNorm, ctx: "_Scratch") -> Tensor:
         """x: the block input row; returns x + wo(attention(norm(x))) in ctx.h2."""
@@ -76,6 +95,14 @@ class FeedForward:
                                              ctx.g.ptr, self.dim, self.hidden_dim, act_code(x.dtype)))
         return self.w2.call(ctx.g, out=out, residual=x)
 
+    def call_rows(self, xn: Tensor, n: int, rows: "_RowScratch", residual: Tensor, out: Tensor) -> Tensor:
+        """out = residual + w2( silu(w1 xn) * (w3 xn) ) for n rows of normed input."""
+        lib = ffi.load()
+        sp = lambda l: l.scale.ptr if l.scale is not None else None
+        check(lib.jsgrad_hip_gemm_ffn_gate(self.w1.kind, self.w1.weight.ptr, sp(self.w1), self.w3.weight.ptr, sp(self.w3), xn.ptr, n, rows.g.ptr, self.dim, self.hidden_dim))
+        check(lib.jsgrad_hip_gemm(self.w2.kind, self.w2.weight.ptr, sp(self.w2), self.dim, self.hidden_dim, rows.g.ptr, n, out.ptr, residual.ptr))
+        return out
+
 
 class TransformerBlock:
     def __init__(self, dim: int, hidden_dim: int, n_heads: int, n_kv_heads: int | None, norm_eps: float, max_context: int, linear=Linear, feed_forward=FeedForward):
@@ -87,6 +114,14 @@ class TransformerBlock:
     def call(self, x: Tensor, state: Tensor, freqs_cis: Tensor, ctx: "_Scratch") -> Tensor:
         h = self.attention.call(x, state, freqs_cis, self.attention_norm, ctx)     # ctx.h2
         return self.feed_forward.call(h, self.ffn_norm, ctx, out=x)                # back into x
+
+    def call_rows(self, x: Tensor, bsz: int, seqlen: int, start_pos: int, state: Tensor, freqs_cis: Tensor, rows: "_RowScratch") -> Tensor:
+        """TransformerBlock.call (llama.ts:124-127) on x [bsz*seqlen, dim]; the result is written back into x."""
+        lib, n = ffi.load(), bsz * seqlen
+        check(lib.jsgrad_hip_rmsnorm_rows(x.ptr, self.attention_norm.weight.ptr, rows.xn.ptr, n, self.attention.dim, self.attention_norm.eps))
+        h = self.attention.call_rows(rows.xn, bsz, seqlen, start_pos, state, freqs_cis, rows, residual=x, out=rows.h2)
+        check(lib.jsgrad_hip_rmsnorm_rows(h.ptr, self.ffn_norm.weight.ptr, rows.xn.ptr, n, self.attention.dim, self.ffn_norm.eps))
+        return self.feed_forward.call_rows(rows.xn, n, rows, residual=h, out=x)
 
 
 class _Scratch:
@@ -101,6 +136,30 @@ class _Scratch:
         self.logits = Tensor.empty((vocab,), dtype, device)
         nbytes = ffi.load().jsgrad_hip_attn_workspace_bytes(n_heads, n_kv_heads, head_dim)
         self.workspace = Tensor.zeros((nbytes,), "uint8", device)
+
+
+class _RowScratch:
+    """Activations of a several-row call: bsz*seqlen rows (grown on demand, never shrunk)."""
+
+    def __init__(self, bsz: int, seqlen: int, dim: int, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int, vocab: int, device: str):
+        n = bsz * seqlen
+        self.bsz, self.n = bsz, n
+        f16 = "float16"
+        self.tokens = Tensor.empty((n,), "int32", device)
+        self.h = Tensor.empty((n, dim), f16, device)
+        self.h2 = Tensor.empty((n, dim), f16, device)
+        self.xn = Tensor.empty((n, dim), f16, device)
+        self.q = Tensor.empty((n, n_heads * head_dim), f16, device)
+        self.attn = Tensor.empty((n, n_heads * head_dim), f16, device)
+        self.g = Tensor.empty((n, hidden), f16, device)
+        self.last = Tensor.empty((bsz, dim), f16, device)
+        self.logits = Tensor.empty((bsz, vocab), f16, device)
+        self.next_tokens = Tensor.empty((bsz,), "int32", device)
+        nbytes = ffi.load().jsgrad_hip_attn_batch_workspace_bytes(bsz, n_heads, n_kv_heads, head_dim)
+        self.workspace = Tensor.zeros((nbytes,), "uint8", device)
+
+    def fits(self, bsz: int, seqlen: int) -> bool:
+        return bsz == self.bsz and bsz * seqlen <= self.n
 
 
 class _FusedStep:
@@ -203,6 +262,7 @@ class Transformer:
         # False: one launch per fused op (the faster of the two today); True: the whole step as one persistent kernel
         self.fused_step = fused_step
         self._fused: _FusedStep | None = None
+        self._rows: _RowScratch | None = None
 
     # ---- plumbing
     @property
@@ -261,12 +321,95 @@ class Transformer:
             raise NotImplementedError("only greedy decoding (temperature 0 -> argmax, llama.ts:137) is built on this device")
         toks = np.asarray(tokens.numpy() if isinstance(tokens, Tensor) else tokens, np.int32)
         if toks.ndim != 2 or toks.shape[0] != 1:
-            raise ValueError(f"tokens must have shape [1, seqlen], got {toks.shape}")
+            raise ValueError(f"tokens must have shape [1, seqlen], got {toks.shape}; several sequences go through forward_rows")
         ret = None
         for i, t in enumerate(toks[0]):
             self.set_state(int(t), start_pos + i)
             ret = self._step()
         return ret
+
+    def forward_rows(self, tokens, start_pos: int) -> Tensor:
+        """llama.ts:201-213 for tokens of shape [bsz, seqlen] in ONE pass: every Linear is a matrix-core GEMM over all
+        bsz*seqlen rows, attention is causal over cache rows [0, start_pos + s].  Returns the greedy next token of every
+        sequence, an int32 tensor [bsz] (the reference flattens the logits of all sequences into one argmax,
+        llama.ts:212, which is only meaningful for bsz == 1).  fp16 activations; fp16 / int8 / NF4 weights.
+        `tokens` may be a device int32 tensor [bsz, seqlen] (e.g. the tensor a previous call returned, reshaped)."""
+        lib = ffi.load()
+        ctx = self._prepare()
+        if self.dtype != "float16":
+            raise NotImplementedError("several rows at once are built for fp16 activations; float32 models take one position per call")
+        if isinstance(tokens, Tensor):
+            if tokens.dtype != "int32" or len(tokens.shape) not in (1, 2):
+                raise ValueError(f"tokens must be int32 [bsz, seqlen] (or [bsz] for one position each), got {tokens.dtype} {tokens.shape}")
+            bsz, seqlen = tokens.shape if len(tokens.shape) == 2 else (tokens.shape[0], 1)
+            tok_dev = tokens
+        else:
+            toks = np.ascontiguousarray(tokens, np.int32)
+            if toks.ndim != 2:
+                raise ValueError(f"tokens must have shape [bsz, seqlen], got {toks.shape}")
+            if toks.size and (toks.min() < 0 or toks.max() >= self.vocab_size):
+                raise ValueError(f"token outside the vocabulary of {self.vocab_size}")
+            bsz, seqlen = toks.shape
+            tok_dev = None
+        if bsz < 1 or seqlen < 1:
+            raise ValueError(f"empty token tensor {bsz}x{seqlen}")
+        if not (0 <= start_pos and start_pos + seqlen <= self.max_context):
+            raise ValueError(f"positions [{start_pos}, {start_pos + seqlen}) outside the KV cache of {self.max_context} positions")
+        hd = self.dim // self.n_heads
+        if self._rows is None or not self._rows.fits(bsz, seqlen):
+            self._rows = _RowScratch(bsz, seqlen, self.dim, self.hidden_dim, self.n_heads, self.n_kv_heads, hd, self.vocab_size, self.device)
+        rows, n = self._rows, bsz * seqlen
+        if any(layer.attention.cache_kv.shape[1] != bsz for layer in self.layers):
+            for layer in self.layers:
+                layer.attention._ensure_cache(self.dtype, self.device, bsz)
+            if self.forward_jit is not None:
+                self.forward_jit.reset()     # a captured step holds the old cache addresses
+            if self._fused is not None:
+                self._fused = _FusedStep(self, ctx)
+        if tok_dev is None:
+            rows.tokens.lazydata.view(n, "int32", 0).ensure_allocated().copyin(toks.reshape(-1))
+            tok_dev = rows.tokens
+        emb = self.tok_embeddings
+        from .nn import _KIND
+        check(lib.jsgrad_hip_embed_rows(_KIND[emb.weight.dtype], emb.weight.ptr, emb.scale.ptr if emb.scale is not None else None, tok_dev.ptr, n, rows.h.ptr,
+                                        self.dim, self.vocab_size))
+        # the attention of a one-position call reads the position from the device state word, like the one-row kernels
+        self.state.lazydata.ensure_allocated().copyin(np.array([0, start_pos + seqlen - 1], np.int32))
+        h = rows.h
+        for layer in self.layers:
+            h = layer.call_rows(h, bsz, seqlen, start_pos, self.state, self.freqs_cis, rows)
+        # logits of the last position of every sequence (llama.ts:210)
+        if seqlen == 1:
+            last = h
+        else:
+            for b in range(bsz):
+                check(lib.jsgrad_hip_copy(rows.last.ptr + b * self.dim * 2, h.ptr + ((b + 1) * seqlen - 1) * self.dim * 2, self.dim * 2))
+            last = rows.last
+        out = self.output
+        if bsz == 1:
+            # one row: the one-row kernels, which also leave {token, start_pos + seqlen} in the state words so that
+            # single-position decode continues from here
+            if seqlen > 1 and self.vocab_size % 128 == 0 and out.kind != ffi.W_F32:
+                # the reference applies the lm_head to all seqlen rows before selecting the last (llama.ts:210), i.e. with
+                # the weight expanded over rows: the several-row kernel reproduces that arithmetic for the row that is kept
+                check(lib.jsgrad_hip_rmsnorm_rows(last.ptr, self.norm.weight.ptr, rows.xn.ptr, 1, self.dim, self.norm.eps))
+                check(lib.jsgrad_hip_gemm(out.kind, out.weight.ptr, out.scale.ptr if out.scale is not None else None, self.vocab_size, self.dim, rows.xn.ptr, 1,
+                                          ctx.logits.ptr, None))
+            else:
+                out.call(Tensor(buffer=last.lazydata.view(self.dim, "float16", 0), shape=(self.dim,), dtype="float16", device=self.device), out=ctx.logits, norm=self.norm)
+            check(lib.jsgrad_hip_argmax(ctx.logits.ptr, self.vocab_size, self.state.ptr, self.tokens_out.ptr, self.max_context, 1, act_code(self.dtype)))
+            check(lib.jsgrad_hip_copy(rows.next_tokens.ptr, self.state.ptr, 4))
+            self._pos = start_pos + seqlen
+        else:
+            check(lib.jsgrad_hip_rmsnorm_rows(last.ptr, self.norm.weight.ptr, rows.xn.ptr, bsz, self.dim, self.norm.eps))
+            check(lib.jsgrad_hip_gemm(out.kind, out.weight.ptr, out.scale.ptr if out.scale is not None else None, self.vocab_size, self.dim, rows.xn.ptr, bsz,
+                                      rows.logits.ptr, None))
+            check(lib.jsgrad_hip_argmax_rows(rows.logits.ptr, bsz, self.vocab_size, rows.next_tokens.ptr))
+        return Tensor(buffer=rows.next_tokens.lazydata.view(bsz, "int32", 0), shape=(bsz,), dtype="int32", device=self.device)
+
+    def rows_logits(self) -> Tensor:
+        """float16 logits [bsz, vocab] of the last forward_rows call (bsz > 1), or the [vocab] row for bsz == 1."""
+        return self._rows.logits if self._rows is not None and self._rows.bsz > 1 else self._prepare().logits
 
     def call(self, tokens, start_pos: int, temperature: float = 0.0, top_k: int = 0, top_p: float = 0.8, alpha_f: float = 0.0, alpha_p: float = 0.0) -> Tensor:
         """llama.ts:214-220: single-token calls past position 0 go through the jit (a captured graph)."""

@@ -125,6 +125,9 @@ class Llama3:
                                  fused_step=fused_step)
         self.start_pos = 0
         self.last_seen_toks: list[int] = []
+        # False: prompts are fed one token per call, as the reference does (llama3.ts:307-311).  True: the prompt is one
+        # several-position call (matrix-core GEMMs + causal attention), the reference's Transformer.forward on [1, S]
+        self.batched_prefill = False
 
     # ---- loading
     @staticmethod
@@ -198,6 +201,10 @@ class Llama3:
             self.start_pos += i
             self.last_seen_toks = toks
             toks = toks[i:]
+        if self.batched_prefill and len(toks) > 1:
+            self.model.forward_rows(np.array([toks], np.int32), self.start_pos)
+            self.start_pos += len(toks)
+            return
         for tok in toks:
             self._call(tok)
             self.start_pos += 1
@@ -220,6 +227,25 @@ class Llama3:
         dt = time.perf_counter() - st
         return {"tokens": out, "usage": {"input_tokens": len(toks) - 1, "output_tokens": len(out), "time_to_first_token": ttft,
                                           "tokens_per_second": len(out) / dt if dt > 0 else float("inf")}}
+
+    def generate_batch(self, prompts, n_new: int) -> np.ndarray:
+        """Several equally long prompts at once, from position 0: one several-position pass over all prompts, then n_new - 1
+        batched decode steps with the tokens fed back on the device.  Returns int32 [bsz, n_new]."""
+        prompts = np.ascontiguousarray(prompts, np.int32)
+        if prompts.ndim != 2:
+            raise ValueError(f"prompts must have shape [bsz, seqlen], got {prompts.shape}")
+        bsz, seqlen = prompts.shape
+        m = self.model
+        hist = Tensor.empty((n_new, bsz), "int32", self.device)
+        tok = m.forward_rows(prompts, 0)
+        pos = seqlen
+        for i in range(n_new):
+            check(ffi.load().jsgrad_hip_copy(hist.ptr + i * bsz * 4, tok.ptr, bsz * 4))
+            if i + 1 < n_new:
+                tok = m.forward_rows(tok, pos)
+                pos += 1
+        self.start_pos = pos
+        return hist.numpy().T.copy()
 
     def generate(self, prompt, n_new: int) -> np.ndarray:
         """Token-serial prefill, then n_new greedy tokens with the token fed back on the device (no per-token host
