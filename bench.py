@@ -215,6 +215,87 @@ def cpu_baseline(llm, cfg, budget_s=15.0):
             "tokens_identical_to_gpu": f"{same}/{n_new}"}
 
 
+MFMA_PEAK_TFLOPS = 2500.0    # MI355X dense fp16 matrix-core peak
+
+
+def run_batched(name, bsz, prompt_len, steps):
+    """Batched prefill (all prompts in one several-position pass, matrix-core GEMMs + causal attention), then batched
+    greedy decode with the tokens fed back on the device.  Prefill is priced against the fp16 MFMA peak, decode against HBM."""
+    from denograd_amd import ffi, synthetic
+    from denograd_amd.ffi import check
+    from denograd_amd.llama3 import Llama3
+
+    lib = ffi.load()
+    ctx = prompt_len + steps + 8
+    cfg = synthetic.config(name, max_context=ctx)
+    llm = Llama3.from_config(cfg).random_init(seed=0, tied=cfg["tied"])
+    m = llm.model
+    prompts = np.stack([synthetic.random_prompt(cfg, prompt_len, seed=100 + b) for b in range(bsz)]).astype(np.int32)
+    m.forward_rows(prompts[:, :64], 0)                 # allocate caches / scratch, load code objects
+    m.forward_rows(prompts, 0)                          # warm-up pass at full size
+    check(lib.jsgrad_hip_sync())
+
+    def read_kinds():
+        kinds = {}
+        for kname, kid in ffi.PROF_KINDS.items():
+            n, tot = C.c_int(), C.c_double()
+            check(lib.jsgrad_hip_profile_read(kid, C.byref(n), C.byref(tot)))
+            if n.value:
+                kinds[kname] = {"launches": n.value, "ms": round(tot.value, 3)}
+        return kinds
+
+    t0 = time.perf_counter()
+    tok = m.forward_rows(prompts, 0)
+    check(lib.jsgrad_hip_sync())
+    prefill_s = time.perf_counter() - t0
+    check(lib.jsgrad_hip_profile(1))
+    tok = m.forward_rows(prompts, 0)
+    pre_kinds = read_kinds()
+    check(lib.jsgrad_hip_profile(0))
+
+    d, L, H, KV, F, V = cfg["dim"], cfg["n_layers"], cfg["n_heads"], cfg["n_kv_heads"], cfg["hidden_dim"], cfg["vocab_size"]
+    hd = d // H
+    e_l = 2 * d * H * hd + 2 * d * KV * hd + 3 * d * F           # linear elements per layer
+    rows = bsz * prompt_len
+    lin_flop = 2.0 * L * e_l * rows + 2.0 * V * d * bsz           # lm_head on the last position only
+    att_flop = 2.0 * prompt_len * prompt_len * H * hd * L * bsz  # causal: QK^T + PV over the lower triangle
+    gemm_ms = pre_kinds.get("gemm", {}).get("ms", 0.0)
+    prefill = {"tok_s": round(rows / prefill_s, 1), "seconds": round(prefill_s, 4), "tokens": rows,
+               "flop": lin_flop + att_flop, "tflops": round((lin_flop + att_flop) / prefill_s / 1e12, 1),
+               "roofline": {"bound": "mfma", "kernel": "gemm_kernel (all Linear layers of the pass)", "achieved": round(lin_flop / (gemm_ms * 1e-3) / 1e12, 1) if gemm_ms else None,
+                            "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(lin_flop / (gemm_ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4) if gemm_ms else None,
+                            "traffic": None},
+               "kernels": pre_kinds}
+
+    # batched decode: one position per sequence per step
+    pos = prompt_len
+    for _ in range(4):
+        tok = m.forward_rows(tok, pos); pos += 1
+    check(lib.jsgrad_hip_sync())
+    t0 = time.perf_counter()
+    for _ in range(steps - 4 - 4):
+        tok = m.forward_rows(tok, pos); pos += 1
+    check(lib.jsgrad_hip_sync())
+    dec_s = time.perf_counter() - t0
+    n_dec = steps - 8
+    check(lib.jsgrad_hip_profile(1))
+    for _ in range(4):
+        tok = m.forward_rows(tok, pos); pos += 1
+    dec_kinds = read_kinds()
+    check(lib.jsgrad_hip_profile(0))
+    t_avg = prompt_len + 4 + n_dec / 2.0
+    bytes_step = synthetic.weight_bytes_per_token(cfg) + bsz * synthetic.kv_bytes_per_position(cfg) * t_avg
+    gpu_ms = sum(v["ms"] for v in dec_kinds.values()) / 4
+    decode = {"tok_s": round(bsz * n_dec / dec_s, 1), "steps_s": round(n_dec / dec_s, 2), "ms_per_step": round(1e3 * dec_s / n_dec, 4),
+              "kernel_ms_per_step": round(gpu_ms, 4), "bytes_per_step": int(bytes_step),
+              "roofline": {"bound": "hbm", "achieved": round(bytes_step * n_dec / dec_s / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": round(bytes_step * n_dec / dec_s / 1e9 / HBM_PEAK_GBS, 4)},
+              "kernels": {k: {"launches_per_step": v["launches"] // 4, "ms_per_step": round(v["ms"] / 4, 4)} for k, v in dec_kinds.items()}}
+    return {"config": {"workload": f"Llama-3 {name}-shaped random init ({cfg['quantize']}), {bsz} sequences x {prompt_len}-token prompts in one pass, "
+                                   f"then {steps} batched greedy steps", "batch": bsz, "prompt": prompt_len, "decode": steps, "max_context": ctx},
+            "prefill": prefill, "decode": decode}
+
+
 def traffic_probe(name):
     from denograd_amd import ffi, synthetic
     from denograd_amd.ffi import check
@@ -244,6 +325,10 @@ def main():
     ap.add_argument("--workload", default="1B", help="primary synthetic config (denograd_amd/synthetic.py)")
     ap.add_argument("--secondary", default="8B-int8", help="second workload measured in the same run ('' to skip)")
     ap.add_argument("--secondary-steps", type=int, default=128)
+    ap.add_argument("--batched", default="8B-int8", help="workload of the batched prefill + batched decode leg ('' to skip)")
+    ap.add_argument("--batch", type=int, default=16)
+    ap.add_argument("--batch-prompt", type=int, default=2048)
+    ap.add_argument("--batch-steps", type=int, default=128)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle baseline")
     ap.add_argument("--traffic-probe", action="store_true", help="for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: one 512 MiB device-to-device copy "
                     "(a plain copy kernel of known size, to scale the counters) followed by 4 eager decode steps of --workload; prints nothing")
@@ -284,6 +369,8 @@ def main():
         out["secondary"] = {"value": round(secondary["tok_s"], 2), "unit": "tok/s", "steps": args.secondary_steps, "ms_per_step": round(secondary["ms_per_step"], 4),
                             "dtype": "i8 weights, f16 activations", "config": secondary["config"], "roofline": secondary["roofline"],
                             "step_roofline": secondary["step_roofline"], "kernels": secondary["kernels"], "per_op_path": secondary.get("per_op_path")}
+    if args.batched:
+        out["batched"] = run_batched(args.batched, args.batch, args.batch_prompt, args.batch_steps)
     print(json.dumps(out), flush=True)
 
 

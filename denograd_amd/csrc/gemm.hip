@@ -13,6 +13,8 @@
 // spreads the 32 rows of a fragment read over all banks.  One LDS buffer, register prefetch of the next K tile issued
 // before the MFMAs of the current one.  Tile ids are remapped so that the blocks resident on one XCD (round-robin by
 // block id) share operand tiles in that XCD's L2.
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace jsg {
@@ -55,7 +57,7 @@ __device__ __forceinline__ void i8x4_to_h2x2(uint32_t q, uint32_t &lo, uint32_t 
 }
 
 template <int KIND, int EPI, int WGM, int WGN, int TM, int TN>
-__global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(GemmArgs a) {
+__global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 : 3))) void gemm_kernel(GemmArgs a) {
   static_assert(WGM * WGN == 4, "four wavefronts");
   static_assert(EPI != GEPI_SWIGLU || TN % 2 == 0, "a wavefront holds the w1 and the w3 tile of the same columns");
   constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32, LS = GEMM_LDS_STRIDE;
@@ -64,9 +66,8 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(GemmArgs a) {
   constexpr int B_CHUNKS = GEMM_THREADS / B_ROWS_PER_PASS;                             // 16-byte chunks per row of the K tile
   constexpr int B_LOADS = BN / B_ROWS_PER_PASS;
   static_assert(B_LOADS >= 1, "tile too narrow for this weight format");
-  __shared__ __align__(16) _Float16 As[BM * LS];
-  __shared__ __align__(16) _Float16 Bs[BN * LS];
-  __shared__ _Float16 lut[16];
+  extern __shared__ __align__(16) _Float16 gemm_lds[];   // [BM + BN rows][LS], then the 16-entry NF4 table
+  _Float16 *As = gemm_lds, *Bs = gemm_lds + BM * LS, *lut = gemm_lds + (BM + BN) * LS;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WGN, wn = wave % WGN;
@@ -280,15 +281,28 @@ template <int KIND, int EPI, int WGM, int WGN, int TM, int TN> static int launch
   constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
   const int out_per_tile = EPI == GEPI_SWIGLU ? BN / 2 : BN;
   const int tiles = ((a.M + BM - 1) / BM) * (a.N / out_per_tile);
-  JSG_LAUNCH(prof_kind, (gemm_kernel<KIND, EPI, WGM, WGN, TM, TN>), dim3(tiles), dim3(GEMM_THREADS), 0, a);
+  constexpr size_t lds = (size_t)(BM + BN) * GEMM_LDS_STRIDE * sizeof(_Float16) + 32;
+  if constexpr (lds > 64 * 1024) {
+    static bool raised = false;   // one process, one device, one thread: set once per instantiation
+    if (!raised) {
+      JSG_HIP(hipFuncSetAttribute((const void *)gemm_kernel<KIND, EPI, WGM, WGN, TM, TN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      raised = true;
+    }
+  }
+  JSG_LAUNCH(prof_kind, (gemm_kernel<KIND, EPI, WGM, WGN, TM, TN>), dim3(tiles), dim3(GEMM_THREADS), lds, a);
   return 0;
 }
 
 template <int EPI> static int dispatch_gemm(int kind, const GemmArgs &a, int prof_kind) {
-  // tall inputs: 256x128 block tiles; short ones (batched decode): 32 rows x 128 columns per block
+  // tall inputs: 256x256 block tiles when the output is wide enough, else 256x128; short ones (batched decode): 32 rows
+  // x 128 columns per block
   const bool tall = a.M > 64;
+  const int n_out = EPI == GEPI_SWIGLU ? 2 * a.N : a.N;
+  const bool wide = tall && getenv("JSG_GEMM_WIDE") && n_out % 256 == 0 && EPI != GEPI_ROPE_KV;
 #define JSG_CASE(K)                                                                                                    \
   case K:                                                                                                              \
+    if (wide) return launch_gemm<K, EPI, 2, 2, 4, 4>(a, prof_kind);                                                   \
+    if (tall && getenv("JSG_GEMM_SMALL")) return launch_gemm<K, EPI, 2, 2, 2, 2>(a, prof_kind);                       \
     return tall ? launch_gemm<K, EPI, 2, 2, 4, 2>(a, prof_kind) : launch_gemm<K, EPI, 1, 4, 1, EPI == GEPI_SWIGLU ? 2 : 1>(a, prof_kind);
   switch (kind) {
     JSG_CASE(JSGRAD_W_F16)
