@@ -80,6 +80,10 @@ __device__ __forceinline__ void grid_barrier(const StepArgs &s, int &epoch) {
   barrier_wait(s, epoch);
 }
 
+#ifndef JSG_STEP_TOUCH
+#define JSG_STEP_TOUCH 0
+#endif
+
 template <int KIND, int HD, int NREP>
 __global__ __launch_bounds__(STEP_THREADS) void decode_step_kernel(StepArgs s) {
   typedef _Float16 AT;
@@ -128,6 +132,11 @@ __global__ __launch_bounds__(STEP_THREADS) void decode_step_kernel(StepArgs s) {
     return a;
   };
 
+  // Lines of the next phase's weights beyond the one prefetched item are pulled into L2 while the block waits at a
+  // barrier or works through attention (TOUCH items per wavefront; 0 switches it off).
+  constexpr int TOUCH = JSG_STEP_TOUCH;
+  uint32_t tw[TOUCH > 0 ? TOUCH : 1], sink = 0;
+
   // first weights of layer 0 go out before anything else
   GemvBuf pre;   // the one buffer that carries the next phase's first item across a barrier
   if (s.n_layers > 0) GQ::prefetch(qkv_args(s.layers[0]), pre, pos);
@@ -151,7 +160,9 @@ __global__ __launch_bounds__(STEP_THREADS) void decode_step_kernel(StepArgs s) {
     const GemvArgs awo = lin_args(L.wo, L.so, s.dim, s.n_heads * HD, s.attn, s.h2, nullptr, s.h, 0.0f);
     barrier_arrive(s, epoch);
     GL::prefetch(awo, pre, pos);
+    if constexpr (TOUCH > 0) GL::template touch<TOUCH>(awo, 1, tw);
     barrier_wait(s, epoch);
+    if constexpr (TOUCH > 0) GL::template touch_wait<TOUCH>(tw, sink);
     stamp();
 
     // attention over cache rows [0, pos]: items (kv head, chunk) spread over the blocks
@@ -181,7 +192,9 @@ __global__ __launch_bounds__(STEP_THREADS) void decode_step_kernel(StepArgs s) {
     stamp();
     barrier_arrive(s, epoch);
     GF::prefetch(ffn_args(L), pre, pos);
+    if constexpr (TOUCH > 0) GF::template touch<TOUCH>(ffn_args(L), 1, tw);
     barrier_wait(s, epoch);
+    if constexpr (TOUCH > 0) GF::template touch_wait<TOUCH>(tw, sink);
     stamp();
 
     // ffn_norm + w1/w3 + SwiGLU -> g
@@ -190,16 +203,25 @@ __global__ __launch_bounds__(STEP_THREADS) void decode_step_kernel(StepArgs s) {
     const GemvArgs aw2 = lin_args(L.w2, L.s2, s.dim, s.hidden, s.g, s.h, nullptr, s.h2, 0.0f);
     barrier_arrive(s, epoch);
     GL::prefetch(aw2, pre, pos);
+    if constexpr (TOUCH > 0) GL::template touch<TOUCH>(aw2, 1, tw);
     barrier_wait(s, epoch);
+    if constexpr (TOUCH > 0) GL::template touch_wait<TOUCH>(tw, sink);
     stamp();
 
     // w2 + residual -> h
     GL::run(aw2, xs, red, lut, pre, true, pos);
     stamp();
     barrier_arrive(s, epoch);
-    if (l + 1 < s.n_layers) GQ::prefetch(qkv_args(s.layers[l + 1]), pre, pos);
-    else GL::prefetch(lin_args(s.out_w, s.out_s, s.vocab, s.dim, s.h, s.logits, s.final_norm, nullptr, inv_dim), pre, pos);
+    if (l + 1 < s.n_layers) {
+      GQ::prefetch(qkv_args(s.layers[l + 1]), pre, pos);
+      if constexpr (TOUCH > 0) GQ::template touch<TOUCH>(qkv_args(s.layers[l + 1]), 1, tw);
+    } else {
+      const GemvArgs alm = lin_args(s.out_w, s.out_s, s.vocab, s.dim, s.h, s.logits, s.final_norm, nullptr, inv_dim);
+      GL::prefetch(alm, pre, pos);
+      if constexpr (TOUCH > 0) GL::template touch<TOUCH>(alm, 1, tw);
+    }
     barrier_wait(s, epoch);
+    if constexpr (TOUCH > 0) GL::template touch_wait<TOUCH>(tw, sink);
     stamp();
   }
 
@@ -238,6 +260,8 @@ __global__ __launch_bounds__(STEP_THREADS) void decode_step_kernel(StepArgs s) {
       }
     }
   }
+
+  if (s.n_layers < 0) st_coherent(s.err, (int)sink);   // never taken (the host checks n_layers): keeps the touched words alive
 
   // ---- leave the barrier words at zero for the next launch: the last block out clears them
   if (tid == 0) {

@@ -1,4 +1,6 @@
 // Stand-alone one-row linear kernels: one launch per Linear / fused group of Linears (see gemv_core.h).
+#include <stdlib.h>
+
 #include "gemv_core.h"
 
 namespace jsg {
@@ -22,9 +24,10 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL> static int launc
   constexpr int NW = 4;
   const int ngroups = (total_rows + ROWS - 1) / ROWS;
   const int need = (ngroups + NW - 1) / NW;      // one group per wavefront
-  const int cap = state().cu_count * 4;          // 16 resident wavefronts per CU; more rows than that are walked grid-stride
+  static const int per_cu = getenv("JSG_GEMV_BLOCKS_PER_CU") ? atoi(getenv("JSG_GEMV_BLOCKS_PER_CU")) : 4;
+  const int cap = state().cu_count * per_cu;      // 16 resident wavefronts per CU; more rows than that are walked grid-stride
   dim3 grid(need < cap ? need : cap), block(NW * 64);
-  size_t lds = (size_t)a.in_f * sizeof(AT);
+  size_t lds = (size_t)Gemv<KIND, AT, EPI, ROWS, UNROLL, false>::x_elems(a.in_f) * sizeof(AT);
   JSG_LAUNCH(kind, (gemv_kernel<KIND, AT, EPI, ROWS, UNROLL>), grid, block, lds, a);
   return 0;
 }

@@ -140,8 +140,11 @@ template <> struct Dot<JSGRAD_W_I8, _Float16> {
 // norm the chunks stay in registers between the sum of squares and the scaling, so x is read from memory once and
 // the whole prologue costs one round of loads and two barriers.  Ends with a barrier.
 // COHERENT: x was written by other blocks of the same launch, so it is read at the device-wide coherence point.
-template <typename AT, bool COHERENT> __device__ __forceinline__ void stage_x(const GemvArgs &a, AT *xs, float *red) {
+// `padded` >= in_f (a multiple of the 16-byte chunk): LDS elements [in_f, padded) are set to zero, so that a k-step
+// that reaches past in_f multiplies whatever weights it loaded by zero.
+template <typename AT, bool COHERENT> __device__ __forceinline__ void stage_x(const GemvArgs &a, AT *xs, float *red, int padded) {
   constexpr int EPC = 16 / sizeof(AT);  // elements per 16-byte chunk
+  for (int c = a.in_f / EPC + threadIdx.x; c < padded / EPC; c += blockDim.x) ((u4_t *)xs)[c] = u4_t{0, 0, 0, 0};
   constexpr int MAXCH = 4;              // chunks a thread keeps in registers on the norm path (host checks the size)
   const int n = a.in_f, tid = threadIdx.x, nt = blockDim.x;
   const int nchunks = n / EPC;          // in_f is a multiple of EPC (checked on the host)
@@ -224,10 +227,19 @@ template <typename AT, bool COHERENT> __device__ __forceinline__ void stage_x(co
 // Every configuration in use moves 8 x 16 bytes per lane and item (UNROLL x NM x ROWS = 8) and has ROWS = 2, so one
 // plain struct serves all of them; the whole-step kernel can then carry ONE prefetched buffer from phase to phase.
 struct GemvBuf {
-  u4_t w[8];       // [u][j][r] flattened
-  float scale[4];  // [j][r] flattened
-  float extra[2];  // EPI_STORE: residual[row]; EPI_ROPE_KV: (cos, sin) of the rotary pair
+  u4_t w[8];            // [u][j][r] flattened
+  // Small per-row operands, kept exactly as the loads returned them (16-bit loads stay 16-bit values) and converted
+  // where they are used: any arithmetic at load time, even a zero-extension, waits for the load, and loads complete in
+  // order, so it would wait for the weight vectors issued before it as well.
+  _Float16 scale[4];    // [j][r] flattened: the int8 row scale
+  _Float16 extra_h[2];  // fp16 activations - EPI_STORE: residual[row]; EPI_ROPE_KV: cos or sin of the rotary pair
+  float extra_f[2];     // the same for float32 activations
 };
+template <typename AT> __device__ __forceinline__ float extra_of(const GemvBuf &b, int r);
+template <> __device__ __forceinline__ float extra_of<float>(const GemvBuf &b, int r) { return b.extra_f[r]; }
+template <> __device__ __forceinline__ float extra_of<_Float16>(const GemvBuf &b, int r) { return (float)b.extra_h[r]; }
+__device__ __forceinline__ void set_extra(GemvBuf &b, int r, float v) { b.extra_f[r] = v; }
+__device__ __forceinline__ void set_extra(GemvBuf &b, int r, _Float16 v) { b.extra_h[r] = v; }
 
 // The GEMV of one launch (or of one phase of the whole-step kernel).  A block stages x once, then its wavefronts walk
 // row groups (ROWS consecutive output rows of the NM matrices that share x) grid-stride.  A wavefront's work is the flat
@@ -268,6 +280,8 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
     return ((EPI == EPI_SWIGLU ? a.rows0 : a.rows0 + a.rows1 + a.rows2) + ROWS - 1) / ROWS;
   }
   __device__ static __forceinline__ int nbatch(const GemvArgs &a) { return ((a.in_f + STEP - 1) / STEP + UNROLL - 1) / UNROLL; }
+  // LDS elements the staged x needs: in_f rounded up to whole batches (host side)
+  static int x_elems(int in_f) { return (((in_f + STEP - 1) / STEP + UNROLL - 1) / UNROLL) * UNROLL * STEP; }
 
   // issue the loads of item (grp, b)
   __device__ static __forceinline__ void load_item(const GemvArgs &a, Buf &buf, int grp, int b, int pos) {
@@ -275,17 +289,18 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
     const Where w = locate(a, grp);
 #pragma unroll
     for (int u = 0; u < UNROLL; u++) {
-      const int k = (b * UNROLL + u) * STEP + lane * VEC;
-      if (k < in_f) {
+      // Lanes past the end of the row reload its last vector instead of branching around the load (their x is zero,
+      // see stage_x): a load under a lane mask makes the compiler wait for every outstanding load at the join.
+      int k = (b * UNROLL + u) * STEP + lane * VEC;
+      k = k < in_f ? k : in_f - VEC;
 #pragma unroll
-        for (int j = 0; j < NM; j++)
+      for (int j = 0; j < NM; j++)
 #pragma unroll
-          for (int r = 0; r < ROWS; r++) {
-            const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;  // tail rows reload the last row, never stored
-            const char *p = (const char *)wbase(a, w.m, j) + (((size_t)row * in_f + (size_t)k) * BITS) / 8;
-            buf.w[wi(u, j, r)] = __builtin_nontemporal_load((const u4_t *)p);
-          }
-      }
+        for (int r = 0; r < ROWS; r++) {
+          const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;  // tail rows reload the last row, never stored
+          const char *p = (const char *)wbase(a, w.m, j) + (((size_t)row * in_f + (size_t)k) * BITS) / 8;
+          buf.w[wi(u, j, r)] = __builtin_nontemporal_load((const u4_t *)p);
+        }
     }
     if (b != nbatch(a) - 1) return;
 #pragma unroll
@@ -293,18 +308,20 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
       const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;
       if constexpr (KIND == JSGRAD_W_I8) {
 #pragma unroll
-        for (int j = 0; j < NM; j++) buf.scale[si(j, r)] = (float)((const _Float16 *)sbase(a, w.m, j))[row];
+        for (int j = 0; j < NM; j++) buf.scale[si(j, r)] = ((const _Float16 *)sbase(a, w.m, j))[row];
       }
       if constexpr (EPI == EPI_STORE) {
-        const AT *res = (const AT *)a.residual;
-        if (res == nullptr) buf.extra[r] = 0.0f;
-        else if constexpr (COHERENT) buf.extra[r] = (float)ld_coherent(res + row);
-        else buf.extra[r] = (float)res[row];
+        // no residual: read element 0 of x instead (always readable; the value is not used), so that there is one
+        // straight-line load here and no branch for the register allocator to merge
+        const uintptr_t has = a.residual != nullptr;
+        const AT *res = (const AT *)((uintptr_t)a.residual * has + (uintptr_t)a.x * (1 - has)) + (size_t)row * has;
+        if constexpr (COHERENT) set_extra(buf, r, ld_coherent(res));
+        else set_extra(buf, r, *res);
       } else if constexpr (EPI == EPI_ROPE_KV) {
         // table row `pos`, entry (cos, sin) of pair i = (row % head_dim) / 2: even r gets cos, odd r gets sin
         const bool ok = pos >= 0 && pos < a.max_context;
         const int i = (row % a.head_dim) >> 1;
-        buf.extra[r] = ok ? (float)((const AT *)a.rope_table)[(size_t)pos * a.head_dim + 2 * i + (r & 1)] : 0.0f;
+        set_extra(buf, r, ((const AT *)a.rope_table)[ok ? (size_t)pos * a.head_dim + 2 * i + (r & 1) : 0]);
       }
     }
   }
@@ -313,6 +330,40 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
   __device__ static __forceinline__ void prefetch(const GemvArgs &a, Buf &buf, int pos) {
     const int grp = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (grp < ngroups(a)) load_item(a, buf, grp, 0, pos);
+  }
+
+  // Ask for one dword of every 128-byte line of items [first, first + DEPTH) of this wavefront's sequence without
+  // waiting for it, so that the lines sit in this XCD's L2 when load_item() wants them (item 0 is what prefetch()
+  // loads).  One load instruction covers one item: 8 vectors x 8 lines = 64 lanes.  The loads are issued from inline
+  // assembly, so the compiler does not know they are in flight: the caller must run touch_wait() before it reads t[].
+  template <int DEPTH> __device__ static __forceinline__ void touch(const GemvArgs &a, int first, uint32_t (&t)[DEPTH]) {
+    const int lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+    const int ng = ngroups(a), nb = nbatch(a), gstride = gridDim.x * nw;
+    int grp = blockIdx.x * nw + (threadIdx.x >> 6), b = 0;
+    const int v = lane >> 3, line = lane & 7;
+    const int u = v / (NM * ROWS), j = (v / ROWS) % NM, r = v % ROWS;
+    for (int i = 0; i < first; i++)
+      if (++b == nb) { b = 0; grp += gstride; }
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) {
+      t[d] = 0;
+      if (grp < ng) {
+        const Where w = locate(a, grp);
+        const int k = (b * UNROLL + u) * STEP + line * (1024 / BITS);   // first element of this lane's 128-byte line
+        if (k < a.in_f) {
+          const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;
+          const char *p = (const char *)wbase(a, w.m, j) + (((size_t)row * a.in_f + (size_t)k) * BITS) / 8;
+          asm volatile("global_load_dword %0, %1, off" : "=v"(t[d]) : "v"(p) : "memory");
+        }
+      }
+      if (++b == nb) { b = 0; grp += gstride; }
+    }
+  }
+  // wait for every outstanding load of this wavefront (touch() loads included) and fold the touched words into `sink`
+  template <int DEPTH> __device__ static __forceinline__ void touch_wait(uint32_t (&t)[DEPTH], uint32_t &sink) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) sink ^= t[d];
   }
 
   __device__ static __forceinline__ void store_out(AT *p, float v) {
@@ -332,22 +383,21 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; u++) {
-      const int k = (b * UNROLL + u) * STEP + lane * VEC;
-      if (k < in_f) {
-        XFrag<AT, VEC> xf;
-        xf.load(xs + k);
+      const int k = (b * UNROLL + u) * STEP + lane * VEC;   // may lie in the zero padding of xs
+      XFrag<AT, VEC> xf;
+      xf.load(xs + k);
 #pragma unroll
-        for (int j = 0; j < NM; j++)
+      for (int j = 0; j < NM; j++)
 #pragma unroll
-          for (int r = 0; r < ROWS; r++) {
-            float bs = 1.0f;
-            if constexpr (KIND == JSGRAD_W_NF4) {
-              const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;
-              bs = (float)((const _Float16 *)sbase(a, w.m, j))[((size_t)row * in_f + k) >> 6];
-            }
-            acc[j][r] = Dot<KIND, AT>::run(buf.w[wi(u, j, r)], xf, acc[j][r], bs, lut);
+        for (int r = 0; r < ROWS; r++) {
+          float bs = 1.0f;
+          if constexpr (KIND == JSGRAD_W_NF4) {
+            const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;
+            const int kc = k < in_f ? k : in_f - VEC;
+            bs = (float)((const _Float16 *)sbase(a, w.m, j))[((size_t)row * in_f + kc) >> 6];
           }
-      }
+          acc[j][r] = Dot<KIND, AT>::run(buf.w[wi(u, j, r)], xf, acc[j][r], bs, lut);
+        }
     }
     if (b != nbatch(a) - 1) return;
 
@@ -357,7 +407,7 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
 #pragma unroll
       for (int r = 0; r < ROWS; r++) {
         float v = wave_sum(acc[j][r]);
-        if constexpr (KIND == JSGRAD_W_I8) v = v * buf.scale[si(j, r)];
+        if constexpr (KIND == JSGRAD_W_I8) v = v * (float)buf.scale[si(j, r)];
         val[j][r] = Act<AT>::rn(v);
       }
     const int r0 = w.r0, mrows = w.mrows;
@@ -368,7 +418,7 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
       for (int r = 0; r < ROWS; r++)
         if (lane == r && r0 + r < mrows) {
           float v = val[0][r];
-          if (has_res) v = Act<AT>::rn(buf.extra[r] + v);
+          if (has_res) v = Act<AT>::rn(extra_of<AT>(buf, r) + v);
           store_out(y + r0 + r, v);
         }
     } else if constexpr (EPI == EPI_SWIGLU) {
@@ -388,7 +438,7 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
 #pragma unroll
         for (int r = 0; r < ROWS; r += 2)
           if (lane == r && r0 + r + 1 < mrows) {
-            const float c = buf.extra[r], d = buf.extra[r + 1];
+            const float c = extra_of<AT>(buf, r), d = extra_of<AT>(buf, r + 1);
             const float av = val[0][r], bv = val[0][r + 1];
             store_out(dst + r0 + r, Act<AT>::rn(av * c - bv * d));  // the build keeps a*b+c unfused: two roundings as in plain C
             store_out(dst + r0 + r + 1, Act<AT>::rn(av * d + bv * c));
@@ -404,25 +454,29 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
     if (KIND == JSGRAD_W_NF4 && threadIdx.x < 16) lut[threadIdx.x] = NF4_CODE[threadIdx.x];
     int grp = blockIdx.x * nw + wave, b = 0;
     if (!preloaded && grp < ng) load_item(a, bufA, grp, 0, pos);
-
-    stage_x<AT, COHERENT>(a, xs, red);  // block-wide, ends with a barrier (which also publishes lut)
-
-    float acc[NM][ROWS];
-    Buf bufB;
     auto advance = [&](int &g, int &bb) {
       if (++bb == nb) { bb = 0; g += gstride; }
     };
+    // the second item goes out before x is staged too: staging (a read of x, the RMSNorm reduction, a block barrier)
+    // would otherwise be a stretch with nothing new in flight
+    Buf bufB;
+    int gB = grp, bB = b;
+    advance(gB, bB);
+    if (gB < ng) load_item(a, bufB, gB, bB, pos);
+
+    stage_x<AT, COHERENT>(a, xs, red, nb * UNROLL * STEP);  // block-wide, ends with a barrier (which also publishes lut)
+
+    float acc[NM][ROWS];
     while (grp < ng) {
-      int g1 = grp, b1 = b;
-      advance(g1, b1);
-      if (g1 < ng) load_item(a, bufB, g1, b1, pos);
       use_item(a, bufA, grp, b, acc, xs, lut, pos);
-      if (g1 >= ng) break;
-      grp = g1; b = b1;
-      advance(g1, b1);
-      if (g1 < ng) load_item(a, bufA, g1, b1, pos);
-      use_item(a, bufB, grp, b, acc, xs, lut, pos);
-      grp = g1; b = b1;
+      if (gB >= ng) break;
+      grp = gB; b = bB;
+      advance(grp, b);                                   // the item after B goes into A
+      if (grp < ng) load_item(a, bufA, grp, b, pos);
+      use_item(a, bufB, gB, bB, acc, xs, lut, pos);
+      gB = grp; bB = b;
+      advance(gB, bB);                                   // and the one after that into B
+      if (grp < ng && gB < ng) load_item(a, bufB, gB, bB, pos);
     }
   }
 };
