@@ -91,16 +91,26 @@ template <> struct Act<_Float16> {
 // coherence point rather than from a per-XCD L2 copy.  A block publishes by: coherent stores -> __syncthreads (which
 // waits for the stores to be acknowledged) -> one relaxed agent-scope atomic on a counter.  A full release/acquire
 // fence would write back and invalidate the whole L2 of the XCD once per block, which costs far more than the kernel.
-__device__ __forceinline__ void st_coherent(float *p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-__device__ __forceinline__ void st_coherent(int *p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+// Pointers that were loaded from memory (a table of layer tensors) or built with integer arithmetic are generic to the
+// compiler, which then emits flat_* instructions: those count against the LDS counter as well as the vector-memory one,
+// so every LDS wait also waits for them.  Everything below the C ABI is device memory: say so.
+#define JSG_GLOBAL __attribute__((address_space(1)))
+template <typename T> __device__ __forceinline__ const JSG_GLOBAL T *as_global(const void *p) { return (const JSG_GLOBAL T *)(uintptr_t)p; }
+template <typename T> __device__ __forceinline__ JSG_GLOBAL T *as_global_mut(void *p) { return (JSG_GLOBAL T *)(uintptr_t)p; }
+// 16 bytes that are read once: streamed past the caches
+__device__ __forceinline__ u4_t ldg_stream16(const void *p) { return __builtin_nontemporal_load(as_global<u4_t>(p)); }
+template <typename T> __device__ __forceinline__ T ldg(const T *p) { return *as_global<T>(p); }
+
+__device__ __forceinline__ void st_coherent(float *p, float v) { __hip_atomic_store(as_global_mut<float>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void st_coherent(int *p, int v) { __hip_atomic_store(as_global_mut<int>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void st_coherent(_Float16 *p, _Float16 v) {
-  __hip_atomic_store((uint16_t *)p, __builtin_bit_cast(uint16_t, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(as_global_mut<uint16_t>(p), __builtin_bit_cast(uint16_t, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ _Float16 ld_coherent(const _Float16 *p) {
-  return __builtin_bit_cast(_Float16, __hip_atomic_load((const uint16_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+  return __builtin_bit_cast(_Float16, __hip_atomic_load(as_global<uint16_t>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
 }
-__device__ __forceinline__ float ld_coherent(const float *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-__device__ __forceinline__ int ld_coherent(const int *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ float ld_coherent(const float *p) { return __hip_atomic_load(as_global<float>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ int ld_coherent(const int *p) { return __hip_atomic_load(as_global<int>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
 // DPP cross-lane moves inside a 64-lane wavefront
 template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {

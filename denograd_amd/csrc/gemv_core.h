@@ -299,7 +299,7 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
         for (int r = 0; r < ROWS; r++) {
           const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;  // tail rows reload the last row, never stored
           const char *p = (const char *)wbase(a, w.m, j) + (((size_t)row * in_f + (size_t)k) * BITS) / 8;
-          buf.w[wi(u, j, r)] = __builtin_nontemporal_load((const u4_t *)p);
+          buf.w[wi(u, j, r)] = ldg_stream16(p);
         }
     }
     if (b != nbatch(a) - 1) return;
@@ -308,7 +308,7 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
       const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;
       if constexpr (KIND == JSGRAD_W_I8) {
 #pragma unroll
-        for (int j = 0; j < NM; j++) buf.scale[si(j, r)] = ((const _Float16 *)sbase(a, w.m, j))[row];
+        for (int j = 0; j < NM; j++) buf.scale[si(j, r)] = ldg((const _Float16 *)sbase(a, w.m, j) + row);
       }
       if constexpr (EPI == EPI_STORE) {
         // no residual: read element 0 of x instead (always readable; the value is not used), so that there is one
@@ -316,7 +316,7 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
         const uintptr_t has = a.residual != nullptr;
         const AT *res = (const AT *)((uintptr_t)a.residual * has + (uintptr_t)a.x * (1 - has)) + (size_t)row * has;
         if constexpr (COHERENT) set_extra(buf, r, ld_coherent(res));
-        else set_extra(buf, r, *res);
+        else set_extra(buf, r, ldg(res));
       } else if constexpr (EPI == EPI_ROPE_KV) {
         // table row `pos`, entry (cos, sin) of pair i = (row % head_dim) / 2: even r gets cos, odd r gets sin
         const bool ok = pos >= 0 && pos < a.max_context;
@@ -394,7 +394,7 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
           if constexpr (KIND == JSGRAD_W_NF4) {
             const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;
             const int kc = k < in_f ? k : in_f - VEC;
-            bs = (float)((const _Float16 *)sbase(a, w.m, j))[((size_t)row * in_f + kc) >> 6];
+            bs = (float)ldg((const _Float16 *)sbase(a, w.m, j) + (((size_t)row * in_f + kc) >> 6));
           }
           acc[j][r] = Dot<KIND, AT>::run(buf.w[wi(u, j, r)], xf, acc[j][r], bs, lut);
         }

@@ -1,0 +1,1081 @@
+// One decode step of the whole Llama decoder as a single persistent kernel with role-specialised wavefronts (gfx950).
+//
+// At batch 1 every weight byte is used once, so a step is as fast as the weight stream from HBM is continuous.  One launch
+// per fused op leaves the memory system idle at every launch boundary (dispatch ramp, the read of the input row, its
+// RMSNorm, the first load round trip, the tail), which at five boundaries per layer costs as much as the stream itself.
+// Here one block of 12 wavefronts per CU stays resident for the whole step (Transformer.forward,
+// /root/reference/jsgrad/models/llama.ts:201-213) and its wavefronts have fixed roles:
+//
+//   * weight wavefronts do nothing but stream: each walks its own static list of weight items (2 rows x 4 KiB of a
+//     matrix, or 2 rows x 2 KiB of the w1/w3 pair) through ALL phases of the step with two register buffers, so the
+//     loads of the next phase are in flight while the current phase is handed over.  They never issue any other global
+//     load or store (vector memory operations of a wavefront complete in order, so anything else would wait behind the
+//     stream): the input row comes from LDS, the raw row sums go to LDS.
+//   * the control wavefront of the block owns every hand-off: it waits for the other blocks, stages the input row of a
+//     phase in LDS (RMSNorm included), and when the block's weight wavefronts have delivered their sums it applies the
+//     epilogue (row scale, fp16 rounding, residual / rotary + KV-cache write / SwiGLU / logits + arg-max partial), stores
+//     the results for the other blocks and raises the block's flag.
+//   * attention wavefronts run grouped-query attention over the KV cache (llama.ts:89-95) between the QKV and the wo
+//     phase, one (kv head, chunk of positions) item per wavefront, the last item of a kv head merging the chunks.
+//
+// Blocks synchronise through one flag per block (its own 128-byte line) that every control wavefront polls; data that
+// crosses blocks is written with agent-scope stores and read with agent-scope loads.  Every wait is bounded: when a spin
+// runs out the error word is raised, all later waits fall through and the grid drains.
+//
+// The arithmetic is that of the stand-alone kernels (gemv_core.h): an output row is summed by one wavefront in the same
+// order, scaled, rounded and combined by the same expressions.
+#include <algorithm>
+
+#include "gemv_core.h"
+
+namespace jsg {
+
+constexpr int SS_NWW = 8;                        // weight wavefronts per block
+constexpr int SS_NAW = 3;                        // attention wavefronts per block
+constexpr int SS_THREADS = (SS_NWW + 1 + SS_NAW) * 64;
+constexpr int SS_YMAX = 1024;                    // raw row sums a block can hold per phase
+constexpr int SS_CHUNK = 128;                    // most positions per attention item
+constexpr int SS_MAXCH = 64;                     // most attention items per kv head
+constexpr int SS_FLAG_STRIDE = 32;               // ints between block flags: one 128-byte line each
+constexpr int SS_MAX_BLOCKS = 1024;
+constexpr int SS_SPIN_GLOBAL = 1 << 18;          // polls of ~0.5 us
+constexpr int SS_SPIN_LDS = 1 << 21;             // polls of ~0.1 us
+constexpr int SS_NORM_CHUNKS = 8;                // 16-byte chunks of the input row a lane keeps for the fused RMSNorm
+
+// workspace layout (bytes)
+constexpr size_t SS_WS_EPOCH = 0, SS_WS_ERR = 128, SS_WS_COUNTERS = 256, SS_WS_AMAX_VAL = 512, SS_WS_AMAX_IDX = 512 + 4096,
+                 SS_WS_FLAGS = 16384, SS_WS_PARTIAL = SS_WS_FLAGS + (size_t)SS_MAX_BLOCKS * SS_FLAG_STRIDE * 4;
+
+struct SsLayer {   // = jsgrad_hip_layer_t
+  const void *wq, *wk, *wv, *wo, *w1, *w2, *w3;
+  const void *sq, *sk, *sv, *so, *s1, *s2, *s3;
+  const void *attention_norm, *ffn_norm;
+  void *cache_k, *cache_v;
+};
+struct SsArgs {
+  const SsLayer *layers;
+  int n_layers, dim, hidden, n_heads, n_kv_heads, head_dim, vocab, max_context;
+  float eps;
+  int embed_kind;
+  const void *tok_emb, *tok_scale, *out_w, *out_s, *final_norm, *rope_table;
+  int32_t *state, *tokens_out;
+  int tokens_cap;
+  void *h, *h2, *q, *attn, *g, *logits;
+  int *epoch, *err, *flags, *attn_counters;
+  float *attn_partial;   // [n_kv_heads][SS_MAXCH][n_rep][HD + 2]
+  float *amax_val;
+  int *amax_idx;
+  long long *trace;
+  int x_bytes;           // LDS bytes reserved for the staged input row
+};
+
+// LDS control words of a block
+struct SsCtl {
+  int x_ready;            // weight phases whose input row is staged
+  int go;                 // attention phases released
+  int abort;              // a bounded wait ran out somewhere: nobody waits any more
+  int pad;
+  // One progress word per wavefront, not a shared count: a wavefront without work in a phase passes it at once and
+  // may be several phases ahead, so a count of completions would say nothing about the slowest wavefront.
+  int wdone[SS_NWW];      // weight phases wavefront w has delivered
+  int adone[4];           // attention phases attention wavefront a has finished (SS_NAW <= 4)
+};
+static_assert(SS_NAW <= 4 && sizeof(SsCtl) % 8 == 0, "the table of layer tensors follows the control words, 8-byte aligned");
+
+enum { PH_QKV = 0, PH_ATTN = 1, PH_WO = 2, PH_FFN = 3, PH_W2 = 4, PH_LM = 5 };
+
+// Two tables are built in LDS when the kernel starts, because a weight wavefront must not fetch a pointer from global
+// memory (that load would sit behind its weight stream; an LDS read does not touch that queue):
+//   * the layer tensors (a copy of the jsgrad_hip_layer_t array), and
+//   * one record per phase with everything that depends on the phase kind (matrices, scales, shapes, input row,
+//     norm weight, residual, output).  Each record is filled by ONE THREAD with ordinary per-lane code, and the
+//     wavefronts later read whole records by index: selecting among pointers with wavefront-uniform branches on the
+//     phase kind was compiled wrongly (the pointer of another branch survived), a table lookup has nothing to select.
+typedef const __attribute__((address_space(3))) uint64_t *LtPtr;
+struct SsTabs { LtPtr layers, phases; };
+constexpr int SS_LAYER_WORDS = sizeof(SsLayer) / 8;
+constexpr int SS_PHASE_WORDS = 14;   // w0 w1 w2 s0 s1 s2 src norm_w residual y (rows0,rows1) (rows2,in_f) (nm,kind) pad
+// a value that is the same in every lane, moved to scalar registers
+__device__ __forceinline__ uint64_t uni64(uint64_t v) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return ((uint64_t)hi << 32) | lo;
+}
+__device__ __forceinline__ SsLayer ss_layer(const SsTabs &lt, int l) {
+  LtPtr w = lt.layers + (size_t)l * SS_LAYER_WORDS;
+  auto P = [&](int i) { return (const void *)uni64(w[i]); };
+  SsLayer L;
+  L.wq = P(0); L.wk = P(1); L.wv = P(2); L.wo = P(3); L.w1 = P(4); L.w2 = P(5); L.w3 = P(6);
+  L.sq = P(7); L.sk = P(8); L.sv = P(9); L.so = P(10); L.s1 = P(11); L.s2 = P(12); L.s3 = P(13);
+  L.attention_norm = P(14); L.ffn_norm = P(15);
+  L.cache_k = (void *)P(16); L.cache_v = (void *)P(17);
+  return L;
+}
+
+// ---- small helpers -------------------------------------------------------------------------------------------------
+__device__ __forceinline__ int lds_ld(const int *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
+__device__ __forceinline__ void lds_st(int *p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
+// the compiler must not move LDS accesses across a hand-off; the LDS pipeline itself runs a wavefront's accesses in order
+__device__ __forceinline__ void lds_fence() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void vm_drain() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// 16 bytes at the device-wide coherence point, as two 64-bit accesses
+__device__ __forceinline__ u4_t ld16_coherent(const void *p) {
+  const JSG_GLOBAL uint64_t *q = as_global<uint64_t>(p);
+  const uint64_t a = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const uint64_t b = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return u4_t{(uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32)};
+}
+__device__ __forceinline__ void st16_coherent(void *p, u4_t v) {
+  JSG_GLOBAL uint64_t *q = as_global_mut<uint64_t>(p);
+  __hip_atomic_store(q, (uint64_t)v[0] | ((uint64_t)v[1] << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(q + 1, (uint64_t)v[2] | ((uint64_t)v[3] << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Wait until an LDS word reaches `target`.  Returns false when the wait was abandoned.
+__device__ __forceinline__ bool lds_wait(const SsArgs &s, SsCtl &ctl, const int *word, int target) {
+  int it = 0;
+  while (__builtin_amdgcn_readfirstlane(lds_ld(word)) - target < 0) {
+    __builtin_amdgcn_s_sleep(1);
+    if ((++it & 255) == 0) {
+      if (lds_ld(&ctl.abort) != 0) return false;
+      if (it > SS_SPIN_LDS) {
+        st_coherent(s.err, 1);
+        lds_st(&ctl.abort, 1);
+        return false;
+      }
+    }
+  }
+  return true;
+}
+
+// Wait until every one of n (<= 64) LDS words has reached `target`.
+__device__ __forceinline__ bool lds_wait_all(const SsArgs &s, SsCtl &ctl, const int *words, int n, int target) {
+  const int lane = threadIdx.x & 63;
+  int it = 0;
+  while (true) {
+    const int v = lds_ld(words + (lane < n ? lane : 0));
+    if (__all(v - target >= 0)) return true;
+    __builtin_amdgcn_s_sleep(1);
+    if ((++it & 255) == 0) {
+      if (lds_ld(&ctl.abort) != 0) return false;
+      if (it > SS_SPIN_LDS) {
+        st_coherent(s.err, 1);
+        lds_st(&ctl.abort, 1);
+        return false;
+      }
+    }
+  }
+}
+
+// ---- weight phases -------------------------------------------------------------------------------------------------
+struct WDesc {
+  const char *w0, *w1, *w2;   // QKV: wq, wk, wv stacked; FFN: w1 and w3 on the same rows (nm == 2); otherwise w0 alone
+  const void *s0, *s1, *s2;   // int8 row scales
+  const void *src, *norm_w, *residual;   // input row (activation dtype), RMSNorm weight or null, residual row or null
+  void *y;                    // output row (null for QKV: queries and cache rows have their own places)
+  int rows0, rows1, rows2;
+  int in_f, nm, kind;
+};
+__device__ __forceinline__ int ss_phases(const SsArgs &s) { return 5 * s.n_layers + 1; }
+__device__ __forceinline__ int ss_kind(const SsArgs &s, int p) { return p == 5 * s.n_layers ? PH_LM : p % 5; }
+// weight phases before phase p (p itself a weight phase)
+__device__ __forceinline__ int ss_wordinal(const SsArgs &s, int p) {
+  const int l = p / 5, k = p % 5;
+  return p == 5 * s.n_layers ? 4 * s.n_layers : 4 * l + (k == 0 ? 0 : k - 1);
+}
+__device__ __forceinline__ int ss_next_weight(const SsArgs &s, int p) {
+  p++;
+  if (p < 5 * s.n_layers && p % 5 == PH_ATTN) p++;
+  return p;
+}
+// record of phase p, written by one thread (per-lane code: the selects below are plain conditional moves)
+__device__ __forceinline__ void ss_build_phase(const SsArgs &s, uint64_t *rec, int p) {
+  const int k = ss_kind(s, p);
+  const int l = k == PH_LM ? s.n_layers - 1 : p / 5;
+  const uint64_t *L = (const uint64_t *)s.layers + (size_t)l * SS_LAYER_WORDS;
+  // word indices of jsgrad_hip_layer_t: wq wk wv wo w1 w2 w3 | sq sk sv so s1 s2 s3 | attention_norm ffn_norm | cache_k cache_v
+  uint64_t w0 = 0, w1 = 0, w2 = 0, s0 = 0, s1 = 0, s2 = 0, src = 0, norm_w = 0, residual = 0, y = 0;
+  int rows0 = 0, rows1 = 0, rows2 = 0, in_f = 0, nm = 1;
+  const int qdim = s.n_heads * s.head_dim, kvdim = s.n_kv_heads * s.head_dim;
+  if (k == PH_QKV) {
+    w0 = ldg(L + 0); w1 = ldg(L + 1); w2 = ldg(L + 2); s0 = ldg(L + 7); s1 = ldg(L + 8); s2 = ldg(L + 9);
+    rows0 = qdim; rows1 = kvdim; rows2 = kvdim; in_f = s.dim; src = (uint64_t)(uintptr_t)s.h; norm_w = ldg(L + 14);
+  } else if (k == PH_WO) {
+    w0 = ldg(L + 3); s0 = ldg(L + 10); rows0 = s.dim; in_f = qdim;
+    src = (uint64_t)(uintptr_t)s.attn; residual = (uint64_t)(uintptr_t)s.h; y = (uint64_t)(uintptr_t)s.h2;
+  } else if (k == PH_FFN) {
+    w0 = ldg(L + 4); w1 = ldg(L + 6); s0 = ldg(L + 11); s1 = ldg(L + 13); rows0 = s.hidden; in_f = s.dim; nm = 2;
+    src = (uint64_t)(uintptr_t)s.h2; norm_w = ldg(L + 15); y = (uint64_t)(uintptr_t)s.g;
+  } else if (k == PH_W2) {
+    w0 = ldg(L + 5); s0 = ldg(L + 12); rows0 = s.dim; in_f = s.hidden;
+    src = (uint64_t)(uintptr_t)s.g; residual = (uint64_t)(uintptr_t)s.h2; y = (uint64_t)(uintptr_t)s.h;
+  } else if (k == PH_LM) {
+    w0 = (uint64_t)(uintptr_t)s.out_w; s0 = (uint64_t)(uintptr_t)s.out_s; rows0 = s.vocab; in_f = s.dim;
+    src = (uint64_t)(uintptr_t)s.h; norm_w = (uint64_t)(uintptr_t)s.final_norm; y = (uint64_t)(uintptr_t)s.logits;
+  }
+  rec[0] = w0; rec[1] = w1; rec[2] = w2; rec[3] = s0; rec[4] = s1; rec[5] = s2; rec[6] = src; rec[7] = norm_w; rec[8] = residual; rec[9] = y;
+  rec[10] = (uint32_t)rows0 | ((uint64_t)(uint32_t)rows1 << 32);
+  rec[11] = (uint32_t)rows2 | ((uint64_t)(uint32_t)in_f << 32);
+  rec[12] = (uint32_t)nm | ((uint64_t)(uint32_t)k << 32);
+  rec[13] = 0;
+}
+// the record of phase p, in scalar registers
+__device__ __forceinline__ WDesc ss_wdesc(const SsArgs &s, const SsTabs &lt, int p) {
+  LtPtr r = lt.phases + (size_t)p * SS_PHASE_WORDS;
+  WDesc d;
+  d.w0 = (const char *)uni64(r[0]); d.w1 = (const char *)uni64(r[1]); d.w2 = (const char *)uni64(r[2]);
+  d.s0 = (const void *)uni64(r[3]); d.s1 = (const void *)uni64(r[4]); d.s2 = (const void *)uni64(r[5]);
+  d.src = (const void *)uni64(r[6]); d.norm_w = (const void *)uni64(r[7]); d.residual = (const void *)uni64(r[8]); d.y = (void *)uni64(r[9]);
+  const uint64_t a = uni64(r[10]), b = uni64(r[11]), c = uni64(r[12]);
+  d.rows0 = (int)(uint32_t)a; d.rows1 = (int)(a >> 32); d.rows2 = (int)(uint32_t)b; d.in_f = (int)(b >> 32);
+  d.nm = (int)(uint32_t)c; d.kind = (int)(c >> 32);
+  return d;
+}
+__device__ __forceinline__ int wd_rows(const WDesc &d) { return d.rows0 + (d.nm == 1 ? d.rows1 + d.rows2 : 0); }
+__device__ __forceinline__ int wd_groups(const WDesc &d) { return (wd_rows(d) + 1) >> 1; }
+
+// The weight format of the step: VEC elements per 16-byte load, STEP elements per wavefront k-step; an item is 8 loads:
+// 2 rows x 4 k-steps of one matrix, or 2 rows x 2 k-steps of two.
+template <int KIND> struct SsFmt {
+  static constexpr int VEC = WFmt<KIND>::VEC;
+  static constexpr int BITS = KIND == JSGRAD_W_F16 ? 16 : 8;
+  static constexpr int STEP = 64 * VEC;
+  __device__ static __forceinline__ int unroll(int nm) { return nm == 2 ? 2 : 4; }
+  __device__ static __forceinline__ int nbatch(const WDesc &d) { const int u = unroll(d.nm); return ((d.in_f + STEP - 1) / STEP + u - 1) / u; }
+};
+// LDS elements the staged input row of a phase occupies (whole batches; the tail is zero)
+static int ss_x_elems(int kind, int in_f, int nm) {
+  const int step = 64 * (kind == JSGRAD_W_F16 ? 8 : 16), u = nm == 2 ? 2 : 4;
+  return (((in_f + step - 1) / step + u - 1) / u) * u * step;
+}
+
+struct WBuf { u4_t w[8]; };
+
+// position of a wavefront in its item list: phase, row group, k-batch
+struct WIter {
+  int p, grp, b, ngroups, nb;
+  bool live;
+  WDesc d;
+};
+
+template <int KIND> struct SsWeights {
+  typedef SsFmt<KIND> F;
+
+  __device__ static __forceinline__ void enter(const SsArgs &s, const SsTabs &lt, WIter &it, int p, int gw) {
+    it.p = p;
+    it.d = ss_wdesc(s, lt, p);
+    it.ngroups = wd_groups(it.d);
+    it.nb = F::nbatch(it.d);
+    it.grp = gw;
+    it.b = 0;
+  }
+  // first phase at or after p in which wavefront gw has an item; when there is none the iterator parks on an item that
+  // exists (group 0 of the lm_head), so that the loads it keeps issuing stay inside a matrix
+  __device__ static __forceinline__ void seek(const SsArgs &s, const SsTabs &lt, WIter &it, int p, int gw) {
+    const int nph = ss_phases(s);
+    while (p < nph) {
+      enter(s, lt, it, p, gw);
+      if (gw < it.ngroups) { it.live = true; return; }
+      p = ss_next_weight(s, p);
+    }
+    enter(s, lt, it, nph - 1, 0);
+    it.live = false;
+  }
+  __device__ static __forceinline__ void advance(const SsArgs &s, const SsTabs &lt, WIter &it, int gw, int ngw) {
+    if (!it.live) return;
+    if (++it.b < it.nb) return;
+    it.b = 0;
+    it.grp += ngw;
+    if (it.grp < it.ngroups) return;
+    seek(s, lt, it, ss_next_weight(s, it.p), gw);
+  }
+
+  // issue the 8 loads of the item the iterator stands on
+  __device__ static __forceinline__ void load(WBuf &buf, const WIter &it) {
+    const WDesc &d = it.d;
+    const int lane = threadIdx.x & 63;
+    // rows of the group: matrix m of the stacked wq | wk | wv, first row r0 inside it
+    int m = 0, r0 = it.grp * 2;
+    if (d.nm == 1 && d.rows1 > 0) {
+      if (r0 >= d.rows0) { r0 -= d.rows0; m = 1; }
+      if (m == 1 && r0 >= d.rows1) { r0 -= d.rows1; m = 2; }
+    }
+    const int mrows = d.rows0 * (m == 0) + d.rows1 * (m == 1) + d.rows2 * (m == 2);
+    const uintptr_t base_m = (uintptr_t)d.w0 * (uintptr_t)(m == 0) + (uintptr_t)d.w1 * (uintptr_t)(m == 1) + (uintptr_t)d.w2 * (uintptr_t)(m == 2);
+    const int un = F::unroll(d.nm);
+#pragma unroll
+    for (int v = 0; v < 8; v++) {
+      const int u = d.nm == 2 ? v >> 2 : v >> 1, j = d.nm == 2 ? (v >> 1) & 1 : 0, r = v & 1;
+      int k = (it.b * un + u) * F::STEP + lane * F::VEC;
+      k = k < d.in_f ? k : d.in_f - F::VEC;   // lanes past the end reload the last vector; their x is zero
+      const int row = r0 + r < mrows ? r0 + r : mrows - 1;
+      const uintptr_t base = d.nm == 2 ? (j ? (uintptr_t)d.w1 : (uintptr_t)d.w0) : base_m;
+      const char *p = (const char *)base + (((size_t)row * d.in_f + (size_t)k) * F::BITS) / 8;
+      buf.w[v] = ldg_stream16(p);
+    }
+  }
+
+  // consume the item (grp round `round`, batch b) of a phase with NM matrices; on the last batch the row sums go to LDS
+  template <int NM>
+  __device__ static __forceinline__ void consume(const WBuf &buf, int b, int nb, float (&acc)[2][2], const _Float16 *xs, float *y_local, int round, int wave) {
+    constexpr int UN = NM == 2 ? 2 : 4;
+    const int lane = threadIdx.x & 63;
+    if (b == 0) {
+#pragma unroll
+      for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int r = 0; r < 2; r++) acc[j][r] = 0.0f;
+    }
+#pragma unroll
+    for (int u = 0; u < UN; u++) {
+      const int k = (b * UN + u) * F::STEP + lane * F::VEC;   // may lie in the zero padding of xs
+      XFrag<_Float16, F::VEC> xf;
+      xf.load(xs + k);
+#pragma unroll
+      for (int j = 0; j < NM; j++)
+#pragma unroll
+        for (int r = 0; r < 2; r++) acc[j][r] = Dot<KIND, _Float16>::run(buf.w[(u * NM + j) * 2 + r], xf, acc[j][r], 1.0f, nullptr);
+    }
+    if (b != nb - 1) return;
+    float tot[NM][2];
+#pragma unroll
+    for (int j = 0; j < NM; j++)
+#pragma unroll
+      for (int r = 0; r < 2; r++) tot[j][r] = wave_sum(acc[j][r]);
+    if (lane == 0) {
+      float *dst = y_local + ((round * SS_NWW + wave) * NM) * 2;
+#pragma unroll
+      for (int j = 0; j < NM; j++)
+#pragma unroll
+        for (int r = 0; r < 2; r++) dst[j * 2 + r] = tot[j][r];
+    }
+  }
+
+  // the whole life of a weight wavefront
+  __device__ static __forceinline__ void run(const SsArgs &s, const SsTabs &lt, SsCtl &ctl, const _Float16 *xs, float *y_local, int wave) {
+    const int G = gridDim.x, gw = wave * G + blockIdx.x, ngw = SS_NWW * G, nph = ss_phases(s);
+    WIter li;
+    WBuf A, B;
+    seek(s, lt, li, 0, gw);
+    load(A, li);
+    advance(s, lt, li, gw, ngw);
+    load(B, li);
+    advance(s, lt, li, gw, ngw);
+    int n = 0;
+    float acc[2][2];
+    for (int p = 0; p < nph; p = ss_next_weight(s, p)) {
+      const WDesc d = ss_wdesc(s, lt, p);
+      const int ngroups = wd_groups(d), nb = F::nbatch(d);
+      if (gw < ngroups) {
+        lds_wait(s, ctl, &ctl.x_ready, ss_wordinal(s, p) + 1);
+        lds_fence();
+        int round = 0;
+        for (int grp = gw; grp < ngroups; grp += ngw, round++) {
+          for (int b = 0; b < nb; b++) {
+#ifdef JSG_SS_DEBUG
+            if (s.trace && blockIdx.x == 0 && wave == 0 && ss_kind(s, p) == JSG_SS_DEBUG && b == 0 && grp == gw) {
+              uint32_t *dbg = (uint32_t *)s.trace;
+              const int lane = threadIdx.x & 63;
+              for (int v = 0; v < 8; v++)
+                for (int e2 = 0; e2 < 4; e2++) {
+                  dbg[32768 + (v * 64 + lane) * 4 + e2] = A.w[v][e2];
+                  dbg[36864 + (v * 64 + lane) * 4 + e2] = B.w[v][e2];
+                }
+              if (lane == 0) { dbg[40960] = n; dbg[40961] = li.p; dbg[40962] = li.grp; dbg[40963] = li.b; dbg[40964] = li.live; dbg[40965] = nb; dbg[40966] = p; }
+            }
+#endif
+#ifdef JSG_SS_DEBUG
+            if (s.trace && blockIdx.x == 0 && wave == 0 && (threadIdx.x & 63) == 0 && n < 16) {
+              uint32_t *dbg = (uint32_t *)s.trace + 45056 + n * 16;
+              dbg[0] = n; dbg[1] = li.p; dbg[2] = li.grp; dbg[3] = li.b; dbg[4] = (uint32_t)(uintptr_t)li.d.w0; dbg[5] = (uint32_t)((uintptr_t)li.d.w0 >> 32);
+              dbg[6] = li.d.in_f; dbg[7] = li.d.rows0; dbg[8] = li.d.nm; dbg[9] = p; dbg[10] = li.live;
+            }
+#endif
+            if (n & 1) {
+              if (d.nm == 2) consume<2>(B, b, nb, acc, xs, y_local, round, wave);
+              else consume<1>(B, b, nb, acc, xs, y_local, round, wave);
+              load(B, li);
+            } else {
+              if (d.nm == 2) consume<2>(A, b, nb, acc, xs, y_local, round, wave);
+              else consume<1>(A, b, nb, acc, xs, y_local, round, wave);
+              load(A, li);
+            }
+            advance(s, lt, li, gw, ngw);
+            n++;
+          }
+        }
+      }
+      lds_fence();   // the sums are in LDS before the phase is marked delivered
+      if ((threadIdx.x & 63) == 0) lds_st(&ctl.wdone[wave], ss_wordinal(s, p) + 1);
+    }
+  }
+};
+
+// ---- attention wavefronts ------------------------------------------------------------------------------------------
+template <int G> __device__ __forceinline__ float ss_group_sum(float v) {
+  static_assert(G == 8 || G == 16, "lane group");
+  v += dpp_f<0xB1>(v);
+  v += dpp_f<0x4E>(v);
+  v += dpp_f<0x141>(v);
+  if (G == 16) v += dpp_f<0x140>(v);
+  return v;
+}
+
+template <int HD, int NREP> struct SsAttn {
+  static constexpr int GL = HD / 8;     // lanes per cache row (8 halves = one 128-bit load per lane)
+  static constexpr int RPI = 64 / GL;   // rows per wavefront load
+
+  // rows per item for T visible positions when `waves` wavefronts are available per kv head
+  __device__ static __forceinline__ int chunk_rows(int T, int waves) {
+    int per = waves < SS_MAXCH ? waves : SS_MAXCH;
+    per = per < 1 ? 1 : per;
+    int chunk = (T + per - 1) / per;
+    chunk = chunk < 32 ? 32 : chunk;
+    return chunk > SS_CHUNK ? SS_CHUNK : chunk;   // the host keeps max_context <= SS_MAXCH * SS_CHUNK
+  }
+
+  // item (kv head g, chunk c): scores, softmax numerators and P.V of rows [c * chunk, ...) for the NREP query heads of
+  // the kv head; the wavefront that completes the kv head merges all chunks.  sc: this wavefront's LDS float[NREP][SS_CHUNK].
+  __device__ static void item(const SsArgs &s, const SsLayer &L, float *sc, int g, int c, int T, int chunk, int n_active) {
+    typedef _Float16 AT;
+    const int lane = threadIdx.x & 63, sub = lane % GL, grp = lane / GL;
+    const int t0 = c * chunk, t1 = min(T, t0 + chunk), CH = t1 - t0;
+    const size_t row_stride = (size_t)s.n_kv_heads * HD;
+    const AT *kbase = (const AT *)L.cache_k + (size_t)g * HD + (size_t)sub * 8;
+    const AT *vbase = (const AT *)L.cache_v + (size_t)g * HD + (size_t)sub * 8;
+    const float scale = (float)(1.0 / sqrt((double)HD));
+
+    // A batch is 8 loads of RPI rows each; the first batch of K and of V goes out at once (most chunks are one batch)
+    constexpr int BR = 8 * RPI;
+    u4_t kraw[8], vraw[8];
+    auto load_batch = [&](u4_t (&raw)[8], const AT *base, int tb) {
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const int t = tb + u * RPI + grp;
+        raw[u] = ldg((const u4_t *)(base + (size_t)(t < t1 ? t : t1 - 1) * row_stride));
+      }
+    };
+    load_batch(kraw, kbase, t0);
+    load_batch(vraw, vbase, t0);
+    h2_t qh[NREP][4];
+#pragma unroll
+    for (int j = 0; j < NREP; j++) {
+      const u4_t raw = ld16_coherent((const AT *)s.q + (size_t)(g * NREP + j) * HD + sub * 8);
+#pragma unroll
+      for (int e = 0; e < 4; e++) qh[j][e] = as_h2(raw[e]);
+    }
+    // scores of the chunk and their maximum
+    float mx[NREP];
+#pragma unroll
+    for (int j = 0; j < NREP; j++) mx[j] = -INFINITY;
+    for (int tb = t0; tb < t1; tb += BR) {
+      if (tb != t0) load_batch(kraw, kbase, tb);
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const int t = tb + u * RPI + grp;
+#pragma unroll
+        for (int j = 0; j < NREP; j++) {
+          float p = 0.0f;
+#pragma unroll
+          for (int e = 0; e < 4; e++) p = __builtin_amdgcn_fdot2(qh[j][e], as_h2(kraw[u][e]), p, false);
+          p = ss_group_sum<GL>(p) * scale;
+          if (t < t1) {
+            if (sub == 0) sc[j * SS_CHUNK + (t - t0)] = p;
+            mx[j] = fmaxf(mx[j], p);
+          }
+        }
+      }
+    }
+    float ls[NREP];
+#pragma unroll
+    for (int j = 0; j < NREP; j++) { mx[j] = wave_max(mx[j]); ls[j] = 0.0f; }
+    lds_fence();
+    for (int i = lane; i < CH; i += 64)
+#pragma unroll
+      for (int j = 0; j < NREP; j++) {
+        const float e = exp_f32(sc[j * SS_CHUNK + i] - mx[j]);
+        sc[j * SS_CHUNK + i] = e;
+        ls[j] += e;
+      }
+#pragma unroll
+    for (int j = 0; j < NREP; j++) ls[j] = wave_sum(ls[j]);
+    lds_fence();
+    // o[j][d] = sum_t p[j][t] * V[t][d]
+    float of[NREP][8];
+#pragma unroll
+    for (int j = 0; j < NREP; j++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) of[j][e] = 0.0f;
+    for (int tb = t0; tb < t1; tb += BR) {
+      if (tb != t0) load_batch(vraw, vbase, tb);
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const int t = tb + u * RPI + grp;
+        float vf[8];
+#pragma unroll
+        for (int e = 0; e < 4; e++) { h2_t h = as_h2(vraw[u][e]); vf[2 * e] = (float)h[0]; vf[2 * e + 1] = (float)h[1]; }
+#pragma unroll
+        for (int j = 0; j < NREP; j++) {
+          const float p = t < t1 ? sc[j * SS_CHUNK + (t - t0)] : 0.0f;
+#pragma unroll
+          for (int e = 0; e < 8; e++) of[j][e] = fmaf(p, vf[e], of[j][e]);
+        }
+      }
+    }
+    // lanes with the same `sub` hold different rows: fold the row groups of the wavefront together
+#pragma unroll
+    for (int j = 0; j < NREP; j++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        float v = of[j][e];
+#pragma unroll
+        for (int off = GL; off < 64; off <<= 1) v += __shfl_xor(v, off);
+        of[j][e] = v;
+      }
+    float *mine = s.attn_partial + ((size_t)g * SS_MAXCH + c) * NREP * (HD + 2);
+    if (grp == 0) {
+#pragma unroll
+      for (int j = 0; j < NREP; j++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) st_coherent(&mine[j * (HD + 2) + sub * 8 + e], of[j][e]);
+    }
+#pragma unroll
+    for (int j = 0; j < NREP; j++)
+      if (lane == j) {
+        st_coherent(&mine[j * (HD + 2) + HD], mx[j]);
+        st_coherent(&mine[j * (HD + 2) + HD + 1], ls[j]);
+      }
+    vm_drain();   // the partial is at the coherence point before the item is counted
+    int old = 0;
+    if (lane == 0) old = __hip_atomic_fetch_add(&s.attn_counters[g], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    old = __builtin_amdgcn_readfirstlane(old);
+    if (old != n_active - 1) return;
+
+    // ---- merge the chunks of kv head g: weights exp(m_s - M), normalisation 1 / sum(l_s * w_s)
+    const float *base = s.attn_partial + (size_t)g * SS_MAXCH * NREP * (HD + 2);
+    float inv[NREP];
+#pragma unroll
+    for (int j = 0; j < NREP; j++) {
+      const bool on = lane < n_active;   // n_active <= SS_MAXCH = 64: one chunk per lane
+      const float *ps = base + ((size_t)(on ? lane : 0) * NREP + j) * (HD + 2);
+      const float ms = on ? ld_coherent(ps + HD) : -INFINITY;
+      const float lsum = on ? ld_coherent(ps + HD + 1) : 0.0f;
+      const float M = wave_max(ms);
+      const float w = on ? exp_f32(ms - M) : 0.0f;
+      if (on) sc[j * SS_CHUNK + lane] = w;
+      const float Ls = wave_sum(lsum * w);
+      inv[j] = 1.0f / Ls;   // softmax normalisation is e * (1/sum) (tensor.ts:2211-2214)
+    }
+    lds_fence();
+#pragma unroll
+    for (int j = 0; j < NREP; j++) {
+#pragma unroll
+      for (int d0 = 0; d0 < HD; d0 += 64) {
+        const int d = d0 + lane;
+        const float *po = base + (size_t)j * (HD + 2) + d;
+        float O = 0.0f;
+        for (int c2 = 0; c2 < n_active; c2 += 8) {   // eight independent loads in flight, summed in chunk order
+          float t8[8];
+#pragma unroll
+          for (int u = 0; u < 8; u++) t8[u] = ld_coherent(po + (size_t)(c2 + u < n_active ? c2 + u : n_active - 1) * NREP * (HD + 2));
+#pragma unroll
+          for (int u = 0; u < 8; u++)
+            if (c2 + u < n_active) O = fmaf(t8[u], sc[j * SS_CHUNK + c2 + u], O);
+        }
+        st_coherent((AT *)s.attn + (size_t)(g * NREP + j) * HD + d, (AT)rn16(O * inv[j]));
+      }
+    }
+    if (lane == 0) __hip_atomic_store(&s.attn_counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+
+  __device__ static __forceinline__ void run(const SsArgs &s, const SsTabs &lt, SsCtl &ctl, float *sc, int aw, int pos) {
+    const int G = gridDim.x, gid = aw * G + blockIdx.x, na = SS_NAW * G;
+    const bool pos_ok = pos >= 0 && pos < s.max_context;
+    for (int l = 0; l < s.n_layers; l++) {
+      lds_wait(s, ctl, &ctl.go, l + 1);
+      if (pos_ok && lds_ld(&ctl.abort) == 0) {
+        const int T = pos + 1;
+        const int chunk = chunk_rows(T, na / s.n_kv_heads);
+        const int n_active = (T + chunk - 1) / chunk;
+        const SsLayer L = ss_layer(lt, l);
+        for (int item_id = gid; item_id < s.n_kv_heads * n_active; item_id += na)
+          item(s, L, sc, item_id / n_active, item_id % n_active, T, chunk, n_active);
+      }
+      vm_drain();   // this wavefront's outputs are at the coherence point
+      if ((threadIdx.x & 63) == 0) lds_st(&ctl.adone[aw], l + 1);
+    }
+  }
+};
+
+// ---- the control wavefront -----------------------------------------------------------------------------------------
+template <int KIND> struct SsControl {
+  typedef _Float16 AT;
+  typedef SsFmt<KIND> F;
+
+  // wait until every block's flag has reached `target`
+  __device__ static __forceinline__ void wait_flags(const SsArgs &s, SsCtl &ctl, int target) {
+    const int lane = threadIdx.x & 63, G = gridDim.x;
+    int it = 0;
+    while (true) {
+      int worst = 0;
+      for (int b0 = 0; b0 < G; b0 += 256) {
+        int v[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+          const int b = b0 + k * 64 + lane;
+          v[k] = b < G ? ld_coherent(&s.flags[b * SS_FLAG_STRIDE]) - target : 0;
+        }
+        worst = min(worst, min(min(v[0], v[1]), min(v[2], v[3])));
+      }
+      if (__all(worst >= 0)) return;
+      if ((++it & 15) == 0) {
+        if (lds_ld(&ctl.abort) != 0) return;
+        if (it > SS_SPIN_GLOBAL || ld_coherent(s.err) != 0) {
+          st_coherent(s.err, 1);
+          lds_st(&ctl.abort, 1);
+          return;
+        }
+      }
+    }
+  }
+
+  // 16-byte chunk c of the input row: written by other blocks in the activation dtype, or (EMB_I8) eight codes of an
+  // int8 embedding row, each becoming RN16(code * scale) (llama3.ts:71-77)
+  template <bool EMB_I8> __device__ static __forceinline__ u4_t fetch_x(const void *src, int c, float emb_scale) {
+    if constexpr (!EMB_I8) {
+      return ld16_coherent((const u4_t *)src + c);
+    } else {
+      const uint64_t raw = ldg((const uint64_t *)src + c);
+      u4_t o;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        h2_t y;
+        y[0] = mul_rn16((float)(int8_t)(raw >> (16 * e)), emb_scale);
+        y[1] = mul_rn16((float)(int8_t)(raw >> (16 * e + 8)), emb_scale);
+        o[e] = __builtin_bit_cast(uint32_t, y);
+      }
+      return o;
+    }
+  }
+  // RMSNorm'ed row -> LDS (nn/index.ts:586-588); a lane keeps NR chunks between the sum of squares and the scaling.
+  // Loads are unconditional (lanes past the end re-read the last chunk): a load under a lane mask costs a full wait.
+  // mirror: where the raw row is left for later phases (block 0 and the embedding row only).
+  template <bool EMB_I8, int NR>
+  __device__ static __forceinline__ void stage_norm(const SsArgs &s, u4_t *xl, const void *src, const void *norm_w, int nchunks, float inv_d, float emb_scale, void *mirror) {
+    const int lane = threadIdx.x & 63;
+    u4_t xr[NR];
+#pragma unroll
+    for (int i = 0; i < NR; i++) {
+      const int c = i * 64 + lane;
+      xr[i] = fetch_x<EMB_I8>(src, c < nchunks ? c : nchunks - 1, emb_scale);
+    }
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NR; i++) {
+      const int c = i * 64 + lane;
+      float part = ss;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        h2_t h = as_h2(xr[i][e]);
+        part = fmaf((float)h[0], (float)h[0], part);
+        part = fmaf((float)h[1], (float)h[1], part);
+      }
+      ss = c < nchunks ? part : ss;
+      if (mirror != nullptr && c < nchunks) st16_coherent((u4_t *)mirror + c, xr[i]);
+    }
+    const float tot = wave_sum(ss);
+    // sqrt(1 / (mean + eps)), mean = sum * float(1/d)  (nn/index.ts:586, tensor.ts:2944-2946)
+    const float r = __fsqrt_rn(__fdiv_rn(1.0f, __fadd_rn(__fmul_rn(tot, inv_d), s.eps)));
+    constexpr int WB = NR < 8 ? NR : 8;   // norm weights are fetched WB chunks at a time
+#pragma unroll
+    for (int i0 = 0; i0 < NR; i0 += WB) {
+      u4_t wr[WB];
+#pragma unroll
+      for (int i = 0; i < WB; i++) {
+        const int c = (i0 + i) * 64 + lane;
+        wr[i] = ldg((const u4_t *)norm_w + (c < nchunks ? c : nchunks - 1));
+      }
+#pragma unroll
+      for (int i = 0; i < WB; i++) {
+        const int c = (i0 + i) * 64 + lane;
+        u4_t o;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          h2_t h = as_h2(xr[i0 + i][e]), w = as_h2(wr[i][e]), y;
+          // .cast(x.dtype) before the weight multiply (nn/index.ts:588)
+          y[0] = (_Float16)((float)(_Float16)((float)h[0] * r) * (float)w[0]);
+          y[1] = (_Float16)((float)(_Float16)((float)h[1] * r) * (float)w[1]);
+          o[e] = __builtin_bit_cast(uint32_t, y);
+        }
+        if (c < nchunks) xl[c] = o;
+      }
+    }
+  }
+  // Stage the input row of a weight phase in LDS.  src: in_f halves written by other blocks (or the embedding row);
+  // norm_w != nullptr applies RMSNorm.  The tail up to `padded` is zeroed.
+  template <bool EMB_I8>
+  __device__ static __forceinline__ void stage_x(const SsArgs &s, AT *xs, const void *src, const void *norm_w, int in_f, int padded, float inv_d, float emb_scale, void *mirror) {
+    const int lane = threadIdx.x & 63;
+    const int nchunks = in_f / 8;
+    u4_t *xl = (u4_t *)xs;
+    for (int c = nchunks + lane; c < padded / 8; c += 64) xl[c] = u4_t{0, 0, 0, 0};
+    if (norm_w == nullptr) {
+      for (int c0 = 0; c0 < nchunks; c0 += 64 * 8) {
+        u4_t t[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          const int c = c0 + i * 64 + lane;
+          t[i] = fetch_x<EMB_I8>(src, c < nchunks ? c : nchunks - 1, emb_scale);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          const int c = c0 + i * 64 + lane;
+          if (c < nchunks) xl[c] = t[i];
+        }
+      }
+      return;
+    }
+    const int nr = (nchunks + 63) / 64;   // <= SS_NORM_CHUNKS (host)
+    if (nr <= 1) stage_norm<EMB_I8, 1>(s, xl, src, norm_w, nchunks, inv_d, emb_scale, mirror);
+    else if (nr <= 2) stage_norm<EMB_I8, 2>(s, xl, src, norm_w, nchunks, inv_d, emb_scale, mirror);
+    else if (nr <= 4) stage_norm<EMB_I8, 4>(s, xl, src, norm_w, nchunks, inv_d, emb_scale, mirror);
+    else stage_norm<EMB_I8, 8>(s, xl, src, norm_w, nchunks, inv_d, emb_scale, mirror);
+  }
+
+  // what the epilogue of one 64-slot pass needs besides the sums
+  struct EpiOps {
+    float sc0, sc1;   // row scale(s)
+    float e0, e1;     // residual | (cos, sin)
+  };
+  struct EpiCtx {
+    int kind;          // PH_*
+    WDesc d;
+    int ngroups;
+    const void *residual;
+    void *y;
+    SsLayer L;
+    int pos;
+    bool pos_ok;
+  };
+  // slot -> stacked row of the phase (or -1): slots are (round, weight wavefront, row of the pair)
+  __device__ static __forceinline__ int slot_row(const EpiCtx &e, int slot) {
+    const int G = gridDim.x, pair = slot >> 1, w = pair % SS_NWW, round = pair / SS_NWW;
+    const int g = w * G + blockIdx.x + round * (SS_NWW * G);
+    return g < e.ngroups ? 2 * g + (slot & 1) : -1;
+  }
+  __device__ static __forceinline__ void locate(const WDesc &d, int row, int &m, int &rr) {
+    m = 0; rr = row;
+    if (d.nm == 1 && d.rows1 > 0) {
+      if (rr >= d.rows0) { rr -= d.rows0; m = 1; }
+      if (m == 1 && rr >= d.rows1) { rr -= d.rows1; m = 2; }
+    }
+  }
+  __device__ static __forceinline__ EpiOps epi_load(const SsArgs &s, const EpiCtx &e, int slot) {
+    EpiOps o = {1.0f, 1.0f, 0.0f, 0.0f};
+    const int row = slot_row(e, slot);
+    if (row < 0) return o;
+    int m, rr;
+    locate(e.d, row, m, rr);
+    if constexpr (KIND == JSGRAD_W_I8) {
+      const _Float16 *sp = (const _Float16 *)((uintptr_t)e.d.s0 * (uintptr_t)(m == 0) + (uintptr_t)e.d.s1 * (uintptr_t)(m == 1) + (uintptr_t)e.d.s2 * (uintptr_t)(m == 2));
+      o.sc0 = (float)ldg(sp + rr);
+      if (e.d.nm == 2) o.sc1 = (float)ldg((const _Float16 *)e.d.s1 + rr);
+    }
+    if (e.kind == PH_QKV) {
+      if (e.pos_ok && m < 2) {
+        const int i = (rr % s.head_dim) >> 1;
+        const AT *tp = (const AT *)s.rope_table + (size_t)e.pos * s.head_dim + 2 * i;
+        o.e0 = (float)ldg(tp);
+        o.e1 = (float)ldg(tp + 1);
+      }
+    } else if (e.residual != nullptr) {
+      o.e0 = (float)ld_coherent((const AT *)e.residual + row);
+    }
+    return o;
+  }
+  // best: running arg-max of the logits this lane has stored (PH_LM)
+  __device__ static __forceinline__ void epi_apply(const SsArgs &s, const EpiCtx &e, int slot, const EpiOps &o, const float *y_local, float &best, int &best_i) {
+    const int row = slot_row(e, slot);
+    float v0 = 0.0f, v1 = 0.0f;
+    if (row >= 0) {
+      if (e.d.nm == 2) {
+        const int idx = (slot >> 1) * 4 + (slot & 1);
+        v0 = y_local[idx];
+        v1 = y_local[idx + 2];
+      } else {
+        v0 = y_local[slot];
+      }
+    }
+    if constexpr (KIND == JSGRAD_W_I8) { v0 = v0 * o.sc0; v1 = v1 * o.sc1; }
+#ifdef JSG_SS_DEBUG
+    if (s.trace && row >= 0 && e.kind == JSG_SS_DEBUG) {
+      float *dbg = (float *)s.trace;
+      dbg[row * 4 + 0] = v0;
+      dbg[row * 4 + 1] = o.e0;
+      dbg[row * 4 + 2] = (float)blockIdx.x;
+      dbg[row * 4 + 3] = (float)slot;
+    }
+#endif
+    v0 = rn16(v0);
+    v1 = rn16(v1);
+    // the other row of the pair sits in the neighbouring lane
+    const float partner = dpp_f<0xB1>(v0);
+    if (row < 0) return;
+    if (e.kind == PH_QKV) {
+      if (!e.pos_ok) return;
+      int m, rr;
+      locate(e.d, row, m, rr);
+      if (m == 2) {
+        st_coherent((AT *)e.L.cache_v + (size_t)e.pos * e.d.rows2 + rr, (AT)v0);
+      } else {
+        // interleaved pairs (llama.ts:17-32): (a, b) -> (a cos - b sin, a sin + b cos), unfused as in plain C
+        const float c = o.e0, d = o.e1;
+        const float out = (row & 1) ? rn16(partner * d + v0 * c) : rn16(v0 * c - partner * d);
+        AT *dst = m == 0 ? (AT *)s.q : (AT *)e.L.cache_k + (size_t)e.pos * e.d.rows1;
+        st_coherent(dst + rr, (AT)out);
+      }
+    } else if (e.kind == PH_FFN) {
+      st_coherent((AT *)e.y + row, (AT)rn16(silu_act<AT>(v0) * v1));
+    } else {
+      float v = v0;
+      if (e.residual != nullptr) v = rn16(o.e0 + v);
+      st_coherent((AT *)e.y + row, (AT)v);
+      if (e.kind == PH_LM && (v > best || (v == best && row < best_i))) { best = v; best_i = row; }
+    }
+  }
+
+  __device__ static __forceinline__ void run(const SsArgs &s, const SsTabs &lt, SsCtl &ctl, AT *xs, const float *y_local, int pos, int tok) {
+    const int lane = threadIdx.x & 63, G = gridDim.x, nph = ss_phases(s);
+    const bool pos_ok = pos >= 0 && pos < s.max_context;
+    const int base = ld_coherent(s.epoch);
+    int tr = 0;
+    auto stamp = [&]() {
+#ifdef JSG_SS_DEBUG
+      return;
+#endif
+      if (s.trace && blockIdx.x == 0 && lane == 0 && tr < 2040) s.trace[tr++] = (long long)__builtin_amdgcn_s_memrealtime();
+    };
+    stamp();
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+    for (int p = 0; p < nph; p++) {
+      const int kind = ss_kind(s, p);
+      if (p > 0) wait_flags(s, ctl, base + p);
+      stamp();
+      if (kind == PH_ATTN) {
+        lds_st(&ctl.go, p / 5 + 1);
+        stamp();
+        lds_wait_all(s, ctl, ctl.adone, SS_NAW, p / 5 + 1);
+        stamp();
+      } else {
+        EpiCtx e;
+        e.kind = kind;
+        e.d = ss_wdesc(s, lt, p);
+        e.ngroups = wd_groups(e.d);
+        e.pos = pos;
+        e.pos_ok = pos_ok;
+        e.L = ss_layer(lt, kind == PH_LM ? 0 : p / 5);
+        e.residual = e.d.residual;
+        e.y = e.d.y;
+        const void *src = e.d.src, *norm_w = e.d.norm_w;
+        bool emb_i8 = false;
+        float emb_scale = 1.0f;
+        void *mirror = nullptr;
+        if (p == 0) {   // the embedding row is the first input (Embedding.call: a row gather); block 0 also leaves it in h
+          emb_i8 = s.embed_kind == JSGRAD_W_I8;
+          src = (const char *)s.tok_emb + (size_t)tok * s.dim * (emb_i8 ? 1 : 2);
+          if (emb_i8) emb_scale = (float)ldg((const _Float16 *)s.tok_scale + tok);
+          if (blockIdx.x == 0) mirror = s.h;
+        }
+        const int padded = F::nbatch(e.d) * F::unroll(e.d.nm) * F::STEP;
+        const float inv_d = (float)(1.0 / (double)e.d.in_f);
+        if (emb_i8) stage_x<true>(s, xs, src, norm_w, e.d.in_f, padded, inv_d, emb_scale, mirror);
+        else stage_x<false>(s, xs, src, norm_w, e.d.in_f, padded, inv_d, emb_scale, mirror);
+        lds_fence();
+#ifdef JSG_SS_DEBUG
+        if (s.trace && blockIdx.x == 0 && kind == JSG_SS_DEBUG) {
+          float *dbg = (float *)s.trace + 16384;
+          for (int i = lane; i < padded; i += 64) dbg[i] = (float)xs[i];
+        }
+#endif
+        lds_st(&ctl.x_ready, ss_wordinal(s, p) + 1);
+        stamp();
+        const int rounds = (e.ngroups + SS_NWW * G - 1) / (SS_NWW * G);
+        const int nslots = rounds * SS_NWW * 2;
+        EpiOps cur = epi_load(s, e, lane);
+        lds_wait_all(s, ctl, ctl.wdone, SS_NWW, ss_wordinal(s, p) + 1);
+        lds_fence();
+        stamp();
+        for (int s0 = 0; s0 < nslots; s0 += 64) {
+          EpiOps nxt = cur;
+          if (s0 + 64 < nslots) nxt = epi_load(s, e, s0 + 64 + lane);
+          epi_apply(s, e, s0 + lane, cur, y_local, best, best_i);
+          cur = nxt;
+        }
+        if (kind == PH_LM) {
+          for (int off = 32; off > 0; off >>= 1) {
+            const float ov = __shfl_xor(best, off);
+            const int oi = __shfl_xor(best_i, off);
+            if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+          }
+          if (lane == 0) { st_coherent(&s.amax_val[blockIdx.x], best); st_coherent(&s.amax_idx[blockIdx.x], best_i); }
+        }
+        vm_drain();   // every store of this phase is at the coherence point
+        stamp();
+      }
+      if (lane == 0) st_coherent(&s.flags[blockIdx.x * SS_FLAG_STRIDE], base + p + 1);
+    }
+    if (blockIdx.x != 0) return;
+    // ---- greedy arg-max over the blocks' partials (Tensor.argmax: lowest index among the maxima), state update
+    wait_flags(s, ctl, base + nph);
+    best = -INFINITY;
+    best_i = 0x7fffffff;
+    for (int b = lane; b < G; b += 64) {
+      const float ov = ld_coherent(&s.amax_val[b]);
+      const int oi = ld_coherent(&s.amax_idx[b]);
+      if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ov = __shfl_xor(best, off);
+      const int oi = __shfl_xor(best_i, off);
+      if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+    }
+    if (lane == 0) {
+      if (best_i == 0x7fffffff) best_i = s.vocab;
+      if (s.tokens_out && pos >= 0 && pos < s.tokens_cap) s.tokens_out[pos] = best_i;
+      s.state[0] = best_i;
+      s.state[1] = pos + 1;
+      st_coherent(s.epoch, base + nph + 1);
+    }
+    stamp();
+  }
+};
+
+template <int KIND, int HD, int NREP>
+__global__ __launch_bounds__(SS_THREADS) void stream_step_kernel(SsArgs s) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  _Float16 *xs = (_Float16 *)smem;
+  float *y_local = (float *)(smem + s.x_bytes);
+  float *att_sc = y_local + SS_YMAX;
+  SsCtl &ctl = *(SsCtl *)(att_sc + SS_NAW * NREP * SS_CHUNK);
+  uint64_t *lt_w = (uint64_t *)(&ctl + 1);   // 8-byte aligned: everything before it is a multiple of 8 bytes
+  uint64_t *pt_w = lt_w + (size_t)s.n_layers * SS_LAYER_WORDS;
+  SsTabs lt;
+  lt.layers = (LtPtr)lt_w;
+  lt.phases = (LtPtr)pt_w;
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int pos = s.state[1];
+  int tok = s.state[0];
+  tok = tok < 0 ? 0 : (tok >= s.vocab ? s.vocab - 1 : tok);
+  if (threadIdx.x < (int)(sizeof(SsCtl) / sizeof(int))) ((int *)&ctl)[threadIdx.x] = 0;
+  for (int i = threadIdx.x; i < s.n_layers * SS_LAYER_WORDS; i += SS_THREADS) lt_w[i] = ldg((const uint64_t *)s.layers + i);
+  for (int p = threadIdx.x; p < ss_phases(s); p += SS_THREADS) ss_build_phase(s, pt_w + (size_t)p * SS_PHASE_WORDS, p);
+  __syncthreads();   // the only block-wide barrier: from here on the wavefronts go their own ways
+
+  if (wave < SS_NWW) SsWeights<KIND>::run(s, lt, ctl, xs, y_local, wave);
+  else if (wave == SS_NWW) SsControl<KIND>::run(s, lt, ctl, xs, y_local, pos, tok);
+  else SsAttn<HD, NREP>::run(s, lt, ctl, att_sc + (wave - SS_NWW - 1) * NREP * SS_CHUNK, wave - SS_NWW - 1, pos);
+}
+
+template <int KIND, int HD> static int launch_stream(const SsArgs &s, int n_rep, int grid, size_t lds) {
+#define JSG_REP(N)                                                                                                              \
+  case N: {                                                                                                                     \
+    static size_t configured = 0;                                                                                               \
+    if (lds > 48 * 1024 && lds > configured) {                                                                                  \
+      JSG_HIP(hipFuncSetAttribute((const void *)stream_step_kernel<KIND, HD, N>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
+      configured = lds;                                                                                                         \
+    }                                                                                                                           \
+    JSG_LAUNCH(PROF_STEP, (stream_step_kernel<KIND, HD, N>), dim3(grid), dim3(SS_THREADS), lds, s);                            \
+  } break;
+  switch (n_rep) {
+    JSG_REP(1) JSG_REP(2) JSG_REP(4)
+    default: return fail("jsgrad_hip_stream_step: n_heads/n_kv_heads = %d is not one of 1,2,4", n_rep);
+  }
+#undef JSG_REP
+  return 0;
+}
+
+}  // namespace jsg
+
+using namespace jsg;
+
+extern "C" {
+
+size_t jsgrad_hip_stream_workspace_bytes(int n_heads, int n_kv_heads, int head_dim) {
+  (void)n_kv_heads;
+  return SS_WS_PARTIAL + (size_t)n_heads * SS_MAXCH * (head_dim + 2) * sizeof(float);
+}
+
+int jsgrad_hip_stream_step(const jsgrad_hip_step_t *d) {
+  const char *who = "jsgrad_hip_stream_step";
+  JSG_READY();
+  JSG_REQUIRE(d && d->layers && d->workspace && d->state && d->h && d->h2 && d->q && d->attn && d->g && d->logits && d->tok_emb && d->out_w && d->final_norm && d->rope_table,
+              "%s: null pointer in the descriptor", who);
+  JSG_REQUIRE(d->act == JSGRAD_F16, "%s: built for fp16 activations", who);
+  JSG_REQUIRE(d->kind == JSGRAD_W_F16 || d->kind == JSGRAD_W_I8, "%s: weight kind %d (fp16 and int8 are built)", who, d->kind);
+  JSG_REQUIRE(d->out_kind == d->kind, "%s: the lm_head must be stored like the layers (kind %d vs %d)", who, d->out_kind, d->kind);
+  JSG_REQUIRE(d->embed_kind == JSGRAD_W_F16 || (d->embed_kind == JSGRAD_W_I8 && d->tok_scale), "%s: embedding kind %d", who, d->embed_kind);
+  JSG_REQUIRE(d->n_layers >= 1 && d->dim > 0 && d->hidden > 0 && d->vocab > 0 && d->max_context > 0, "%s: bad shape", who);
+  JSG_REQUIRE(d->n_kv_heads > 0 && d->n_kv_heads <= 64 && d->n_heads % d->n_kv_heads == 0, "%s: n_heads %d / n_kv_heads %d", who, d->n_heads, d->n_kv_heads);
+  JSG_REQUIRE(d->head_dim == 64 || d->head_dim == 128, "%s: head_dim %d (64 and 128 are built)", who, d->head_dim);
+  const int vec = d->kind == JSGRAD_W_F16 ? 8 : 16;
+  const int qdim = d->n_heads * d->head_dim;
+  JSG_REQUIRE(d->dim % vec == 0 && d->hidden % vec == 0 && qdim % vec == 0, "%s: feature sizes must be multiples of %d", who, vec);
+  JSG_REQUIRE(d->dim % 2 == 0 && d->hidden % 2 == 0 && d->vocab % 2 == 0, "%s: row counts must be even", who);
+  JSG_REQUIRE(d->dim <= SS_NORM_CHUNKS * 64 * 8, "%s: dim %d exceeds the fused RMSNorm limit of %d", who, d->dim, SS_NORM_CHUNKS * 64 * 8);
+  JSG_REQUIRE(d->kind == JSGRAD_W_F16 || d->out_s, "%s: quantised lm_head needs a scale", who);
+  JSG_REQUIRE(d->max_context <= SS_MAXCH * SS_CHUNK, "%s: max_context %d exceeds %d", who, d->max_context, SS_MAXCH * SS_CHUNK);
+  const int grid = state().cu_count;   // one block per CU: every block is resident, which the flags need
+  JSG_REQUIRE(grid <= SS_MAX_BLOCKS, "%s: %d CUs exceed the flag array", who, grid);
+  const int ngw = SS_NWW * grid;
+  auto sums = [&](int rows, int nm) { return ((rows / 2 + ngw - 1) / ngw) * SS_NWW * 2 * nm; };
+  const int most = std::max(std::max(sums(qdim + 2 * d->n_kv_heads * d->head_dim, 1), sums(d->hidden, 2)), std::max(sums(d->dim, 1), sums(d->vocab, 1)));
+  JSG_REQUIRE(most <= SS_YMAX, "%s: %d row sums per block exceed %d", who, most, SS_YMAX);
+  const int n_rep = d->n_heads / d->n_kv_heads;
+  int xe = std::max(ss_x_elems(d->kind, d->dim, 1), ss_x_elems(d->kind, d->dim, 2));
+  xe = std::max(xe, std::max(ss_x_elems(d->kind, qdim, 1), ss_x_elems(d->kind, d->hidden, 1)));
+  const size_t x_bytes = ((size_t)xe * sizeof(_Float16) + 255) & ~(size_t)255;
+  const size_t lds = x_bytes + SS_YMAX * sizeof(float) + (size_t)SS_NAW * n_rep * SS_CHUNK * sizeof(float) + sizeof(SsCtl) + (size_t)d->n_layers * sizeof(SsLayer) +
+                     (size_t)(5 * d->n_layers + 1) * SS_PHASE_WORDS * 8;
+  JSG_REQUIRE(d->n_layers <= 128, "%s: %d layers exceed the LDS table of layer tensors", who, d->n_layers);
+  JSG_REQUIRE(lds <= 160 * 1024, "%s: %zu bytes of LDS needed", who, lds);
+
+  SsArgs s = {};
+  s.layers = (const SsLayer *)d->layers;
+  s.n_layers = d->n_layers; s.dim = d->dim; s.hidden = d->hidden; s.n_heads = d->n_heads; s.n_kv_heads = d->n_kv_heads; s.head_dim = d->head_dim;
+  s.vocab = d->vocab; s.max_context = d->max_context; s.eps = d->eps; s.embed_kind = d->embed_kind;
+  s.tok_emb = d->tok_emb; s.tok_scale = d->tok_scale; s.out_w = d->out_w; s.out_s = d->out_s; s.final_norm = d->final_norm; s.rope_table = d->rope_table;
+  s.state = d->state; s.tokens_out = d->tokens_out; s.tokens_cap = d->tokens_cap;
+  s.h = d->h; s.h2 = d->h2; s.q = d->q; s.attn = d->attn; s.g = d->g; s.logits = d->logits;
+  char *ws = (char *)d->workspace;
+  s.epoch = (int *)(ws + SS_WS_EPOCH);
+  s.err = (int *)(ws + SS_WS_ERR);
+  s.attn_counters = (int *)(ws + SS_WS_COUNTERS);
+  s.amax_val = (float *)(ws + SS_WS_AMAX_VAL);
+  s.amax_idx = (int *)(ws + SS_WS_AMAX_IDX);
+  s.flags = (int *)(ws + SS_WS_FLAGS);
+  s.attn_partial = (float *)(ws + SS_WS_PARTIAL);
+  s.trace = d->trace;
+  s.x_bytes = (int)x_bytes;
+#define JSG_KIND(K)                                                                                  \
+  case K:                                                                                            \
+    return d->head_dim == 64 ? launch_stream<K, 64>(s, n_rep, grid, lds) : launch_stream<K, 128>(s, n_rep, grid, lds);
+  switch (d->kind) {
+    JSG_KIND(JSGRAD_W_F16)
+    JSG_KIND(JSGRAD_W_I8)
+  }
+#undef JSG_KIND
+  return fail("%s: weight kind %d", who, d->kind);
+}
+
+int jsgrad_hip_stream_status(const void *workspace, int *host_out_error) {
+  JSG_READY();
+  JSG_REQUIRE(workspace && host_out_error, "jsgrad_hip_stream_status: null pointer");
+  JSG_REQUIRE(!state().capturing, "jsgrad_hip_stream_status during graph capture");
+  JSG_HIP(hipMemcpyAsync(host_out_error, (const char *)workspace + SS_WS_ERR, sizeof(int), hipMemcpyDeviceToHost, state().stream));
+  JSG_HIP(hipStreamSynchronize(state().stream));
+  return 0;
+}
+
+}  // extern "C"

@@ -72,6 +72,9 @@ SIGNATURES: dict[str, tuple[list, object]] = {
     "jsgrad_hip_step_workspace_bytes": ([_i32, _i32, _i32], _sz),
     "jsgrad_hip_decode_step": ([_vp], _i32),
     "jsgrad_hip_step_status": ([_vp, C.POINTER(_i32)], _i32),
+    "jsgrad_hip_stream_workspace_bytes": ([_i32, _i32, _i32], _sz),
+    "jsgrad_hip_stream_step": ([_vp], _i32),
+    "jsgrad_hip_stream_status": ([_vp, C.POINTER(_i32)], _i32),
     "jsgrad_hip_int8_quantize": ([_vp, _i32, _i32, _vp, _vp, _i32], _i32),
     "jsgrad_hip_int8_dequant": ([_vp, _vp, _i32, _i32, _vp], _i32),
     "jsgrad_hip_nf4_quantize": ([_vp, _sz, _vp, _vp, _i32], _i32),

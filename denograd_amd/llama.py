@@ -167,16 +167,19 @@ class _FusedStep:
     activation rows and the workspace.  Built once per model; plays the role of the GraphRunner that replaces a captured
     list of kernels by one device-side program (engine/jit.ts:71)."""
 
-    def __init__(self, model: "Transformer", ctx: "_Scratch"):
+    def __init__(self, model: "Transformer", ctx: "_Scratch", mode: str = "barrier"):
         lib = ffi.load()
         m = model
+        self.mode = mode   # "barrier": jsgrad_hip_decode_step; "stream": jsgrad_hip_stream_step
         kinds = {l.kind for blk in m.layers for l in (blk.attention.wq, blk.attention.wk, blk.attention.wv, blk.attention.wo,
                                                       blk.feed_forward.w1, blk.feed_forward.w2, blk.feed_forward.w3)}
         if m.dtype != "float16" or len(kinds) != 1 or next(iter(kinds)) not in (ffi.W_F16, ffi.W_I8) or m.output.kind != next(iter(kinds)):
             raise NotImplementedError("the single-kernel step is built for fp16 activations with fp16 or int8 layers and an lm_head stored the same way")
         hd = m.dim // m.n_heads
-        if hd not in (64, 128) or m.n_heads // m.n_kv_heads not in (1, 2, 3, 4):
+        if hd not in (64, 128) or m.n_heads // m.n_kv_heads not in ((1, 2, 4) if mode == "stream" else (1, 2, 3, 4)):
             raise NotImplementedError("the single-kernel step is built for head_dim 64/128 and up to 4 query heads per kv head")
+        if mode == "stream" and (m.dim > 4096 or m.max_context > 8192 or len(m.layers) < 1):
+            raise NotImplementedError("the streaming step is built for dim <= 4096 and max_context <= 8192")
         arr = (ffi.LayerDesc * len(m.layers))()
         p = lambda t: t.ptr if t is not None else None
         for i, blk in enumerate(m.layers):
@@ -187,7 +190,7 @@ class _FusedStep:
                                    blk.attention_norm.weight.ptr, blk.ffn_norm.weight.ptr, a.cache_kv.ptr, a.cache_kv.ptr + half)
         raw = np.frombuffer(bytes(arr), np.uint8) if len(m.layers) else np.zeros(1, np.uint8)
         self.layers = Tensor(raw.copy(), device=m.device)
-        nbytes = lib.jsgrad_hip_step_workspace_bytes(m.n_heads, m.n_kv_heads, hd)
+        nbytes = (lib.jsgrad_hip_stream_workspace_bytes if mode == "stream" else lib.jsgrad_hip_step_workspace_bytes)(m.n_heads, m.n_kv_heads, hd)
         self.workspace = Tensor.zeros((nbytes,), "uint8", m.device)
         emb = m.tok_embeddings
         from .nn import _KIND
@@ -198,11 +201,13 @@ class _FusedStep:
                                  ctx.h.ptr, ctx.h2.ptr, ctx.q.ptr, ctx.attn.ptr, ctx.g.ptr, ctx.logits.ptr, self.workspace.ptr, None)
 
     def launch(self) -> None:
-        check(ffi.load().jsgrad_hip_decode_step(C.byref(self.desc)))
+        lib = ffi.load()
+        check((lib.jsgrad_hip_stream_step if self.mode == "stream" else lib.jsgrad_hip_decode_step)(C.byref(self.desc)))
 
     def error(self) -> int:
         e = C.c_int(0)
-        check(ffi.load().jsgrad_hip_step_status(self.workspace.ptr, C.byref(e)))
+        lib = ffi.load()
+        check((lib.jsgrad_hip_stream_status if self.mode == "stream" else lib.jsgrad_hip_step_status)(self.workspace.ptr, C.byref(e)))
         return e.value
 
 
@@ -269,6 +274,9 @@ class Transformer:
     def dtype(self) -> str:
         return self.tok_embeddings.out_dtype
 
+    def _fused_mode(self) -> str:
+        return "stream" if self.fused_step == "stream" else "barrier"
+
     def _prepare(self) -> _Scratch:
         if self._ctx is None:
             hd = self.dim // self.n_heads
@@ -277,7 +285,7 @@ class Transformer:
             for layer in self.layers:
                 layer.attention._ensure_cache(self.dtype, self.device)
             if self.fused_step:
-                self._fused = _FusedStep(self, self._ctx)      # raises NotImplementedError for models it was not built for
+                self._fused = _FusedStep(self, self._ctx, self._fused_mode())      # raises NotImplementedError for models it was not built for
         return self._ctx
 
     def _step(self) -> Tensor:
@@ -365,7 +373,7 @@ class Transformer:
             if self.forward_jit is not None:
                 self.forward_jit.reset()     # a captured step holds the old cache addresses
             if self._fused is not None:
-                self._fused = _FusedStep(self, ctx)
+                self._fused = _FusedStep(self, ctx, self._fused_mode())
         if tok_dev is None:
             rows.tokens.lazydata.view(n, "int32", 0).ensure_allocated().copyin(toks.reshape(-1))
             tok_dev = rows.tokens
