@@ -333,6 +333,7 @@ def main():
     ap.add_argument("--traffic-probe", action="store_true", help="for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: one 512 MiB device-to-device copy "
                     "(a plain copy kernel of known size, to scale the counters) followed by 4 eager decode steps of --workload; prints nothing")
     ap.add_argument("--fused-step", action="store_true", help="run each token as one persistent kernel (jsgrad_hip_decode_step) instead of one launch per fused op")
+    ap.add_argument("--stream-step", action="store_true", help="run each token as one persistent kernel with streaming wavefronts (jsgrad_hip_stream_step)")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel eagerly instead of replaying a captured HIP graph "
                     "(rocprofv3 --kernel-trace on this image crashes inside hipGraphLaunch, so profiles are taken this way)")
     args = ap.parse_args()
@@ -348,12 +349,13 @@ def main():
     if args.traffic_probe:
         traffic_probe(args.workload)
         return
-    llm, cfg, res = run_workload(args.workload, args.prompt, args.steps, args.warmup, use_graph=not args.no_graph, fused_step=args.fused_step)
+    step_mode = "stream" if args.stream_step else args.fused_step
+    llm, cfg, res = run_workload(args.workload, args.prompt, args.steps, args.warmup, use_graph=not args.no_graph, fused_step=step_mode)
     cpu = None if args.no_cpu else cpu_baseline(llm, cfg)
     del llm
     secondary = None
     if args.secondary:
-        llm2, cfg2, secondary = run_workload(args.secondary, args.prompt, args.secondary_steps, args.warmup, use_graph=not args.no_graph, fused_step=args.fused_step)
+        llm2, cfg2, secondary = run_workload(args.secondary, args.prompt, args.secondary_steps, args.warmup, use_graph=not args.no_graph, fused_step=step_mode)
         del llm2
 
     out = {

@@ -126,7 +126,11 @@ template <> struct Dot<JSGRAD_W_I8, _Float16> {
     const h2_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};  // 1024 + 128
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      uint32_t u = wv[i] ^ 0x80808080u;  // signed byte w -> unsigned w + 128
+      // The empty asm pins the unpacking of this word here.  Left alone, the scheduler unpacks a whole item as its loads
+      // arrive, which doubles the registers the item occupies.
+      uint32_t word = wv[i];
+      asm volatile("" : "+v"(word));
+      uint32_t u = word ^ 0x80808080u;  // signed byte w -> unsigned w + 128
       h2_t lo = as_h2(__builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias;
       h2_t hi = as_h2(__builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias;
       acc = __builtin_amdgcn_fdot2(lo, xf.v[2 * i], acc, false);
@@ -396,7 +400,9 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
             const int kc = k < in_f ? k : in_f - VEC;
             bs = (float)ldg((const _Float16 *)sbase(a, w.m, j) + (((size_t)row * in_f + kc) >> 6));
           }
-          acc[j][r] = Dot<KIND, AT>::run(buf.w[wi(u, j, r)], xf, acc[j][r], bs, lut);
+          // every 16-byte vector is summed on its own and then added: eight short dependent chains per item
+          // instead of two long ones
+          acc[j][r] += Dot<KIND, AT>::run(buf.w[wi(u, j, r)], xf, 0.0f, bs, lut);
         }
     }
     if (b != nbatch(a) - 1) return;

@@ -30,12 +30,15 @@
 
 namespace jsg {
 
-constexpr int SS_NWW = 8;                        // weight wavefronts per block
-constexpr int SS_NAW = 3;                        // attention wavefronts per block
-constexpr int SS_THREADS = (SS_NWW + 1 + SS_NAW) * 64;
+constexpr int SS_NWW = 7;                        // weight wavefronts per block; the eighth wavefront is the control wavefront
+#ifndef SS_NBUF
+#define SS_NBUF 4
+#endif                                           // register buffers (8 x 16 bytes per lane each) of a weight wavefront
+constexpr int SS_THREADS = (SS_NWW + 1) * 64;    // 8 wavefronts per CU = 2 per SIMD: 256 registers per lane
 constexpr int SS_YMAX = 1024;                    // raw row sums a block can hold per phase
 constexpr int SS_CHUNK = 128;                    // most positions per attention item
 constexpr int SS_MAXCH = 64;                     // most attention items per kv head
+constexpr int SS_ATT_LOADS = 12;                 // 128-bit loads of K (and of V) an attention item keeps in flight per lane
 constexpr int SS_FLAG_STRIDE = 32;               // ints between block flags: one 128-byte line each
 constexpr int SS_MAX_BLOCKS = 1024;
 constexpr int SS_SPIN_GLOBAL = 1 << 18;          // polls of ~0.5 us
@@ -72,15 +75,15 @@ struct SsArgs {
 // LDS control words of a block
 struct SsCtl {
   int x_ready;            // weight phases whose input row is staged
-  int go;                 // attention phases released
+  int go;                 // unused
   int abort;              // a bounded wait ran out somewhere: nobody waits any more
   int pad;
   // One progress word per wavefront, not a shared count: a wavefront without work in a phase passes it at once and
   // may be several phases ahead, so a count of completions would say nothing about the slowest wavefront.
-  int wdone[SS_NWW];      // weight phases wavefront w has delivered
-  int adone[4];           // attention phases attention wavefront a has finished (SS_NAW <= 4)
+  int wdone[8];           // weight phases wavefront w has delivered (SS_NWW <= 8)
+  int pad2[4];
 };
-static_assert(SS_NAW <= 4 && sizeof(SsCtl) % 8 == 0, "the table of layer tensors follows the control words, 8-byte aligned");
+static_assert(SS_NWW <= 8 && sizeof(SsCtl) % 8 == 0, "the table of layer tensors follows the control words, 8-byte aligned");
 
 enum { PH_QKV = 0, PH_ATTN = 1, PH_WO = 2, PH_FFN = 3, PH_W2 = 4, PH_LM = 5 };
 
@@ -251,43 +254,52 @@ static int ss_x_elems(int kind, int in_f, int nm) {
 
 struct WBuf { u4_t w[8]; };
 
-// position of a wavefront in its item list: phase, row group, k-batch
+// Work split of a weight phase.  Row groups (2 consecutive rows) are dealt to the blocks round-robin: block b owns groups
+// b, b + G, b + 2G, ...  An item is one k-batch of one group; the items of a block, in (group, batch) order, are dealt to
+// its weight wavefronts round-robin, so the wavefronts of a block differ by at most one item whatever the shapes are.  The
+// partial sum of every item goes to LDS and the control wavefront adds the batches of a row in batch order.
 struct WIter {
-  int p, grp, b, ngroups, nb;
+  int p, t, gl, b;      // phase, item index in the block's list, local group index, k-batch
+  int nitems, nb;       // items of this block in the phase, k-batches per group
   bool live;
   WDesc d;
 };
+__device__ __forceinline__ int ss_block_groups(int ngroups) {   // groups of this block
+  const int G = gridDim.x, b = blockIdx.x;
+  return ngroups > b ? (ngroups - b + G - 1) / G : 0;
+}
 
 template <int KIND> struct SsWeights {
   typedef SsFmt<KIND> F;
 
-  __device__ static __forceinline__ void enter(const SsArgs &s, const SsTabs &lt, WIter &it, int p, int gw) {
+  __device__ static __forceinline__ void enter(const SsArgs &s, const SsTabs &lt, WIter &it, int p, int wave) {
     it.p = p;
     it.d = ss_wdesc(s, lt, p);
-    it.ngroups = wd_groups(it.d);
     it.nb = F::nbatch(it.d);
-    it.grp = gw;
-    it.b = 0;
+    it.nitems = ss_block_groups(wd_groups(it.d)) * it.nb;
+    it.t = wave;
+    it.gl = wave / it.nb;
+    it.b = wave % it.nb;
   }
-  // first phase at or after p in which wavefront gw has an item; when there is none the iterator parks on an item that
-  // exists (group 0 of the lm_head), so that the loads it keeps issuing stay inside a matrix
-  __device__ static __forceinline__ void seek(const SsArgs &s, const SsTabs &lt, WIter &it, int p, int gw) {
+  // first phase at or after p in which this wavefront has an item; when there is none the iterator parks on an item that
+  // exists (the block's first lm_head item), so that the loads it keeps issuing stay inside a matrix
+  __device__ static __forceinline__ void seek(const SsArgs &s, const SsTabs &lt, WIter &it, int p, int wave) {
     const int nph = ss_phases(s);
     while (p < nph) {
-      enter(s, lt, it, p, gw);
-      if (gw < it.ngroups) { it.live = true; return; }
+      enter(s, lt, it, p, wave);
+      if (it.t < it.nitems) { it.live = true; return; }
       p = ss_next_weight(s, p);
     }
     enter(s, lt, it, nph - 1, 0);
     it.live = false;
   }
-  __device__ static __forceinline__ void advance(const SsArgs &s, const SsTabs &lt, WIter &it, int gw, int ngw) {
+  __device__ static __forceinline__ void advance(const SsArgs &s, const SsTabs &lt, WIter &it, int wave) {
     if (!it.live) return;
-    if (++it.b < it.nb) return;
-    it.b = 0;
-    it.grp += ngw;
-    if (it.grp < it.ngroups) return;
-    seek(s, lt, it, ss_next_weight(s, it.p), gw);
+    it.t += SS_NWW;
+    it.b += SS_NWW;
+    while (it.b >= it.nb) { it.b -= it.nb; it.gl++; }
+    if (it.t < it.nitems) return;
+    seek(s, lt, it, ss_next_weight(s, it.p), wave);
   }
 
   // issue the 8 loads of the item the iterator stands on
@@ -295,7 +307,7 @@ template <int KIND> struct SsWeights {
     const WDesc &d = it.d;
     const int lane = threadIdx.x & 63;
     // rows of the group: matrix m of the stacked wq | wk | wv, first row r0 inside it
-    int m = 0, r0 = it.grp * 2;
+    int m = 0, r0 = (blockIdx.x + it.gl * gridDim.x) * 2;
     if (d.nm == 1 && d.rows1 > 0) {
       if (r0 >= d.rows0) { r0 -= d.rows0; m = 1; }
       if (m == 1 && r0 >= d.rows1) { r0 -= d.rows1; m = 2; }
@@ -303,6 +315,7 @@ template <int KIND> struct SsWeights {
     const int mrows = d.rows0 * (m == 0) + d.rows1 * (m == 1) + d.rows2 * (m == 2);
     const uintptr_t base_m = (uintptr_t)d.w0 * (uintptr_t)(m == 0) + (uintptr_t)d.w1 * (uintptr_t)(m == 1) + (uintptr_t)d.w2 * (uintptr_t)(m == 2);
     const int un = F::unroll(d.nm);
+    const size_t row_bytes = ((size_t)d.in_f * F::BITS) / 8;
 #pragma unroll
     for (int v = 0; v < 8; v++) {
       const int u = d.nm == 2 ? v >> 2 : v >> 1, j = d.nm == 2 ? (v >> 1) & 1 : 0, r = v & 1;
@@ -310,22 +323,24 @@ template <int KIND> struct SsWeights {
       k = k < d.in_f ? k : d.in_f - F::VEC;   // lanes past the end reload the last vector; their x is zero
       const int row = r0 + r < mrows ? r0 + r : mrows - 1;
       const uintptr_t base = d.nm == 2 ? (j ? (uintptr_t)d.w1 : (uintptr_t)d.w0) : base_m;
-      const char *p = (const char *)base + (((size_t)row * d.in_f + (size_t)k) * F::BITS) / 8;
-      buf.w[v] = ldg_stream16(p);
+      // wavefront-uniform row address + 32-bit lane offset: the load takes its base from scalar registers and needs
+      // one address register per lane instead of two
+      const char *rowp = (const char *)base + (size_t)row * row_bytes;
+      const uint32_t koff = ((uint32_t)k * F::BITS) / 8;
+      buf.w[v] = ldg_stream16(rowp + koff);
     }
   }
 
-  // consume the item (grp round `round`, batch b) of a phase with NM matrices; on the last batch the row sums go to LDS
+  // consume item t (k-batch b) of a phase with NM matrices: its partial row sums go to LDS
   template <int NM>
-  __device__ static __forceinline__ void consume(const WBuf &buf, int b, int nb, float (&acc)[2][2], const _Float16 *xs, float *y_local, int round, int wave) {
+  __device__ static __forceinline__ void consume(const WBuf &buf, int t, int b, const _Float16 *xs, float *y_local) {
     constexpr int UN = NM == 2 ? 2 : 4;
     const int lane = threadIdx.x & 63;
-    if (b == 0) {
+    float acc[NM][2];
 #pragma unroll
-      for (int j = 0; j < 2; j++)
+    for (int j = 0; j < NM; j++)
 #pragma unroll
-        for (int r = 0; r < 2; r++) acc[j][r] = 0.0f;
-    }
+      for (int r = 0; r < 2; r++) acc[j][r] = 0.0f;
 #pragma unroll
     for (int u = 0; u < UN; u++) {
       const int k = (b * UN + u) * F::STEP + lane * F::VEC;   // may lie in the zero padding of xs
@@ -334,16 +349,15 @@ template <int KIND> struct SsWeights {
 #pragma unroll
       for (int j = 0; j < NM; j++)
 #pragma unroll
-        for (int r = 0; r < 2; r++) acc[j][r] = Dot<KIND, _Float16>::run(buf.w[(u * NM + j) * 2 + r], xf, acc[j][r], 1.0f, nullptr);
+        for (int r = 0; r < 2; r++) acc[j][r] += Dot<KIND, _Float16>::run(buf.w[(u * NM + j) * 2 + r], xf, 0.0f, 1.0f, nullptr);
     }
-    if (b != nb - 1) return;
     float tot[NM][2];
 #pragma unroll
     for (int j = 0; j < NM; j++)
 #pragma unroll
       for (int r = 0; r < 2; r++) tot[j][r] = wave_sum(acc[j][r]);
     if (lane == 0) {
-      float *dst = y_local + ((round * SS_NWW + wave) * NM) * 2;
+      float *dst = y_local + (size_t)t * NM * 2;
 #pragma unroll
       for (int j = 0; j < NM; j++)
 #pragma unroll
@@ -351,62 +365,55 @@ template <int KIND> struct SsWeights {
     }
   }
 
-  // the whole life of a weight wavefront
+  // The whole life of a weight wavefront: ONE flat loop over its items of all phases, unrolled over the register buffers,
+  // so that buffer i is always filled and consumed by the same instructions.  (With the buffer chosen by a run-time
+  // index the compiler can no longer tell the loads of one buffer from those of another and waits for every load in
+  // flight before each item, which is the end of all prefetching.)  The consuming iterator walks the same item list as
+  // the loading one, SS_NBUF items behind.
   __device__ static __forceinline__ void run(const SsArgs &s, const SsTabs &lt, SsCtl &ctl, const _Float16 *xs, float *y_local, int wave) {
-    const int G = gridDim.x, gw = wave * G + blockIdx.x, ngw = SS_NWW * G, nph = ss_phases(s);
-    WIter li;
-    WBuf A, B;
-    seek(s, lt, li, 0, gw);
-    load(A, li);
-    advance(s, lt, li, gw, ngw);
-    load(B, li);
-    advance(s, lt, li, gw, ngw);
-    int n = 0;
-    float acc[2][2];
-    for (int p = 0; p < nph; p = ss_next_weight(s, p)) {
-      const WDesc d = ss_wdesc(s, lt, p);
-      const int ngroups = wd_groups(d), nb = F::nbatch(d);
-      if (gw < ngroups) {
-        lds_wait(s, ctl, &ctl.x_ready, ss_wordinal(s, p) + 1);
-        lds_fence();
-        int round = 0;
-        for (int grp = gw; grp < ngroups; grp += ngw, round++) {
-          for (int b = 0; b < nb; b++) {
-#ifdef JSG_SS_DEBUG
-            if (s.trace && blockIdx.x == 0 && wave == 0 && ss_kind(s, p) == JSG_SS_DEBUG && b == 0 && grp == gw) {
-              uint32_t *dbg = (uint32_t *)s.trace;
-              const int lane = threadIdx.x & 63;
-              for (int v = 0; v < 8; v++)
-                for (int e2 = 0; e2 < 4; e2++) {
-                  dbg[32768 + (v * 64 + lane) * 4 + e2] = A.w[v][e2];
-                  dbg[36864 + (v * 64 + lane) * 4 + e2] = B.w[v][e2];
-                }
-              if (lane == 0) { dbg[40960] = n; dbg[40961] = li.p; dbg[40962] = li.grp; dbg[40963] = li.b; dbg[40964] = li.live; dbg[40965] = nb; dbg[40966] = p; }
-            }
-#endif
-#ifdef JSG_SS_DEBUG
-            if (s.trace && blockIdx.x == 0 && wave == 0 && (threadIdx.x & 63) == 0 && n < 16) {
-              uint32_t *dbg = (uint32_t *)s.trace + 45056 + n * 16;
-              dbg[0] = n; dbg[1] = li.p; dbg[2] = li.grp; dbg[3] = li.b; dbg[4] = (uint32_t)(uintptr_t)li.d.w0; dbg[5] = (uint32_t)((uintptr_t)li.d.w0 >> 32);
-              dbg[6] = li.d.in_f; dbg[7] = li.d.rows0; dbg[8] = li.d.nm; dbg[9] = p; dbg[10] = li.live;
-            }
-#endif
-            if (n & 1) {
-              if (d.nm == 2) consume<2>(B, b, nb, acc, xs, y_local, round, wave);
-              else consume<1>(B, b, nb, acc, xs, y_local, round, wave);
-              load(B, li);
-            } else {
-              if (d.nm == 2) consume<2>(A, b, nb, acc, xs, y_local, round, wave);
-              else consume<1>(A, b, nb, acc, xs, y_local, round, wave);
-              load(A, li);
-            }
-            advance(s, lt, li, gw, ngw);
-            n++;
+    const int n_weight_phases = 4 * s.n_layers + 1;
+    WIter li, ci;
+    WBuf buf[SS_NBUF];   // indexed with compile-time constants only: they live in registers
+    seek(s, lt, li, 0, wave);
+    ci = li;
+#pragma unroll
+    for (int i = 0; i < SS_NBUF; i++) {
+      load(buf[i], li);
+      advance(s, lt, li, wave);
+    }
+    int wtr = 0;
+    auto wstamp = [&](int tag) {   // optional trace of block 0's first weight wavefront: (100 MHz clock, tag) pairs
+      if (s.trace && blockIdx.x == 0 && wave == 0 && (threadIdx.x & 63) == 0 && wtr < 3000) {
+        s.trace[4096 + 2 * wtr] = (long long)__builtin_amdgcn_s_memrealtime();
+        s.trace[4096 + 2 * wtr + 1] = tag;
+        wtr++;
+      }
+    };
+    // phases before the first item need nothing from this wavefront
+    if ((threadIdx.x & 63) == 0) lds_st(&ctl.wdone[wave], ci.live ? ss_wordinal(s, ci.p) : n_weight_phases);
+    int cur_p = -1;
+    while (ci.live) {
+#pragma unroll
+      for (int i = 0; i < SS_NBUF; i++) {
+        if (ci.live) {
+          if (ci.p != cur_p) {   // first item of a phase: its input row must be staged
+            cur_p = ci.p;
+            lds_wait(s, ctl, &ctl.x_ready, ss_wordinal(s, cur_p) + 1);
+            lds_fence();
+            wstamp(1000 + cur_p);
           }
+          if (ci.d.nm == 2) consume<2>(buf[i], ci.t, ci.b, xs, y_local);
+          else consume<1>(buf[i], ci.t, ci.b, xs, y_local);
+          load(buf[i], li);
+          advance(s, lt, li, wave);
+          advance(s, lt, ci, wave);
+          if (!ci.live || ci.p != cur_p) {   // last item of the phase: everything up to the next item's phase is delivered
+            lds_fence();
+            if ((threadIdx.x & 63) == 0) lds_st(&ctl.wdone[wave], ci.live ? ss_wordinal(s, ci.p) : n_weight_phases);
+          }
+          wstamp(i);
         }
       }
-      lds_fence();   // the sums are in LDS before the phase is marked delivered
-      if ((threadIdx.x & 63) == 0) lds_st(&ctl.wdone[wave], ss_wordinal(s, p) + 1);
     }
   }
 };
@@ -426,16 +433,31 @@ template <int HD, int NREP> struct SsAttn {
   static constexpr int RPI = 64 / GL;   // rows per wavefront load
 
   // rows per item for T visible positions when `waves` wavefronts are available per kv head
+  // Rows per item for T visible positions.  The wavefront that merges a kv head fetches the partials of 16 chunks per
+  // round trip and an item fetches up to SS_ATT_LOADS x RPI rows of K and of V per round trip, so up to ~750 positions
+  // (head_dim 128) everything is one round trip each; longer contexts get longer items, at most SS_MAXCH per kv head.
   __device__ static __forceinline__ int chunk_rows(int T, int waves) {
-    int per = waves < SS_MAXCH ? waves : SS_MAXCH;
+    int per = waves < 16 ? waves : 16;
     per = per < 1 ? 1 : per;
-    int chunk = (T + per - 1) / per;
+    int chunk = ((T + per - 1) / per + RPI - 1) / RPI * RPI;
     chunk = chunk < 32 ? 32 : chunk;
-    return chunk > SS_CHUNK ? SS_CHUNK : chunk;   // the host keeps max_context <= SS_MAXCH * SS_CHUNK
+    if (chunk > SS_CHUNK) chunk = SS_CHUNK;   // the host keeps max_context <= SS_MAXCH * SS_CHUNK
+    return chunk;
   }
 
   // item (kv head g, chunk c): scores, softmax numerators and P.V of rows [c * chunk, ...) for the NREP query heads of
   // the kv head; the wavefront that completes the kv head merges all chunks.  sc: this wavefront's LDS float[NREP][SS_CHUNK].
+  // optional trace of block 0's first attention wavefront
+  __device__ static __forceinline__ void astamp(const SsArgs &s, int tag) {
+    if (s.trace && blockIdx.x == 0 && (threadIdx.x & 63) == 0) {
+      const int i = (int)s.trace[12288];
+      if (i < 1500) {
+        s.trace[12290 + 2 * i] = (long long)__builtin_amdgcn_s_memrealtime();
+        s.trace[12291 + 2 * i] = tag;
+        s.trace[12288] = i + 1;
+      }
+    }
+  }
   __device__ static void item(const SsArgs &s, const SsLayer &L, float *sc, int g, int c, int T, int chunk, int n_active) {
     typedef _Float16 AT;
     const int lane = threadIdx.x & 63, sub = lane % GL, grp = lane / GL;
@@ -445,12 +467,12 @@ template <int HD, int NREP> struct SsAttn {
     const AT *vbase = (const AT *)L.cache_v + (size_t)g * HD + (size_t)sub * 8;
     const float scale = (float)(1.0 / sqrt((double)HD));
 
-    // A batch is 8 loads of RPI rows each; the first batch of K and of V goes out at once (most chunks are one batch)
-    constexpr int BR = 8 * RPI;
-    u4_t kraw[8], vraw[8];
-    auto load_batch = [&](u4_t (&raw)[8], const AT *base, int tb) {
+    // A batch is NLD loads of RPI rows each; the first batch of K and of V goes out at once (most chunks are one batch)
+    constexpr int NLD = SS_ATT_LOADS, BR = NLD * RPI;
+    u4_t kraw[NLD], vraw[NLD];
+    auto load_batch = [&](u4_t (&raw)[NLD], const AT *base, int tb) {
 #pragma unroll
-      for (int u = 0; u < 8; u++) {
+      for (int u = 0; u < NLD; u++) {
         const int t = tb + u * RPI + grp;
         raw[u] = ldg((const u4_t *)(base + (size_t)(t < t1 ? t : t1 - 1) * row_stride));
       }
@@ -471,7 +493,7 @@ template <int HD, int NREP> struct SsAttn {
     for (int tb = t0; tb < t1; tb += BR) {
       if (tb != t0) load_batch(kraw, kbase, tb);
 #pragma unroll
-      for (int u = 0; u < 8; u++) {
+      for (int u = 0; u < NLD; u++) {
         const int t = tb + u * RPI + grp;
 #pragma unroll
         for (int j = 0; j < NREP; j++) {
@@ -490,6 +512,7 @@ template <int HD, int NREP> struct SsAttn {
 #pragma unroll
     for (int j = 0; j < NREP; j++) { mx[j] = wave_max(mx[j]); ls[j] = 0.0f; }
     lds_fence();
+    astamp(s, 2);
     for (int i = lane; i < CH; i += 64)
 #pragma unroll
       for (int j = 0; j < NREP; j++) {
@@ -509,7 +532,7 @@ template <int HD, int NREP> struct SsAttn {
     for (int tb = t0; tb < t1; tb += BR) {
       if (tb != t0) load_batch(vraw, vbase, tb);
 #pragma unroll
-      for (int u = 0; u < 8; u++) {
+      for (int u = 0; u < NLD; u++) {
         const int t = tb + u * RPI + grp;
         float vf[8];
 #pragma unroll
@@ -532,6 +555,7 @@ template <int HD, int NREP> struct SsAttn {
         for (int off = GL; off < 64; off <<= 1) v += __shfl_xor(v, off);
         of[j][e] = v;
       }
+    astamp(s, 3);
     float *mine = s.attn_partial + ((size_t)g * SS_MAXCH + c) * NREP * (HD + 2);
     if (grp == 0) {
 #pragma unroll
@@ -546,69 +570,95 @@ template <int HD, int NREP> struct SsAttn {
         st_coherent(&mine[j * (HD + 2) + HD + 1], ls[j]);
       }
     vm_drain();   // the partial is at the coherence point before the item is counted
+    astamp(s, 4);
     int old = 0;
     if (lane == 0) old = __hip_atomic_fetch_add(&s.attn_counters[g], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     old = __builtin_amdgcn_readfirstlane(old);
+    astamp(s, 5);
     if (old != n_active - 1) return;
 
     // ---- merge the chunks of kv head g: weights exp(m_s - M), normalisation 1 / sum(l_s * w_s)
     const float *base = s.attn_partial + (size_t)g * SS_MAXCH * NREP * (HD + 2);
-    float inv[NREP];
+    float inv[NREP], ms[NREP], lsum[NREP];
+    const bool on = lane < n_active;   // n_active <= SS_MAXCH = 64: one chunk per lane
+#pragma unroll
+    for (int j = 0; j < NREP; j++) {   // all (m, l) pairs in one round trip; lanes past the end re-read the last chunk
+      const float *ps = base + ((size_t)(on ? lane : n_active - 1) * NREP + j) * (HD + 2);
+      ms[j] = ld_coherent(ps + HD);
+      lsum[j] = ld_coherent(ps + HD + 1);
+    }
 #pragma unroll
     for (int j = 0; j < NREP; j++) {
-      const bool on = lane < n_active;   // n_active <= SS_MAXCH = 64: one chunk per lane
-      const float *ps = base + ((size_t)(on ? lane : 0) * NREP + j) * (HD + 2);
-      const float ms = on ? ld_coherent(ps + HD) : -INFINITY;
-      const float lsum = on ? ld_coherent(ps + HD + 1) : 0.0f;
-      const float M = wave_max(ms);
-      const float w = on ? exp_f32(ms - M) : 0.0f;
+      ms[j] = on ? ms[j] : -INFINITY;
+      lsum[j] = on ? lsum[j] : 0.0f;
+    }
+#pragma unroll
+    for (int j = 0; j < NREP; j++) {
+      const float M = wave_max(ms[j]);
+      const float w = on ? exp_f32(ms[j] - M) : 0.0f;
       if (on) sc[j * SS_CHUNK + lane] = w;
-      const float Ls = wave_sum(lsum * w);
+      const float Ls = wave_sum(lsum[j] * w);
       inv[j] = 1.0f / Ls;   // softmax normalisation is e * (1/sum) (tensor.ts:2211-2214)
     }
     lds_fence();
+    // Every lane owns NOUT of the NREP x HD outputs; the partials of 8 chunks x NOUT outputs are requested at once
+    // (one round trip per 16 chunks), and summed in chunk order.
+    constexpr int NOUT = NREP * HD / 64;
+    float O[NOUT];
+    int off[NOUT], jj[NOUT];
 #pragma unroll
-    for (int j = 0; j < NREP; j++) {
+    for (int i = 0; i < NOUT; i++) {
+      const int e = i * 64 + lane;
+      jj[i] = e / HD;
+      off[i] = jj[i] * (HD + 2) + e % HD;
+      O[i] = 0.0f;
+    }
+    for (int c2 = 0; c2 < n_active; c2 += 16) {
+      float t16[NOUT][16];
 #pragma unroll
-      for (int d0 = 0; d0 < HD; d0 += 64) {
-        const int d = d0 + lane;
-        const float *po = base + (size_t)j * (HD + 2) + d;
-        float O = 0.0f;
-        for (int c2 = 0; c2 < n_active; c2 += 8) {   // eight independent loads in flight, summed in chunk order
-          float t8[8];
+      for (int u = 0; u < 16; u++) {
+        const size_t cb = (size_t)(c2 + u < n_active ? c2 + u : n_active - 1) * NREP * (HD + 2);
 #pragma unroll
-          for (int u = 0; u < 8; u++) t8[u] = ld_coherent(po + (size_t)(c2 + u < n_active ? c2 + u : n_active - 1) * NREP * (HD + 2));
-#pragma unroll
-          for (int u = 0; u < 8; u++)
-            if (c2 + u < n_active) O = fmaf(t8[u], sc[j * SS_CHUNK + c2 + u], O);
-        }
-        st_coherent((AT *)s.attn + (size_t)(g * NREP + j) * HD + d, (AT)rn16(O * inv[j]));
+        for (int i = 0; i < NOUT; i++) t16[i][u] = ld_coherent(base + cb + off[i]);
       }
+#pragma unroll
+      for (int u = 0; u < 16; u++)
+        if (c2 + u < n_active) {
+#pragma unroll
+          for (int i = 0; i < NOUT; i++) O[i] = fmaf(t16[i][u], sc[jj[i] * SS_CHUNK + c2 + u], O[i]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NOUT; i++) {
+      float iv = inv[0];
+#pragma unroll
+      for (int j = 1; j < NREP; j++) iv = jj[i] == j ? inv[j] : iv;
+      st_coherent((AT *)s.attn + (size_t)g * NREP * HD + i * 64 + lane, (AT)rn16(O[i] * iv));
     }
     if (lane == 0) __hip_atomic_store(&s.attn_counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    astamp(s, 6);
   }
 
-  __device__ static __forceinline__ void run(const SsArgs &s, const SsTabs &lt, SsCtl &ctl, float *sc, int aw, int pos) {
-    const int G = gridDim.x, gid = aw * G + blockIdx.x, na = SS_NAW * G;
+  // the attention phase of layer l as the control wavefront of this block runs it: items block, block + G, ...
+  __device__ static __forceinline__ void phase(const SsArgs &s, const SsTabs &lt, SsCtl &ctl, float *sc, int l, int pos) {
+    const int G = gridDim.x;
     const bool pos_ok = pos >= 0 && pos < s.max_context;
-    for (int l = 0; l < s.n_layers; l++) {
-      lds_wait(s, ctl, &ctl.go, l + 1);
-      if (pos_ok && lds_ld(&ctl.abort) == 0) {
-        const int T = pos + 1;
-        const int chunk = chunk_rows(T, na / s.n_kv_heads);
-        const int n_active = (T + chunk - 1) / chunk;
-        const SsLayer L = ss_layer(lt, l);
-        for (int item_id = gid; item_id < s.n_kv_heads * n_active; item_id += na)
-          item(s, L, sc, item_id / n_active, item_id % n_active, T, chunk, n_active);
-      }
-      vm_drain();   // this wavefront's outputs are at the coherence point
-      if ((threadIdx.x & 63) == 0) lds_st(&ctl.adone[aw], l + 1);
+    astamp(s, 1);
+    if (pos_ok && lds_ld(&ctl.abort) == 0) {
+      const int T = pos + 1;
+      const int chunk = chunk_rows(T, G / s.n_kv_heads);
+      const int n_active = (T + chunk - 1) / chunk;
+      const SsLayer L = ss_layer(lt, l);
+      for (int item_id = blockIdx.x; item_id < s.n_kv_heads * n_active; item_id += G)
+        item(s, L, sc, item_id / n_active, item_id % n_active, T, chunk, n_active);
     }
+    vm_drain();   // this wavefront's outputs are at the coherence point
+    astamp(s, 7);
   }
 };
 
 // ---- the control wavefront -----------------------------------------------------------------------------------------
-template <int KIND> struct SsControl {
+template <int KIND, int HD, int NREP> struct SsControl {
   typedef _Float16 AT;
   typedef SsFmt<KIND> F;
 
@@ -750,17 +800,16 @@ template <int KIND> struct SsControl {
   struct EpiCtx {
     int kind;          // PH_*
     WDesc d;
-    int ngroups;
+    int ngroups, nb;
     const void *residual;
     void *y;
     SsLayer L;
     int pos;
     bool pos_ok;
   };
-  // slot -> stacked row of the phase (or -1): slots are (round, weight wavefront, row of the pair)
+  // slot -> stacked row of the phase (or -1): slot = 2 * (local group of this block) + row of the pair
   __device__ static __forceinline__ int slot_row(const EpiCtx &e, int slot) {
-    const int G = gridDim.x, pair = slot >> 1, w = pair % SS_NWW, round = pair / SS_NWW;
-    const int g = w * G + blockIdx.x + round * (SS_NWW * G);
+    const int g = blockIdx.x + (slot >> 1) * gridDim.x;
     return g < e.ngroups ? 2 * g + (slot & 1) : -1;
   }
   __device__ static __forceinline__ void locate(const WDesc &d, int row, int &m, int &rr) {
@@ -797,13 +846,11 @@ template <int KIND> struct SsControl {
   __device__ static __forceinline__ void epi_apply(const SsArgs &s, const EpiCtx &e, int slot, const EpiOps &o, const float *y_local, float &best, int &best_i) {
     const int row = slot_row(e, slot);
     float v0 = 0.0f, v1 = 0.0f;
-    if (row >= 0) {
-      if (e.d.nm == 2) {
-        const int idx = (slot >> 1) * 4 + (slot & 1);
-        v0 = y_local[idx];
-        v1 = y_local[idx + 2];
-      } else {
-        v0 = y_local[slot];
+    if (row >= 0) {   // the k-batches of the row, added in batch order
+      const float *part = y_local + ((size_t)(slot >> 1) * e.nb * e.d.nm) * 2 + (slot & 1);
+      for (int bb = 0; bb < e.nb; bb++) {
+        v0 += part[(bb * e.d.nm) * 2];
+        if (e.d.nm == 2) v1 += part[(bb * e.d.nm + 1) * 2];
       }
     }
     if constexpr (KIND == JSGRAD_W_I8) { v0 = v0 * o.sc0; v1 = v1 * o.sc1; }
@@ -844,7 +891,7 @@ template <int KIND> struct SsControl {
     }
   }
 
-  __device__ static __forceinline__ void run(const SsArgs &s, const SsTabs &lt, SsCtl &ctl, AT *xs, const float *y_local, int pos, int tok) {
+  __device__ static __forceinline__ void run(const SsArgs &s, const SsTabs &lt, SsCtl &ctl, AT *xs, const float *y_local, float *att_sc, int pos, int tok) {
     const int lane = threadIdx.x & 63, G = gridDim.x, nph = ss_phases(s);
     const bool pos_ok = pos >= 0 && pos < s.max_context;
     const int base = ld_coherent(s.epoch);
@@ -863,15 +910,15 @@ template <int KIND> struct SsControl {
       if (p > 0) wait_flags(s, ctl, base + p);
       stamp();
       if (kind == PH_ATTN) {
-        lds_st(&ctl.go, p / 5 + 1);
         stamp();
-        lds_wait_all(s, ctl, ctl.adone, SS_NAW, p / 5 + 1);
+        SsAttn<HD, NREP>::phase(s, lt, ctl, att_sc, p / 5, pos);
         stamp();
       } else {
         EpiCtx e;
         e.kind = kind;
         e.d = ss_wdesc(s, lt, p);
         e.ngroups = wd_groups(e.d);
+        e.nb = F::nbatch(e.d);
         e.pos = pos;
         e.pos_ok = pos_ok;
         e.L = ss_layer(lt, kind == PH_LM ? 0 : p / 5);
@@ -900,8 +947,7 @@ template <int KIND> struct SsControl {
 #endif
         lds_st(&ctl.x_ready, ss_wordinal(s, p) + 1);
         stamp();
-        const int rounds = (e.ngroups + SS_NWW * G - 1) / (SS_NWW * G);
-        const int nslots = rounds * SS_NWW * 2;
+        const int nslots = ss_block_groups(e.ngroups) * 2;
         EpiOps cur = epi_load(s, e, lane);
         lds_wait_all(s, ctl, ctl.wdone, SS_NWW, ss_wordinal(s, p) + 1);
         lds_fence();
@@ -957,7 +1003,7 @@ __global__ __launch_bounds__(SS_THREADS) void stream_step_kernel(SsArgs s) {
   _Float16 *xs = (_Float16 *)smem;
   float *y_local = (float *)(smem + s.x_bytes);
   float *att_sc = y_local + SS_YMAX;
-  SsCtl &ctl = *(SsCtl *)(att_sc + SS_NAW * NREP * SS_CHUNK);
+  SsCtl &ctl = *(SsCtl *)(att_sc + NREP * SS_CHUNK);
   uint64_t *lt_w = (uint64_t *)(&ctl + 1);   // 8-byte aligned: everything before it is a multiple of 8 bytes
   uint64_t *pt_w = lt_w + (size_t)s.n_layers * SS_LAYER_WORDS;
   SsTabs lt;
@@ -974,8 +1020,7 @@ __global__ __launch_bounds__(SS_THREADS) void stream_step_kernel(SsArgs s) {
   __syncthreads();   // the only block-wide barrier: from here on the wavefronts go their own ways
 
   if (wave < SS_NWW) SsWeights<KIND>::run(s, lt, ctl, xs, y_local, wave);
-  else if (wave == SS_NWW) SsControl<KIND>::run(s, lt, ctl, xs, y_local, pos, tok);
-  else SsAttn<HD, NREP>::run(s, lt, ctl, att_sc + (wave - SS_NWW - 1) * NREP * SS_CHUNK, wave - SS_NWW - 1, pos);
+  else SsControl<KIND, HD, NREP>::run(s, lt, ctl, xs, y_local, att_sc, pos, tok);
 }
 
 template <int KIND, int HD> static int launch_stream(const SsArgs &s, int n_rep, int grid, size_t lds) {
@@ -1028,15 +1073,21 @@ int jsgrad_hip_stream_step(const jsgrad_hip_step_t *d) {
   JSG_REQUIRE(d->max_context <= SS_MAXCH * SS_CHUNK, "%s: max_context %d exceeds %d", who, d->max_context, SS_MAXCH * SS_CHUNK);
   const int grid = state().cu_count;   // one block per CU: every block is resident, which the flags need
   JSG_REQUIRE(grid <= SS_MAX_BLOCKS, "%s: %d CUs exceed the flag array", who, grid);
-  const int ngw = SS_NWW * grid;
-  auto sums = [&](int rows, int nm) { return ((rows / 2 + ngw - 1) / ngw) * SS_NWW * 2 * nm; };
-  const int most = std::max(std::max(sums(qdim + 2 * d->n_kv_heads * d->head_dim, 1), sums(d->hidden, 2)), std::max(sums(d->dim, 1), sums(d->vocab, 1)));
-  JSG_REQUIRE(most <= SS_YMAX, "%s: %d row sums per block exceed %d", who, most, SS_YMAX);
+  // partial sums a block holds in LDS per phase: groups per block x k-batches x matrices x 2 rows
+  const int step_k = 64 * (d->kind == JSGRAD_W_F16 ? 8 : 16);
+  auto sums = [&](int rows, int in_f, int nm) {
+    const int u = nm == 2 ? 2 : 4, nb = ((in_f + step_k - 1) / step_k + u - 1) / u;
+    return ((rows / 2 + grid - 1) / grid) * nb * nm * 2;
+  };
+  const int most = std::max(std::max(sums(qdim + 2 * d->n_kv_heads * d->head_dim, d->dim, 1), sums(d->hidden, d->dim, 2)),
+                            std::max(std::max(sums(d->dim, qdim, 1), sums(d->dim, d->hidden, 1)), sums(d->vocab, d->dim, 1)));
+  JSG_REQUIRE(most <= SS_YMAX, "%s: %d partial sums per block exceed %d", who, most, SS_YMAX);
+  JSG_REQUIRE(d->vocab >= 2 * grid, "%s: vocab %d is smaller than two rows per block", who, d->vocab);
   const int n_rep = d->n_heads / d->n_kv_heads;
   int xe = std::max(ss_x_elems(d->kind, d->dim, 1), ss_x_elems(d->kind, d->dim, 2));
   xe = std::max(xe, std::max(ss_x_elems(d->kind, qdim, 1), ss_x_elems(d->kind, d->hidden, 1)));
   const size_t x_bytes = ((size_t)xe * sizeof(_Float16) + 255) & ~(size_t)255;
-  const size_t lds = x_bytes + SS_YMAX * sizeof(float) + (size_t)SS_NAW * n_rep * SS_CHUNK * sizeof(float) + sizeof(SsCtl) + (size_t)d->n_layers * sizeof(SsLayer) +
+  const size_t lds = x_bytes + SS_YMAX * sizeof(float) + (size_t)n_rep * SS_CHUNK * sizeof(float) + sizeof(SsCtl) + (size_t)d->n_layers * sizeof(SsLayer) +
                      (size_t)(5 * d->n_layers + 1) * SS_PHASE_WORDS * 8;
   JSG_REQUIRE(d->n_layers <= 128, "%s: %d layers exceed the LDS table of layer tensors", who, d->n_layers);
   JSG_REQUIRE(lds <= 160 * 1024, "%s: %zu bytes of LDS needed", who, lds);
