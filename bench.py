@@ -159,7 +159,8 @@ def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=Tru
         step_ms = kinds["decode_step"]["ms_per_step"]
         bytes_now = synthetic.weight_bytes_per_token(cfg) + synthetic.kv_bytes_per_position(cfg) * llm.start_pos
         achieved = bytes_now / (step_ms * 1e-3) / 1e9
-        roof = {"bound": "hbm", "kernel": "decode_step_kernel (whole token: embedding, 5 phases x layers, lm_head, argmax)", "achieved": round(achieved, 1),
+        kern = "stream_step_kernel" if m._fused.mode == "stream" else "decode_step_kernel"
+        roof = {"bound": "hbm", "kernel": f"{kern} (whole token: embedding, 5 phases x layers, lm_head, argmax)", "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get((name, "decode_step")),
                 "bytes_per_launch": int(bytes_now), "avg_us_per_launch": round(step_ms * 1e3, 2)}
     else:

@@ -854,15 +854,6 @@ template <int KIND, int HD, int NREP> struct SsControl {
       }
     }
     if constexpr (KIND == JSGRAD_W_I8) { v0 = v0 * o.sc0; v1 = v1 * o.sc1; }
-#ifdef JSG_SS_DEBUG
-    if (s.trace && row >= 0 && e.kind == JSG_SS_DEBUG) {
-      float *dbg = (float *)s.trace;
-      dbg[row * 4 + 0] = v0;
-      dbg[row * 4 + 1] = o.e0;
-      dbg[row * 4 + 2] = (float)blockIdx.x;
-      dbg[row * 4 + 3] = (float)slot;
-    }
-#endif
     v0 = rn16(v0);
     v1 = rn16(v1);
     // the other row of the pair sits in the neighbouring lane
@@ -897,9 +888,6 @@ template <int KIND, int HD, int NREP> struct SsControl {
     const int base = ld_coherent(s.epoch);
     int tr = 0;
     auto stamp = [&]() {
-#ifdef JSG_SS_DEBUG
-      return;
-#endif
       if (s.trace && blockIdx.x == 0 && lane == 0 && tr < 2040) s.trace[tr++] = (long long)__builtin_amdgcn_s_memrealtime();
     };
     stamp();
@@ -939,12 +927,6 @@ template <int KIND, int HD, int NREP> struct SsControl {
         if (emb_i8) stage_x<true>(s, xs, src, norm_w, e.d.in_f, padded, inv_d, emb_scale, mirror);
         else stage_x<false>(s, xs, src, norm_w, e.d.in_f, padded, inv_d, emb_scale, mirror);
         lds_fence();
-#ifdef JSG_SS_DEBUG
-        if (s.trace && blockIdx.x == 0 && kind == JSG_SS_DEBUG) {
-          float *dbg = (float *)s.trace + 16384;
-          for (int i = lane; i < padded; i += 64) dbg[i] = (float)xs[i];
-        }
-#endif
         lds_st(&ctl.x_ready, ss_wordinal(s, p) + 1);
         stamp();
         const int nslots = ss_block_groups(e.ngroups) * 2;

@@ -229,9 +229,10 @@ int jsgrad_hip_decode_step(const jsgrad_hip_step_t *host_desc);
 int jsgrad_hip_step_status(const void *workspace, int *host_out_error);
 
 /* The same step (same descriptor, same results) with role-specialised wavefronts instead of phase-by-phase blocks: in
- * every resident block eight wavefronts only stream weights through all phases of the step, so the loads of the next
- * phase are in flight while the current one is handed over; one wavefront owns the hand-offs (input row -> LDS with the
- * RMSNorm, row epilogues, block flags) and three run the attention items.  Stands for the same reference interfaces as
+ * every resident block seven wavefronts only stream weights through all phases of the step, each with four register
+ * buffers, so the loads of the next phase are in flight while the current one is handed over; the eighth wavefront owns
+ * the hand-offs (input row -> LDS with the RMSNorm, row epilogues, block flags) and the attention items.  fp16
+ * activations with fp16 or int8 weights (lm_head in the same format).  Stands for the same reference interfaces as
  * jsgrad_hip_decode_step (engine/jit.ts:71,190-217; models/llama.ts:201-220).  The workspace has its own layout:
  * jsgrad_hip_stream_workspace_bytes() bytes, zero-filled once before first use.  head_dim 64 or 128, 1, 2 or 4 query
  * heads per kv head, dim <= 4096, max_context <= 8192. */
