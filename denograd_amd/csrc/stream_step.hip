@@ -70,6 +70,7 @@ struct SsArgs {
   int *amax_idx;
   long long *trace;
   int x_bytes;           // LDS bytes reserved for the staged input row
+  int grid;              // blocks of the launch (gridDim.x costs a trip to the dispatch packet wherever it is used)
 };
 
 // LDS control words of a block
@@ -97,7 +98,7 @@ enum { PH_QKV = 0, PH_ATTN = 1, PH_WO = 2, PH_FFN = 3, PH_W2 = 4, PH_LM = 5 };
 typedef const __attribute__((address_space(3))) uint64_t *LtPtr;
 struct SsTabs { LtPtr layers, phases; };
 constexpr int SS_LAYER_WORDS = sizeof(SsLayer) / 8;
-constexpr int SS_PHASE_WORDS = 14;   // w0 w1 w2 s0 s1 s2 src norm_w residual y (rows0,rows1) (rows2,in_f) (nm,kind) pad
+constexpr int SS_PHASE_WORDS = 16;   // w0 w1 w2 s0 s1 s2 src norm_w residual y (rows0,rows1) (rows2,in_f) (nm,kind) + three words of the item walk
 // a value that is the same in every lane, moved to scalar registers
 __device__ __forceinline__ uint64_t uni64(uint64_t v) {
   const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
@@ -192,7 +193,8 @@ __device__ __forceinline__ int ss_next_weight(const SsArgs &s, int p) {
   return p;
 }
 // record of phase p, written by one thread (per-lane code: the selects below are plain conditional moves)
-__device__ __forceinline__ void ss_build_phase(const SsArgs &s, uint64_t *rec, int p) {
+// vec: weight elements per 16-byte load (the walk over the items depends on the weight format)
+__device__ __forceinline__ void ss_build_phase(const SsArgs &s, uint64_t *rec, int p, int vec) {
   const int k = ss_kind(s, p);
   const int l = k == PH_LM ? s.n_layers - 1 : p / 5;
   const uint64_t *L = (const uint64_t *)s.layers + (size_t)l * SS_LAYER_WORDS;
@@ -220,7 +222,19 @@ __device__ __forceinline__ void ss_build_phase(const SsArgs &s, uint64_t *rec, i
   rec[10] = (uint32_t)rows0 | ((uint64_t)(uint32_t)rows1 << 32);
   rec[11] = (uint32_t)rows2 | ((uint64_t)(uint32_t)in_f << 32);
   rec[12] = (uint32_t)nm | ((uint64_t)(uint32_t)k << 32);
-  rec[13] = 0;
+  // the walk of this block's weight wavefronts over the items of the phase
+  uint64_t cnt = 0, str = 0, first = 0;
+  if (in_f > 0) {
+    const int step = 64 * vec, un = nm == 2 ? 2 : 4;
+    const int nb = ((in_f + step - 1) / step + un - 1) / un;
+    const int rows = rows0 + (nm == 1 ? rows1 + rows2 : 0), ngroups = (rows + 1) >> 1;
+    const int G = gridDim.x, blk = blockIdx.x;
+    const int mine = ngroups > blk ? (ngroups - blk + G - 1) / G : 0;
+    cnt = (uint32_t)nb | ((uint64_t)(uint32_t)(mine * nb) << 32);
+    str = (uint32_t)(in_f * 16 / vec) | ((uint64_t)(uint32_t)(SS_NWW / nb) << 32) | ((uint64_t)(uint32_t)(SS_NWW % nb) << 48);
+    for (int w = 0; w < SS_NWW; w++) first |= ((uint64_t)(uint32_t)(w / nb) << (4 * w)) | ((uint64_t)(uint32_t)(w % nb) << (32 + 4 * w));
+  }
+  rec[13] = cnt; rec[14] = str; rec[15] = first;
 }
 // the record of phase p, in scalar registers
 __device__ __forceinline__ WDesc ss_wdesc(const SsArgs &s, const SsTabs &lt, int p) {
@@ -258,77 +272,163 @@ struct WBuf { u4_t w[8]; };
 // b, b + G, b + 2G, ...  An item is one k-batch of one group; the items of a block, in (group, batch) order, are dealt to
 // its weight wavefronts round-robin, so the wavefronts of a block differ by at most one item whatever the shapes are.  The
 // partial sum of every item goes to LDS and the control wavefront adds the batches of a row in batch order.
-struct WIter {
-  int p, t, gl, b;      // phase, item index in the block's list, local group index, k-batch
-  int nitems, nb;       // items of this block in the phase, k-batches per group
-  bool live;
-  WDesc d;
-};
 __device__ __forceinline__ int ss_block_groups(int ngroups) {   // groups of this block
   const int G = gridDim.x, b = blockIdx.x;
   return ngroups > b ? (ngroups - b + G - 1) / G : 0;
 }
 
+// Everything a weight wavefront does per item is on its critical path (two of them share a SIMD and an item is only 8 KiB),
+// so whatever depends on the phase alone is worked out once per block when the phase table is built (words 13-15 of a
+// record) and the walk over the items is a handful of scalar adds:
+//   word 13: k-batches per group | items of this block
+//   word 14: bytes per weight row | (SS_NWW / nb) | (SS_NWW % nb) << 16
+//   word 15: for wavefront w, 4 bits each: w / nb at bit 4w, w % nb at bit 32 + 4w
+struct WIter {
+  int p, w;             // phase and its ordinal among the weight phases
+  int t, gl, b;         // item index in the block's list, local group index, k-batch
+  bool live;
+  // of the phase
+  int nitems, nb, step_gl, step_b, rows0, rows1, grid;
+  uint32_t row_bytes;
+  bool nm2;
+  // of the item: first row inside its matrix, and the matrix pointer(s) as read from the LDS record (per lane, not yet
+  // moved to scalar registers: the read is issued when the iterator moves and waited for when the loads are issued)
+  int row;
+  uint64_t raw0, raw1;
+};
+// what the consumer of a register buffer needs to know about the item in it
+struct WRec {
+  int t, b, w;
+  bool nm2, live;
+};
+
+// v[i] + v[i ^ 16] + v[i ^ 32] + v[i ^ 48] in every lane i, through the two row-swap instructions of the vector ALU (no
+// trip through LDS): with both operands holding v, one swap leaves "v of my half" in one and "v of the other half" in the other
+__device__ __forceinline__ float ss_rows_sum(float v) {
+  const uint32_t a = __float_as_uint(v);
+  const auto h = __builtin_amdgcn_permlane16_swap(a, a, false, false);   // rows 1 and 3 of the first <-> rows 0 and 2 of the second
+  const uint32_t b = __float_as_uint(__uint_as_float(h[0]) + __uint_as_float(h[1]));
+  const auto w = __builtin_amdgcn_permlane32_swap(b, b, false, false);   // upper half of the first <-> lower half of the second
+  return __uint_as_float(w[0]) + __uint_as_float(w[1]);
+}
+
+// Totals of four per-lane values over the wavefront: every lane gets the total of value (lane & 3).  Two exchange steps
+// halve the number of values a lane carries, the rest adds lanes that carry the same value.
+__device__ __forceinline__ float ss_reduce4(float v0, float v1, float v2, float v3) {
+  const int lane = threadIdx.x & 63;
+  const bool o1 = (lane & 1) != 0, o2 = (lane & 2) != 0;
+  float k0 = o1 ? v1 : v0, s0 = o1 ? v0 : v1;
+  float k1 = o1 ? v3 : v2, s1 = o1 ? v2 : v3;
+  k0 += dpp_f<0xB1>(s0);   // quad_perm [1,0,3,2]: value (lane & 1) of the pair
+  k1 += dpp_f<0xB1>(s1);   //                      value 2 + (lane & 1)
+  float k = o2 ? k1 : k0;
+  const float sd = o2 ? k0 : k1;
+  k += dpp_f<0x4E>(sd);    // quad_perm [2,3,0,1]: value (lane & 3) of the quad
+  k += dpp_f<0x124>(k);    // row_ror:4
+  k += dpp_f<0x128>(k);    // row_ror:8: value (lane & 3) of the 16-lane row
+  return ss_rows_sum(k);
+}
+// the same for two values: every lane gets the total of value (lane & 1)
+__device__ __forceinline__ float ss_reduce2(float v0, float v1) {
+  const int lane = threadIdx.x & 63;
+  const bool o1 = (lane & 1) != 0;
+  float k = o1 ? v1 : v0;
+  const float sd = o1 ? v0 : v1;
+  k += dpp_f<0xB1>(sd);
+  k += dpp_f<0x4E>(k);
+  k += dpp_f<0x124>(k);
+  k += dpp_f<0x128>(k);
+  return ss_rows_sum(k);
+}
+
 template <int KIND> struct SsWeights {
   typedef SsFmt<KIND> F;
+  static constexpr uint32_t STEP_BYTES = 64 * 16;   // bytes one k-step of the wavefront covers in a weight row
 
-  __device__ static __forceinline__ void enter(const SsArgs &s, const SsTabs &lt, WIter &it, int p, int wave) {
-    it.p = p;
-    it.d = ss_wdesc(s, lt, p);
-    it.nb = F::nbatch(it.d);
-    it.nitems = ss_block_groups(wd_groups(it.d)) * it.nb;
-    it.t = wave;
-    it.gl = wave / it.nb;
-    it.b = wave % it.nb;
+  // items of this block in phase p
+  __device__ static __forceinline__ int phase_items(const SsTabs &lt, int p) {
+    return (int)(uint32_t)(uni64(lt.phases[(size_t)p * SS_PHASE_WORDS + 13]) >> 32);
   }
-  // first phase at or after p in which this wavefront has an item; when there is none the iterator parks on an item that
-  // exists (the block's first lm_head item), so that the loads it keeps issuing stay inside a matrix
-  __device__ static __forceinline__ void seek(const SsArgs &s, const SsTabs &lt, WIter &it, int p, int wave) {
+  __device__ static __forceinline__ void enter(const SsTabs &lt, WIter &it, int p, int w, int wave) {
+    LtPtr r = lt.phases + (size_t)p * SS_PHASE_WORDS;
+    const uint64_t rows = uni64(r[10]), kind = uni64(r[12]), cnt = uni64(r[13]), str = uni64(r[14]), first = uni64(r[15]);
+    it.p = p;
+    it.w = w;
+    it.rows0 = (int)(uint32_t)rows;
+    it.rows1 = (int)(rows >> 32);
+    it.nm2 = (uint32_t)kind == 2u;
+    it.nb = (int)(uint32_t)cnt;
+    it.nitems = (int)(cnt >> 32);
+    it.row_bytes = (uint32_t)str;
+    it.step_gl = (int)((str >> 32) & 0xffff);
+    it.step_b = (int)(str >> 48);
+    it.t = wave;
+    it.gl = (int)((first >> (4 * wave)) & 15);
+    it.b = (int)((first >> (32 + 4 * wave)) & 15);
+    locate(lt, it);
+  }
+  // Matrix and row of the item the iterator stands on.  The matrix pointers come out of the LDS record by index (the stacked
+  // wq | wk | wv have one each); every row count is even, so both rows of a group are in one matrix.
+  __device__ static __forceinline__ void locate(const SsTabs &lt, WIter &it) {
+    LtPtr r = lt.phases + (size_t)it.p * SS_PHASE_WORDS;
+    int row = (blockIdx.x + it.gl * it.grid) * 2;
+    const int in1 = row >= it.rows0 ? 1 : 0;                  // rows1 is 0 unless the phase stacks three matrices,
+    const int in2 = row >= it.rows0 + it.rows1 ? in1 : 0;     // and then no row reaches past rows0
+    const int m = it.rows1 > 0 ? in1 + in2 : 0;
+    it.row = row - (it.rows1 > 0 ? in1 * it.rows0 + in2 * it.rows1 : 0);
+    it.raw0 = r[m];
+    it.raw1 = r[m + (it.nm2 ? 1 : 0)];
+  }
+  // first phase at or after p (ordinal w) in which this wavefront has an item; when there is none the iterator parks on
+  // an item that exists (the block's first lm_head item), so that the loads it keeps issuing stay inside a matrix
+  __device__ static __forceinline__ void seek(const SsArgs &s, const SsTabs &lt, WIter &it, int p, int w, int wave) {
     const int nph = ss_phases(s);
     while (p < nph) {
-      enter(s, lt, it, p, wave);
-      if (it.t < it.nitems) { it.live = true; return; }
+      if (wave < phase_items(lt, p)) {
+        enter(lt, it, p, w, wave);
+        it.live = true;
+        return;
+      }
       p = ss_next_weight(s, p);
+      w++;
     }
-    enter(s, lt, it, nph - 1, 0);
+    enter(lt, it, nph - 1, 4 * s.n_layers, 0);
     it.live = false;
   }
   __device__ static __forceinline__ void advance(const SsArgs &s, const SsTabs &lt, WIter &it, int wave) {
     if (!it.live) return;
     it.t += SS_NWW;
-    it.b += SS_NWW;
-    while (it.b >= it.nb) { it.b -= it.nb; it.gl++; }
-    if (it.t < it.nitems) return;
-    seek(s, lt, it, ss_next_weight(s, it.p), wave);
+    it.gl += it.step_gl;
+    it.b += it.step_b;
+    if (it.b >= it.nb) { it.b -= it.nb; it.gl++; }
+    if (it.t < it.nitems) { locate(lt, it); return; }
+    seek(s, lt, it, ss_next_weight(s, it.p), it.w + 1, wave);
   }
+  __device__ static __forceinline__ WRec record(const WIter &it) { return WRec{it.t, it.b, it.w, it.nm2, it.live}; }
 
-  // issue the 8 loads of the item the iterator stands on
+  // Issue the 8 loads of the item the iterator stands on.  Load v = a*4 + c*2 + r is row r of the group; with one matrix
+  // it is k-step a*2 + c of the batch, with two it is k-step a of matrix c.
   __device__ static __forceinline__ void load(WBuf &buf, const WIter &it) {
-    const WDesc &d = it.d;
-    const int lane = threadIdx.x & 63;
-    // rows of the group: matrix m of the stacked wq | wk | wv, first row r0 inside it
-    int m = 0, r0 = (blockIdx.x + it.gl * gridDim.x) * 2;
-    if (d.nm == 1 && d.rows1 > 0) {
-      if (r0 >= d.rows0) { r0 -= d.rows0; m = 1; }
-      if (m == 1 && r0 >= d.rows1) { r0 -= d.rows1; m = 2; }
-    }
-    const int mrows = d.rows0 * (m == 0) + d.rows1 * (m == 1) + d.rows2 * (m == 2);
-    const uintptr_t base_m = (uintptr_t)d.w0 * (uintptr_t)(m == 0) + (uintptr_t)d.w1 * (uintptr_t)(m == 1) + (uintptr_t)d.w2 * (uintptr_t)(m == 2);
-    const int un = F::unroll(d.nm);
-    const size_t row_bytes = ((size_t)d.in_f * F::BITS) / 8;
+    const uint32_t lane16 = (threadIdx.x & 63) * 16;
+    const uint64_t rowoff = (uint64_t)(uint32_t)it.row * it.row_bytes;
+    const char *base[4];
+    base[0] = (const char *)(uintptr_t)(uni64(it.raw0) + rowoff);
+    base[1] = base[0] + it.row_bytes;
+    base[2] = (const char *)(uintptr_t)(uni64(it.raw1) + rowoff);
+    base[3] = base[2] + it.row_bytes;
+    const uint32_t un = it.nm2 ? 2u : 4u;
+    const uint32_t k0 = (uint32_t)it.b * un * STEP_BYTES;
+    const uint32_t last = it.row_bytes - 16;   // lanes past the end of the row reload its last vector; their x is zero
 #pragma unroll
-    for (int v = 0; v < 8; v++) {
-      const int u = d.nm == 2 ? v >> 2 : v >> 1, j = d.nm == 2 ? (v >> 1) & 1 : 0, r = v & 1;
-      int k = (it.b * un + u) * F::STEP + lane * F::VEC;
-      k = k < d.in_f ? k : d.in_f - F::VEC;   // lanes past the end reload the last vector; their x is zero
-      const int row = r0 + r < mrows ? r0 + r : mrows - 1;
-      const uintptr_t base = d.nm == 2 ? (j ? (uintptr_t)d.w1 : (uintptr_t)d.w0) : base_m;
-      // wavefront-uniform row address + 32-bit lane offset: the load takes its base from scalar registers and needs
-      // one address register per lane instead of two
-      const char *rowp = (const char *)base + (size_t)row * row_bytes;
-      const uint32_t koff = ((uint32_t)k * F::BITS) / 8;
-      buf.w[v] = ldg_stream16(rowp + koff);
-    }
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+      for (int c = 0; c < 2; c++) {
+        const uint32_t ks = it.nm2 ? (uint32_t)a : (uint32_t)(a * 2 + c);
+        uint32_t koff = k0 + ks * STEP_BYTES + lane16;
+        koff = koff < last ? koff : last;
+#pragma unroll
+        for (int rr = 0; rr < 2; rr++) buf.w[a * 4 + c * 2 + rr] = ldg_stream16(base[c * 2 + rr] + koff);
+      }
   }
 
   // consume item t (k-batch b) of a phase with NM matrices: its partial row sums go to LDS
@@ -351,33 +451,32 @@ template <int KIND> struct SsWeights {
 #pragma unroll
         for (int r = 0; r < 2; r++) acc[j][r] += Dot<KIND, _Float16>::run(buf.w[(u * NM + j) * 2 + r], xf, 0.0f, 1.0f, nullptr);
     }
-    float tot[NM][2];
-#pragma unroll
-    for (int j = 0; j < NM; j++)
-#pragma unroll
-      for (int r = 0; r < 2; r++) tot[j][r] = wave_sum(acc[j][r]);
-    if (lane == 0) {
-      float *dst = y_local + (size_t)t * NM * 2;
-#pragma unroll
-      for (int j = 0; j < NM; j++)
-#pragma unroll
-        for (int r = 0; r < 2; r++) dst[j * 2 + r] = tot[j][r];
+    float *dst = y_local + (size_t)t * NM * 2;
+    if constexpr (NM == 2) {
+      const float tot = ss_reduce4(acc[0][0], acc[0][1], acc[1][0], acc[1][1]);
+      if (lane < 4) dst[lane] = tot;
+    } else {
+      const float tot = ss_reduce2(acc[0][0], acc[0][1]);
+      if (lane < 2) dst[lane] = tot;
     }
   }
 
   // The whole life of a weight wavefront: ONE flat loop over its items of all phases, unrolled over the register buffers,
   // so that buffer i is always filled and consumed by the same instructions.  (With the buffer chosen by a run-time
   // index the compiler can no longer tell the loads of one buffer from those of another and waits for every load in
-  // flight before each item, which is the end of all prefetching.)  The consuming iterator walks the same item list as
-  // the loading one, SS_NBUF items behind.
+  // flight before each item, which is the end of all prefetching.)  One iterator walks the item list, SS_NBUF items ahead
+  // of the arithmetic; a small record per buffer tells the consumer what the buffer holds.  The loads are unconditional
+  // (a parked iterator re-reads an existing item) so that the number of loads in flight is the same on every path.
   __device__ static __forceinline__ void run(const SsArgs &s, const SsTabs &lt, SsCtl &ctl, const _Float16 *xs, float *y_local, int wave) {
     const int n_weight_phases = 4 * s.n_layers + 1;
-    WIter li, ci;
+    WIter li;
+    li.grid = s.grid;
+    WRec rec[SS_NBUF];
     WBuf buf[SS_NBUF];   // indexed with compile-time constants only: they live in registers
-    seek(s, lt, li, 0, wave);
-    ci = li;
+    seek(s, lt, li, 0, 0, wave);
 #pragma unroll
     for (int i = 0; i < SS_NBUF; i++) {
+      rec[i] = record(li);
       load(buf[i], li);
       advance(s, lt, li, wave);
     }
@@ -390,29 +489,30 @@ template <int KIND> struct SsWeights {
       }
     };
     // phases before the first item need nothing from this wavefront
-    if ((threadIdx.x & 63) == 0) lds_st(&ctl.wdone[wave], ci.live ? ss_wordinal(s, ci.p) : n_weight_phases);
-    int cur_p = -1;
-    while (ci.live) {
+    if ((threadIdx.x & 63) == 0) lds_st(&ctl.wdone[wave], rec[0].live ? rec[0].w : n_weight_phases);
+    int cur_w = -1;
+    while (rec[0].live) {
 #pragma unroll
       for (int i = 0; i < SS_NBUF; i++) {
-        if (ci.live) {
-          if (ci.p != cur_p) {   // first item of a phase: its input row must be staged
-            cur_p = ci.p;
-            lds_wait(s, ctl, &ctl.x_ready, ss_wordinal(s, cur_p) + 1);
+        if (rec[i].live) {
+          if (rec[i].w != cur_w) {   // first item of a phase: its input row must be staged
+            cur_w = rec[i].w;
+            lds_wait(s, ctl, &ctl.x_ready, cur_w + 1);
             lds_fence();
-            wstamp(1000 + cur_p);
+            wstamp(1000 + cur_w);
           }
-          if (ci.d.nm == 2) consume<2>(buf[i], ci.t, ci.b, xs, y_local);
-          else consume<1>(buf[i], ci.t, ci.b, xs, y_local);
-          load(buf[i], li);
-          advance(s, lt, li, wave);
-          advance(s, lt, ci, wave);
-          if (!ci.live || ci.p != cur_p) {   // last item of the phase: everything up to the next item's phase is delivered
-            lds_fence();
-            if ((threadIdx.x & 63) == 0) lds_st(&ctl.wdone[wave], ci.live ? ss_wordinal(s, ci.p) : n_weight_phases);
-          }
-          wstamp(i);
+          if (rec[i].nm2) consume<2>(buf[i], rec[i].t, rec[i].b, xs, y_local);
+          else consume<1>(buf[i], rec[i].t, rec[i].b, xs, y_local);
         }
+        rec[i] = record(li);
+        load(buf[i], li);
+        advance(s, lt, li, wave);
+        const WRec &nxt = rec[(i + 1) % SS_NBUF];
+        if (cur_w >= 0 && (!nxt.live || nxt.w != cur_w)) {   // last item of the phase: everything before the next item's phase is delivered
+          lds_fence();
+          if ((threadIdx.x & 63) == 0) lds_st(&ctl.wdone[wave], nxt.live ? nxt.w : n_weight_phases);
+        }
+        wstamp(i);
       }
     }
   }
@@ -998,7 +1098,7 @@ __global__ __launch_bounds__(SS_THREADS) void stream_step_kernel(SsArgs s) {
   tok = tok < 0 ? 0 : (tok >= s.vocab ? s.vocab - 1 : tok);
   if (threadIdx.x < (int)(sizeof(SsCtl) / sizeof(int))) ((int *)&ctl)[threadIdx.x] = 0;
   for (int i = threadIdx.x; i < s.n_layers * SS_LAYER_WORDS; i += SS_THREADS) lt_w[i] = ldg((const uint64_t *)s.layers + i);
-  for (int p = threadIdx.x; p < ss_phases(s); p += SS_THREADS) ss_build_phase(s, pt_w + (size_t)p * SS_PHASE_WORDS, p);
+  for (int p = threadIdx.x; p < ss_phases(s); p += SS_THREADS) ss_build_phase(s, pt_w + (size_t)p * SS_PHASE_WORDS, p, SsFmt<KIND>::VEC);
   __syncthreads();   // the only block-wide barrier: from here on the wavefronts go their own ways
 
   if (wave < SS_NWW) SsWeights<KIND>::run(s, lt, ctl, xs, y_local, wave);
@@ -1091,6 +1191,7 @@ int jsgrad_hip_stream_step(const jsgrad_hip_step_t *d) {
   s.attn_partial = (float *)(ws + SS_WS_PARTIAL);
   s.trace = d->trace;
   s.x_bytes = (int)x_bytes;
+  s.grid = grid;
 #define JSG_KIND(K)                                                                                  \
   case K:                                                                                            \
     return d->head_dim == 64 ? launch_stream<K, 64>(s, n_rep, grid, lds) : launch_stream<K, 128>(s, n_rep, grid, lds);
