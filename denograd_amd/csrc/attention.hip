@@ -28,11 +28,15 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_decode_kernel(AttnArgs a) {
   A::item(a, sm, g, split, T, chunk, n_active);
 }
 
-// splits: enough that a chunk fits the LDS score buffer, and no more than the merge can index there
-static int nsplit_for(int max_context) {
+// splits: enough that a chunk fits the LDS score buffer, and no more than the merge can index there.  One sequence wants
+// short chunks (the launch is a chain of latencies); many sequences fill the chip by themselves, and every extra split
+// only adds its fixed cost (query load, partial store, counter, merge), so the splits stop at about 8 blocks per CU.
+static int nsplit_for(int max_context, int heads_x_batch) {
   int by_lds = (max_context + ATT_CHUNK_MAX - 1) / ATT_CHUNK_MAX;
   int wanted = (max_context + 31) / 32;
   if (wanted > 64) wanted = 64;
+  const int fill = (2048 + heads_x_batch - 1) / heads_x_batch;
+  if (wanted > fill) wanted = fill;
   return by_lds > wanted ? by_lds : wanted;
 }
 
@@ -80,7 +84,7 @@ int jsgrad_hip_attn_decode_batch(const void *q, const void *cache_k, const void 
   a.q = q; a.cache_k = cache_k; a.cache_v = cache_v; a.st = st; a.out = out;
   a.counters = (int *)workspace;                                   // [batch][n_kv_heads], densely packed
   a.partial = (float *)((char *)workspace + (size_t)batch * counter_bytes);
-  a.n_kv_heads = n_kv_heads; a.nsplit = nsplit_for(max_context); a.max_context = max_context;
+  a.n_kv_heads = n_kv_heads; a.nsplit = nsplit_for(max_context, n_kv_heads * batch); a.max_context = max_context;
   a.scale = (float)(1.0 / sqrt((double)head_dim));
   a.q_bstride = (size_t)n_heads * head_dim * sizeof(_Float16);
   a.cache_bstride = (size_t)max_context * n_kv_heads * head_dim * sizeof(_Float16);
@@ -101,7 +105,7 @@ int jsgrad_hip_attn_decode(const void *q, const void *cache_k, const void *cache
   a.q = q; a.cache_k = cache_k; a.cache_v = cache_v; a.st = st; a.out = out;
   a.counters = (int *)workspace;
   a.partial = (float *)((char *)workspace + 256);
-  a.n_kv_heads = n_kv_heads; a.nsplit = nsplit_for(max_context); a.max_context = max_context;
+  a.n_kv_heads = n_kv_heads; a.nsplit = nsplit_for(max_context, 1); a.max_context = max_context;
   a.scale = (float)(1.0 / sqrt((double)head_dim));
   const int n_rep = n_heads / n_kv_heads;
   if (act == JSGRAD_F16) return head_dim == 64 ? launch_attn<_Float16, 64>(a, n_rep) : launch_attn<_Float16, 128>(a, n_rep);

@@ -275,7 +275,267 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
   }
 }
 
+// ---- at most 32 rows (batched decode): the weights are streamed once, straight from memory into the B operand ------------
+//
+// With a handful of rows the launch is bound by reading W once, so it is laid out like the one-row GEMV, not like a tiled
+// GEMM.  v_mfma_f32_16x16x32_f16 takes, per lane, 8 consecutive K elements of one weight row as B and of one x row as
+// A; a lane's 16-byte load is 8 fp16 or 16 int8 codes of weight row n0 + lane % 16, i.e. one or two MFMAs, and goes from
+// memory to registers with nothing in between (the int8 codes become RN16(code * scale) in registers: the realised
+// fp16 matrix the reference multiplies by).  The loads run through a register ring of 12 to 16 loads per wavefront.
+// Only x goes through LDS, one K chunk at a time, double buffered.  The fifth wavefront of a block does nothing but move
+// x chunks from memory to LDS (direct loads, no registers): a wavefront's loads return in order, so x loads issued by
+// the arithmetic wavefronts would have to be waited for together with every weight load issued before them, which
+// empties the ring once per chunk.
+//
+// A block owns 16 weight rows and its four arithmetic wavefronts split K: k-block kb of a chunk belongs to wavefront
+// kb % 4, and the partial accumulators are added in wavefront order through LDS.  N/16 blocks fill the chip even for
+// N = 4096.  (A block shape with 128 weight rows, which reads x once for all of them instead of once per 16, was tried for
+// the wide layers: faster for the lm_head only, and its register ring did not survive the register allocator.)
+template <int KIND> struct SkFmt {
+  static constexpr int VEC = KIND == JSGRAD_W_F16 ? 8 : 16;   // K elements per 16-byte load of a lane
+  static constexpr int KB = 4 * VEC;                          // K elements per wavefront load
+  static constexpr int KC = 16 * KB;                          // K elements per x chunk
+};
+constexpr int SK_THREADS = 320;
+constexpr int SK_KS = 4;                                    // wavefronts that split K
+template <int EPI> struct SkShape {
+  static constexpr int NMAT = EPI == GEPI_SWIGLU ? 2 : 1;
+  static constexpr int SPC = 16 / SK_KS;                    // k-blocks of a chunk one wavefront walks
+  static constexpr int RS = 8;                              // k-blocks in the ring: two chunks
+  static constexpr int BR = 16;                             // weight rows per block
+};
+
+// Block barriers of the weight-streaming kernel.  __syncthreads() also waits for every global load of the wavefront (the
+// counter that tracks loads tracks stores too, and a barrier publishes stores), which would empty the ring of weight loads
+// at every x chunk; what has to be finished at these barriers is only LDS traffic, or, for the wavefront that moves x,
+// its direct loads into LDS.
+__device__ __forceinline__ void sk_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+__device__ __forceinline__ void sk_barrier_after_loads() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+template <int KIND, int EPI, int MB>
+__global__ __launch_bounds__(SK_THREADS, 2) void skinny_gemm_kernel(GemmArgs a) {
+  static_assert(KIND == JSGRAD_W_F16 || KIND == JSGRAD_W_I8, "fp16 and int8 weights");
+  typedef SkFmt<KIND> F;
+  typedef SkShape<EPI> S;
+  constexpr int KS = SK_KS, RTW = 1;
+  constexpr int NMAT = S::NMAT, SPC = S::SPC, RS = S::RS;
+  constexpr int NMF = F::VEC / 8;                        // MFMAs per load
+  constexpr int LS = F::KC + 8;                          // halves per LDS row of x (padded: rows start in different banks)
+  constexpr int XROWS = MB * 16;
+  constexpr int PPR = F::KC / 8;                         // 16-byte pieces per x row of a chunk
+  static_assert(PPR % 64 == 0, "a direct load of the wavefront fills 1 KiB of one LDS row");
+  constexpr int XLOADS = XROWS * PPR / 64;               // direct loads per chunk
+  extern __shared__ __align__(16) _Float16 sk_lds[];     // 2 x [XROWS][LS]; afterwards the partial accumulators
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l16 = lane & 15, lq = lane >> 4;
+  const int nchunks = a.K / F::KC;
+
+  if (wave == 4) {
+    // ---- the x mover: chunk c + 1 goes to the LDS buffer the others are not reading
+    auto move = [&](int c) {
+      _Float16 *dst = sk_lds + (c & 1) * XROWS * LS;
+#pragma unroll
+      for (int i = 0; i < XLOADS; i++) {
+        const int r = (i * 64) / PPR, c8 = (i * 64) % PPR + lane;
+        const int m = r < a.M ? r : a.M - 1;             // rows past the end are computed and never stored
+        const _Float16 *src = a.x + (size_t)m * a.K + (size_t)c * F::KC + c8 * 8;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                         (__attribute__((address_space(3))) void *)(dst + r * LS + ((i * 64) % PPR) * 8), 16, 0, 0);
+      }
+    };
+    move(0);
+    sk_barrier_after_loads();
+    for (int c = 0; c < nchunks; c++) {
+      if (c + 1 < nchunks) move(c + 1);
+      sk_barrier_after_loads();
+    }
+    sk_barrier();
+    return;
+  }
+
+  const int ks = wave;
+  const int n_first = blockIdx.x * S::BR;               // first weight row of the block
+  // ---- the weight rows of this lane: row n_first + rt * 16 + lane % 16 of matrix q
+  const unsigned char *wrow[RTW][NMAT];
+  h2_t wscale[RTW][NMAT];
+#pragma unroll
+  for (int rt = 0; rt < RTW; rt++)
+#pragma unroll
+    for (int q = 0; q < NMAT; q++) {
+      const int n = n_first + rt * 16 + l16;
+      const void *w; const _Float16 *sc; int row;
+      if constexpr (EPI == GEPI_SWIGLU) { w = q ? a.w1 : a.w0; sc = q ? a.s1 : a.s0; row = n; }
+      else if constexpr (EPI == GEPI_ROPE_KV) {
+        if (n < a.n0) { w = a.w0; sc = a.s0; row = n; }
+        else if (n < a.n0 + a.n1) { w = a.w1; sc = a.s1; row = n - a.n0; }
+        else { w = a.w2; sc = a.s2; row = n - a.n0 - a.n1; }
+      } else { w = a.w0; sc = a.s0; row = n; }
+      const size_t e = (size_t)row * a.K;
+      wrow[rt][q] = (const unsigned char *)w + (KIND == JSGRAD_W_F16 ? e * 2 : e) + lq * 16;
+      if constexpr (KIND == JSGRAD_W_I8) { const _Float16 sv = sc[row]; wscale[rt][q] = h2_t{sv, sv}; }
+    }
+  // Step s of this wavefront is k-block (s % SPC) * KS + ks of chunk s / SPC.  Byte offset of the step inside a weight row;
+  // past the end: the first k-block again (a few re-reads of bytes that are in L2 keep the number of loads in flight the
+  // same on every path).
+  const int nsteps = nchunks * SPC;
+  auto woff = [&](int s) -> uint32_t {
+    const int kb = s < nsteps ? (s / SPC) * 16 + (s % SPC) * KS + ks : ks;
+    return (uint32_t)(kb * 4) * 16u;
+  };
+
+  u4_t ring[RS][RTW][NMAT];
+  f4_t acc[NMAT][RTW][MB];
+#pragma unroll
+  for (int q = 0; q < NMAT; q++)
+#pragma unroll
+    for (int rt = 0; rt < RTW; rt++)
+#pragma unroll
+      for (int mb = 0; mb < MB; mb++) acc[q][rt][mb] = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int i = 0; i < RS; i++)
+#pragma unroll
+    for (int rt = 0; rt < RTW; rt++)
+#pragma unroll
+      for (int q = 0; q < NMAT; q++) {
+        ring[i][rt][q] = ldg_stream16(wrow[rt][q] + woff(i));
+        __builtin_amdgcn_sched_barrier(0);               // issued in the order the loop consumes them: the waits count on it
+      }
+  sk_barrier();                                          // x chunk 0 is in LDS
+
+  // The ring slots are refilled on every path, also by the steps past the end (the number of loads in flight then is the
+  // same wherever the wait counters are set, so they can let RS - 1 steps stay in flight instead of none).
+  for (int s0 = 0; s0 < nsteps; s0 += RS) {
+#pragma unroll
+    for (int i = 0; i < RS; i++) {
+      const int s = s0 + i;
+      const bool on = s < nsteps;                        // same for every thread of the block
+      const int c = s / SPC, kb = (s % SPC) * KS + ks;
+      const _Float16 *xs = sk_lds + (c & 1) * XROWS * LS;
+      if (on) {
+        h8_t af[NMF][MB];
+#pragma unroll
+        for (int f = 0; f < NMF; f++)
+#pragma unroll
+          for (int mb = 0; mb < MB; mb++) af[f][mb] = *(const h8_t *)&xs[(mb * 16 + l16) * LS + kb * F::KB + lq * F::VEC + f * 8];
+#pragma unroll
+        for (int rt = 0; rt < RTW; rt++)
+#pragma unroll
+          for (int q = 0; q < NMAT; q++) {
+            const u4_t raw = ring[i][rt][q];
+            h8_t bf[NMF];
+            if constexpr (KIND == JSGRAD_W_F16) bf[0] = __builtin_bit_cast(h8_t, raw);
+            else {
+              const h2_t sc = wscale[rt][q];
+              u4_t o0, o1;
+              uint32_t lo, hi;
+              i8x4_to_h2x2(raw.x, lo, hi); o0.x = pk_mul_h2(lo, sc); o0.y = pk_mul_h2(hi, sc);
+              i8x4_to_h2x2(raw.y, lo, hi); o0.z = pk_mul_h2(lo, sc); o0.w = pk_mul_h2(hi, sc);
+              i8x4_to_h2x2(raw.z, lo, hi); o1.x = pk_mul_h2(lo, sc); o1.y = pk_mul_h2(hi, sc);
+              i8x4_to_h2x2(raw.w, lo, hi); o1.z = pk_mul_h2(lo, sc); o1.w = pk_mul_h2(hi, sc);
+              bf[0] = __builtin_bit_cast(h8_t, o0);
+              bf[NMF - 1] = __builtin_bit_cast(h8_t, o1);
+            }
+#pragma unroll
+            for (int f = 0; f < NMF; f++)
+#pragma unroll
+              for (int mb = 0; mb < MB; mb++) acc[q][rt][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[f][mb], bf[f], acc[q][rt][mb], 0, 0, 0);
+          }
+      }
+      // The slots are refilled only now that their old contents are used up (and the scheduler may not move the loads up):
+      // issued earlier, a load gets registers of its own and a copy into the slot afterwards, and the copy waits for the
+      // load on the spot.
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int rt = 0; rt < RTW; rt++)
+#pragma unroll
+        for (int q = 0; q < NMAT; q++) ring[i][rt][q] = ldg_stream16(wrow[rt][q] + woff(s + RS));
+      if (on && (s + 1) % SPC == 0) sk_barrier();        // chunk c is consumed, chunk c + 1 is in the other buffer
+    }
+  }
+
+  // ---- epilogue of one 16x16 tile.  Accumulator r of a lane is output row 4 * (lane / 16) + r, column lane % 16.
+  auto epilogue = [&](const f4_t (&tot)[NMAT], int n_tile, int mb) {
+    const int n = n_tile + l16;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int m = mb * 16 + lq * 4 + r;
+      if constexpr (EPI == GEPI_SWIGLU) {
+        const float g = rn16(tot[0][r]), u = rn16(tot[NMAT - 1][r]);
+        if (m < a.M) a.y[(size_t)m * a.N + n] = (_Float16)(silu_act<_Float16>(g) * u);
+      } else if constexpr (EPI == GEPI_STORE) {
+        if (m < a.M) {
+          float v = rn16(tot[0][r]);
+          if (a.residual) v = (float)a.residual[(size_t)m * a.N + n] + v;
+          a.y[(size_t)m * a.N + n] = (_Float16)v;
+        }
+      } else {
+        const int which = n < a.n0 ? 0 : (n < a.n0 + a.n1 ? 1 : 2);
+        const int nl = which == 0 ? n : (which == 1 ? n - a.n0 : n - a.n0 - a.n1);
+        const int pair = (nl % a.head_dim) >> 1;
+        const bool odd = nl & 1;
+        const float own = rn16(tot[0][r]);
+        const float other = dpp_f<0xB1>(own);            // the neighbouring column: the other half of the pair
+        if (m < a.M) {
+          const int b = m / a.seq_len, pos = a.start_pos + m % a.seq_len;
+          float v = own;
+          if (which < 2) {
+            const h2_t cs = *(const h2_t *)(a.rope_table + ((size_t)pos * (a.head_dim / 2) + pair) * 2);
+            const float cc = (float)cs.x, dd = (float)cs.y;
+            v = odd ? other * dd + own * cc : own * cc - other * dd;
+          }
+          if (which == 0) a.y[(size_t)m * a.n0 + nl] = (_Float16)v;
+          else {
+            _Float16 *cache = which == 1 ? a.cache_k : a.cache_v;
+            cache[((size_t)b * a.max_context + pos) * a.n1 + nl] = (_Float16)v;
+          }
+        }
+      }
+    }
+  };
+
+  // the four K parts, added in wavefront order; wavefront mb finishes row block mb
+  float *red = (float *)sk_lds;                          // [4][NMAT * MB][64 lanes] x 4 floats
+#pragma unroll
+  for (int q = 0; q < NMAT; q++)
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) *(f4_t *)&red[((wave * NMAT * MB + q * MB + mb) * 64 + lane) * 4] = acc[q][0][mb];
+  sk_barrier();
+  if (wave >= MB) return;
+  const int mb = wave;
+  f4_t tot[NMAT];
+#pragma unroll
+  for (int q = 0; q < NMAT; q++) {
+    tot[q] = *(const f4_t *)&red[((0 * NMAT * MB + q * MB + mb) * 64 + lane) * 4];
+#pragma unroll
+    for (int w = 1; w < 4; w++) tot[q] += *(const f4_t *)&red[((w * NMAT * MB + q * MB + mb) * 64 + lane) * 4];
+  }
+  epilogue(tot, n_first, mb);
+}
+
 // ---- host side ---------------------------------------------------------------------------------------------------
+
+template <int KIND, int EPI, int MB> static int launch_skinny(const GemmArgs &a, int prof_kind) {
+  typedef SkFmt<KIND> F;
+  typedef SkShape<EPI> S;
+  constexpr size_t x_bytes = (size_t)2 * MB * 16 * (F::KC + 8) * sizeof(_Float16);
+  constexpr size_t red_bytes = (size_t)4 * S::NMAT * MB * 64 * 4 * sizeof(float);
+  constexpr size_t lds = x_bytes > red_bytes ? x_bytes : red_bytes;
+  if constexpr (lds > 64 * 1024) {
+    static bool raised = false;   // one process, one device, one thread: set once per instantiation
+    if (!raised) {
+      JSG_HIP(hipFuncSetAttribute((const void *)skinny_gemm_kernel<KIND, EPI, MB>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      raised = true;
+    }
+  }
+  JSG_LAUNCH(prof_kind, (skinny_gemm_kernel<KIND, EPI, MB>), dim3(a.N / S::BR), dim3(SK_THREADS), lds, a);
+  return 0;
+}
+// Few rows: the weight-streaming kernel when K is whole chunks.
+template <int KIND, int EPI> static int dispatch_skinny(const GemmArgs &a, int prof_kind, bool *taken) {
+  *taken = a.M <= 32 && a.K % SkFmt<KIND>::KC == 0 && a.K / SkFmt<KIND>::KC >= 2 && a.N % 16 == 0 && !getenv("JSG_GEMM_NO_SKINNY");
+  if (!*taken) return 0;
+  return a.M <= 16 ? launch_skinny<KIND, EPI, 1>(a, prof_kind) : launch_skinny<KIND, EPI, 2>(a, prof_kind);
+}
 
 template <int KIND, int EPI, int WGM, int WGN, int TM, int TN> static int launch_gemm(const GemmArgs &a, int prof_kind) {
   constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
@@ -299,6 +559,9 @@ template <int EPI> static int dispatch_gemm(int kind, const GemmArgs &a, int pro
   const bool tall = a.M > 64;
   const int n_out = EPI == GEPI_SWIGLU ? 2 * a.N : a.N;
   const bool wide = tall && getenv("JSG_GEMM_WIDE") && n_out % 256 == 0 && EPI != GEPI_ROPE_KV;
+  bool taken = false;
+  if (kind == JSGRAD_W_F16) { const int rc = dispatch_skinny<JSGRAD_W_F16, EPI>(a, prof_kind, &taken); if (taken) return rc; }
+  if (kind == JSGRAD_W_I8) { const int rc = dispatch_skinny<JSGRAD_W_I8, EPI>(a, prof_kind, &taken); if (taken) return rc; }
 #define JSG_CASE(K)                                                                                                    \
   case K:                                                                                                              \
     if (wide) return launch_gemm<K, EPI, 2, 2, 4, 4>(a, prof_kind);                                                   \

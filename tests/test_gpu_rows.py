@@ -37,7 +37,9 @@ def sp(t):
 
 
 @pytest.mark.parametrize("kind", ["float16", "int8", "nf4"])
-@pytest.mark.parametrize("rows,out_f,in_f", [(2, 128, 64), (16, 256, 512), (33, 384, 256), (64, 128, 1024), (65, 256, 128), (300, 384, 192), (512, 512, 512)])
+@pytest.mark.parametrize("rows,out_f,in_f", [(2, 128, 64), (16, 256, 512), (33, 384, 256), (64, 128, 1024), (65, 256, 128), (300, 384, 192), (512, 512, 512),
+                                             # at most 32 rows and K in whole chunks: the weight-streaming kernel (2, 3, 4 and 5 chunks; 16- and 32-row blocks)
+                                             (2, 128, 2048), (5, 256, 2048), (16, 256, 3072), (17, 128, 4096), (32, 384, 5120), (16, 128, 1536), (31, 128, 1024)])
 def test_gemm_matches_several_row_linear(hip, kind, rows, out_f, in_f):
     w, s = make_weight(kind, out_f, in_f)
     x = RNG.standard_normal((rows, in_f)).astype(np.float16)
@@ -95,10 +97,28 @@ def test_gemm_rejects_bad_shapes(hip):
         check(hip.jsgrad_hip_gemm(ffi.W_I8, t.ptr, None, 128, 64, t.ptr, 4, t.ptr, None))
 
 
+def test_few_rows_streaming_kernel_equals_tiled_kernel(hip, monkeypatch):
+    """The two several-row kernels compute the same products; their float sums differ in order only."""
+    out_f, in_f = 256, 4096
+    for kind in ("float16", "int8"):
+        for rows in (16, 29):
+            w, s = make_weight(kind, out_f, in_f)
+            x = RNG.standard_normal((rows, in_f)).astype(np.float16)
+            tw, ts = dev(w, s)
+            tx, ya, yb = Tensor(x), Tensor.empty((rows, out_f), "float16"), Tensor.empty((rows, out_f), "float16")
+            check(hip.jsgrad_hip_gemm(KINDS[kind], tw.ptr, sp(ts), out_f, in_f, tx.ptr, rows, ya.ptr, None))
+            monkeypatch.setenv("JSG_GEMM_NO_SKINNY", "1")
+            check(hip.jsgrad_hip_gemm(KINDS[kind], tw.ptr, sp(ts), out_f, in_f, tx.ptr, rows, yb.ptr, None))
+            monkeypatch.delenv("JSG_GEMM_NO_SKINNY")
+            a, b = ya.numpy().astype(np.float32), yb.numpy().astype(np.float32)
+            assert_close(a, orc.linear(w, s, x, out_f, in_f, True), True, f"streaming {kind} {rows} rows")
+            assert_close(a, b, True, f"streaming vs tiled {kind} {rows} rows")
+            assert (a == b).mean() > 0.97
+
+
 @pytest.mark.parametrize("kind", ["float16", "int8", "nf4"])
-@pytest.mark.parametrize("rows", [3, 16, 130])
-def test_gemm_ffn_gate(hip, kind, rows):
-    dim, hidden = 256, 384
+@pytest.mark.parametrize("rows,dim,hidden", [(3, 256, 384), (16, 256, 384), (130, 256, 384), (16, 2048, 256), (20, 3072, 128)])
+def test_gemm_ffn_gate(hip, kind, rows, dim, hidden):
     w1, s1 = make_weight(kind, hidden, dim)
     w3, s3 = make_weight(kind, hidden, dim)
     x = RNG.standard_normal((rows, dim)).astype(np.float16)
@@ -112,10 +132,11 @@ def test_gemm_ffn_gate(hip, kind, rows):
     assert_close(tg.numpy().astype(np.float32), ref, True, f"ffn_gate {kind} {rows}", composed=True)
 
 
+@pytest.mark.parametrize("B,S,dim", [(2, 37, 256), (16, 1, 2048), (3, 9, 2048)])   # prefill rows; batched decode and few rows on the streaming kernel
 @pytest.mark.parametrize("kind,hd", [("float16", 64), ("int8", 128), ("nf4", 64)])
-def test_gemm_qkv_rope_writes_queries_and_cache(hip, kind, hd):
-    B, S, start, ctx = 2, 37, 5, 64
-    H, KV, dim = (4, 2, 256) if hd == 64 else (2, 1, 256)
+def test_gemm_qkv_rope_writes_queries_and_cache(hip, kind, hd, B, S, dim):
+    start, ctx = 5, 64
+    H, KV = (4, 2) if hd == 64 else (2, 1)
     wq, sq = make_weight(kind, H * hd, dim)
     wk, sk = make_weight(kind, KV * hd, dim)
     wv, sv = make_weight(kind, KV * hd, dim)
