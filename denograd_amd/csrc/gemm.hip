@@ -282,27 +282,30 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
 // A; a lane's 16-byte load is 8 fp16 or 16 int8 codes of weight row n0 + lane % 16, i.e. one or two MFMAs, and goes from
 // memory to registers with nothing in between (the int8 codes become RN16(code * scale) in registers: the realised
 // fp16 matrix the reference multiplies by).  The loads run through a register ring of 12 to 16 loads per wavefront.
-// Only x goes through LDS, one K chunk at a time, double buffered.  The fifth wavefront of a block does nothing but move
-// x chunks from memory to LDS (direct loads, no registers): a wavefront's loads return in order, so x loads issued by
+// Only x goes through LDS, in K chunks of 512, four buffers.  The fifth wavefront of a block does nothing but move
+// x chunks from memory to LDS (direct loads, no registers), up to three chunks ahead: a wavefront's loads return in order, so x loads issued by
 // the arithmetic wavefronts would have to be waited for together with every weight load issued before them, which
 // empties the ring once per chunk.
 //
-// A block owns 16 weight rows and its four arithmetic wavefronts split K: k-block kb of a chunk belongs to wavefront
-// kb % 4, and the partial accumulators are added in wavefront order through LDS.  N/16 blocks fill the chip even for
+// A block owns 16 weight rows and its four arithmetic wavefronts split K: each takes a quarter of the k-blocks of every
+// chunk, and the partial accumulators are added in wavefront order through LDS.  N/16 blocks fill the chip even for
 // N = 4096.  (A block shape with 128 weight rows, which reads x once for all of them instead of once per 16, was tried for
 // the wide layers: faster for the lm_head only, and its register ring did not survive the register allocator.)
 template <int KIND> struct SkFmt {
   static constexpr int VEC = KIND == JSGRAD_W_F16 ? 8 : 16;   // K elements per 16-byte load of a lane
-  static constexpr int KB = 4 * VEC;                          // K elements per wavefront load
-  static constexpr int KC = 16 * KB;                          // K elements per x chunk
+  static constexpr int KB = 4 * VEC;                          // K elements per wavefront load (a k-block)
+  static constexpr int KC = 512;                              // K elements per x chunk: 1 KiB per x row, one direct load
+  static constexpr int KBC = KC / KB;                         // k-blocks per chunk
 };
 constexpr int SK_THREADS = 320;
-constexpr int SK_KS = 4;                                    // wavefronts that split K
-template <int EPI> struct SkShape {
+constexpr int SK_KS = 4;                                      // wavefronts that split K
+constexpr int SK_XBUF = 4;                                    // x chunks in LDS: one being read, up to three on their way
+template <int KIND, int EPI> struct SkShape {
   static constexpr int NMAT = EPI == GEPI_SWIGLU ? 2 : 1;
-  static constexpr int SPC = 16 / SK_KS;                    // k-blocks of a chunk one wavefront walks
-  static constexpr int RS = 8;                              // k-blocks in the ring: two chunks
-  static constexpr int BR = 16;                             // weight rows per block
+  static constexpr int SPC = SkFmt<KIND>::KBC / SK_KS;        // k-blocks of a chunk one wavefront walks
+  static constexpr int RS = 8;                                // k-blocks in the ring
+  static constexpr int BR = 16;                               // weight rows per block
+  static_assert(RS % SPC == 0, "chunk ends fall on fixed ring slots");
 };
 
 // Block barriers of the weight-streaming kernel.  __syncthreads() also waits for every global load of the wavefront (the
@@ -310,13 +313,12 @@ template <int EPI> struct SkShape {
 // at every x chunk; what has to be finished at these barriers is only LDS traffic, or, for the wavefront that moves x,
 // its direct loads into LDS.
 __device__ __forceinline__ void sk_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-__device__ __forceinline__ void sk_barrier_after_loads() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 template <int KIND, int EPI, int MB>
 __global__ __launch_bounds__(SK_THREADS, 2) void skinny_gemm_kernel(GemmArgs a) {
   static_assert(KIND == JSGRAD_W_F16 || KIND == JSGRAD_W_I8, "fp16 and int8 weights");
   typedef SkFmt<KIND> F;
-  typedef SkShape<EPI> S;
+  typedef SkShape<KIND, EPI> S;
   constexpr int KS = SK_KS, RTW = 1;
   constexpr int NMAT = S::NMAT, SPC = S::SPC, RS = S::RS;
   constexpr int NMF = F::VEC / 8;                        // MFMAs per load
@@ -325,15 +327,16 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_gemm_kernel(GemmArgs a) 
   constexpr int PPR = F::KC / 8;                         // 16-byte pieces per x row of a chunk
   static_assert(PPR % 64 == 0, "a direct load of the wavefront fills 1 KiB of one LDS row");
   constexpr int XLOADS = XROWS * PPR / 64;               // direct loads per chunk
-  extern __shared__ __align__(16) _Float16 sk_lds[];     // 2 x [XROWS][LS]; afterwards the partial accumulators
+  extern __shared__ __align__(16) _Float16 sk_lds[];     // SK_XBUF x [XROWS][LS]; afterwards the partial accumulators
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l16 = lane & 15, lq = lane >> 4;
   const int nchunks = a.K / F::KC;
 
   if (wave == 4) {
-    // ---- the x mover: chunk c + 1 goes to the LDS buffer the others are not reading
+    // ---- the x mover: up to three chunks ahead of the one being read (a chunk takes a trip to L2 to arrive, longer than
+    // the others need for a chunk), into the buffer whose readers passed the barrier of the chunk before
     auto move = [&](int c) {
-      _Float16 *dst = sk_lds + (c & 1) * XROWS * LS;
+      _Float16 *dst = sk_lds + (c % SK_XBUF) * XROWS * LS;
 #pragma unroll
       for (int i = 0; i < XLOADS; i++) {
         const int r = (i * 64) / PPR, c8 = (i * 64) % PPR + lane;
@@ -343,11 +346,23 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_gemm_kernel(GemmArgs a) 
                                          (__attribute__((address_space(3))) void *)(dst + r * LS + ((i * 64) % PPR) * 8), 16, 0, 0);
       }
     };
-    move(0);
-    sk_barrier_after_loads();
+    // wait until chunk `target` has landed: the direct loads complete in order, so whatever was issued after it may stay
+    // in flight (the counter holds 63 loads at most)
+    constexpr int MAX_BEHIND = 63 / XLOADS < 2 ? 63 / XLOADS : 2;
+    int issued = 0;
+    auto landed = [&](int target) {
+      const int behind = issued - target - 1;
+      if (MAX_BEHIND >= 2 && behind >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * XLOADS <= 63 ? 2 * XLOADS : 0) : "memory");
+      else if (MAX_BEHIND >= 1 && behind >= 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(XLOADS <= 63 ? XLOADS : 0) : "memory");
+      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    };
+    while (issued < SK_XBUF - 1 && issued < nchunks) move(issued++);
+    landed(0);
+    sk_barrier();
     for (int c = 0; c < nchunks; c++) {
-      if (c + 1 < nchunks) move(c + 1);
-      sk_barrier_after_loads();
+      if (issued < nchunks) move(issued++);              // into the buffer of chunk c - 1
+      if (c + 1 < nchunks) landed(c + 1);
+      sk_barrier();
     }
     sk_barrier();
     return;
@@ -374,12 +389,13 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_gemm_kernel(GemmArgs a) 
       wrow[rt][q] = (const unsigned char *)w + (KIND == JSGRAD_W_F16 ? e * 2 : e) + lq * 16;
       if constexpr (KIND == JSGRAD_W_I8) { const _Float16 sv = sc[row]; wscale[rt][q] = h2_t{sv, sv}; }
     }
-  // Step s of this wavefront is k-block (s % SPC) * KS + ks of chunk s / SPC.  Byte offset of the step inside a weight row;
+  // Step s of this wavefront is k-block ks * SPC + s % SPC of chunk s / SPC: its SPC k-blocks of a chunk are neighbours, so
+  // that the halves of a 128-byte line of a weight row are asked for by one wavefront, back to back.  Byte offset of the step inside a weight row;
   // past the end: the first k-block again (a few re-reads of bytes that are in L2 keep the number of loads in flight the
   // same on every path).
   const int nsteps = nchunks * SPC;
   auto woff = [&](int s) -> uint32_t {
-    const int kb = s < nsteps ? (s / SPC) * 16 + (s % SPC) * KS + ks : ks;
+    const int kb = s < nsteps ? (s / SPC) * F::KBC + ks * SPC + s % SPC : ks * SPC;
     return (uint32_t)(kb * 4) * 16u;
   };
 
@@ -409,8 +425,8 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_gemm_kernel(GemmArgs a) 
     for (int i = 0; i < RS; i++) {
       const int s = s0 + i;
       const bool on = s < nsteps;                        // same for every thread of the block
-      const int c = s / SPC, kb = (s % SPC) * KS + ks;
-      const _Float16 *xs = sk_lds + (c & 1) * XROWS * LS;
+      const int c = s / SPC, kb = ks * SPC + s % SPC;
+      const _Float16 *xs = sk_lds + (c % SK_XBUF) * XROWS * LS;
       if (on) {
         h8_t af[NMF][MB];
 #pragma unroll
@@ -516,8 +532,8 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_gemm_kernel(GemmArgs a) 
 
 template <int KIND, int EPI, int MB> static int launch_skinny(const GemmArgs &a, int prof_kind) {
   typedef SkFmt<KIND> F;
-  typedef SkShape<EPI> S;
-  constexpr size_t x_bytes = (size_t)2 * MB * 16 * (F::KC + 8) * sizeof(_Float16);
+  typedef SkShape<KIND, EPI> S;
+  constexpr size_t x_bytes = (size_t)SK_XBUF * MB * 16 * (F::KC + 8) * sizeof(_Float16);
   constexpr size_t red_bytes = (size_t)4 * S::NMAT * MB * 64 * 4 * sizeof(float);
   constexpr size_t lds = x_bytes > red_bytes ? x_bytes : red_bytes;
   if constexpr (lds > 64 * 1024) {
