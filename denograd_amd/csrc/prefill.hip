@@ -209,21 +209,54 @@ __global__ void embed_rows_kernel(int kind, const void *table, const _Float16 *s
   }
 }
 
-// RMSNorm.call (nn/index.ts:586-588), one block per row
+// RMSNorm.call (nn/index.ts:586-588), one block per row.  A thread keeps its 16-byte chunks of the row (and of the weight)
+// in registers between the sum of squares and the scaling: one round of loads.  MAXCH chunks per thread (d <= 2048 * MAXCH);
+// longer rows take the two-pass loop.
+template <int MAXCH>
 __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const _Float16 *x, const _Float16 *w, _Float16 *y, int d, float eps, float inv_d) {
   __shared__ float red[4];
   const _Float16 *xr = x + (size_t)blockIdx.x * d;
   _Float16 *yr = y + (size_t)blockIdx.x * d;
   float ss = 0.0f;
-  for (int i = threadIdx.x; i < d; i += 256) { const float f = (float)xr[i]; ss = fmaf(f, f, ss); }
-  ss = wave_sum(ss);
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
-  __syncthreads();
-  const float tot = (red[0] + red[1]) + (red[2] + red[3]);
-  const float r = __fsqrt_rn(__fdiv_rn(1.0f, __fadd_rn(__fmul_rn(tot, inv_d), eps)));
-  for (int i = threadIdx.x; i < d; i += 256) {
-    const float v = rn16(__fmul_rn((float)xr[i], r));
-    yr[i] = (_Float16)__fmul_rn(v, (float)w[i]);
+  if constexpr (MAXCH > 0) {
+    const int nch = d / 8;
+    h8_t xv[MAXCH], wv[MAXCH];
+#pragma unroll
+    for (int c = 0; c < MAXCH; c++) {
+      const int i = threadIdx.x + c * 256;
+      if (i < nch) { xv[c] = *(const h8_t *)(xr + i * 8); wv[c] = *(const h8_t *)(w + i * 8); }
+    }
+#pragma unroll
+    for (int c = 0; c < MAXCH; c++)
+      if (threadIdx.x + c * 256 < nch)
+#pragma unroll
+        for (int e = 0; e < 8; e++) { const float f = (float)xv[c][e]; ss = fmaf(f, f, ss); }
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float tot = (red[0] + red[1]) + (red[2] + red[3]);
+    const float r = __fsqrt_rn(__fdiv_rn(1.0f, __fadd_rn(__fmul_rn(tot, inv_d), eps)));
+#pragma unroll
+    for (int c = 0; c < MAXCH; c++) {
+      const int i = threadIdx.x + c * 256;
+      if (i < nch) {
+        h8_t o;
+#pragma unroll
+        for (int e = 0; e < 8; e++) o[e] = (_Float16)__fmul_rn(rn16(__fmul_rn((float)xv[c][e], r)), (float)wv[c][e]);
+        *(h8_t *)(yr + i * 8) = o;
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < d; i += 256) { const float f = (float)xr[i]; ss = fmaf(f, f, ss); }
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float tot = (red[0] + red[1]) + (red[2] + red[3]);
+    const float r = __fsqrt_rn(__fdiv_rn(1.0f, __fadd_rn(__fmul_rn(tot, inv_d), eps)));
+    for (int i = threadIdx.x; i < d; i += 256) {
+      const float v = rn16(__fmul_rn((float)xr[i], r));
+      yr[i] = (_Float16)__fmul_rn(v, (float)w[i]);
+    }
   }
 }
 
@@ -282,7 +315,10 @@ int jsgrad_hip_embed_rows(int kind, const void *table, const void *scale, const 
 int jsgrad_hip_rmsnorm_rows(const void *x, const void *w, void *y, int rows, int d, float eps) {
   JSG_READY();
   JSG_REQUIRE(x && w && y && rows > 0 && d > 0, "jsgrad_hip_rmsnorm_rows: bad argument");
-  JSG_LAUNCH(PROF_RMSNORM, rmsnorm_rows_kernel, dim3(rows), dim3(256), 0, (const _Float16 *)x, (const _Float16 *)w, (_Float16 *)y, d, eps, (float)(1.0 / (double)d));
+  const float inv_d = (float)(1.0 / (double)d);
+  if (d % 8 == 0 && d <= 2048) JSG_LAUNCH(PROF_RMSNORM, rmsnorm_rows_kernel<1>, dim3(rows), dim3(256), 0, (const _Float16 *)x, (const _Float16 *)w, (_Float16 *)y, d, eps, inv_d);
+  else if (d % 8 == 0 && d <= 8192) JSG_LAUNCH(PROF_RMSNORM, rmsnorm_rows_kernel<4>, dim3(rows), dim3(256), 0, (const _Float16 *)x, (const _Float16 *)w, (_Float16 *)y, d, eps, inv_d);
+  else JSG_LAUNCH(PROF_RMSNORM, rmsnorm_rows_kernel<0>, dim3(rows), dim3(256), 0, (const _Float16 *)x, (const _Float16 *)w, (_Float16 *)y, d, eps, inv_d);
   return 0;
 }
 
