@@ -297,7 +297,7 @@ def run_batched(name, bsz, prompt_len, steps):
             "prefill": prefill, "decode": decode}
 
 
-def traffic_probe(name):
+def traffic_probe(name, batch=1):
     from denograd_amd import ffi, synthetic
     from denograd_amd.ffi import check
     from denograd_amd.llama3 import Llama3
@@ -315,6 +315,12 @@ def traffic_probe(name):
         llm._call(t)
         llm.start_pos += 1
     check(lib.jsgrad_hip_sync())
+    if batch > 1:      # two batched decode steps (the few-row kernels) after an 8-token batched prefill
+        prompts = np.stack([synthetic.random_prompt(cfg, 8, seed=100 + b) for b in range(batch)]).astype(np.int32)
+        tok = llm.model.forward_rows(prompts, 0)
+        tok = llm.model.forward_rows(tok, 8)
+        tok = llm.model.forward_rows(tok, 9)
+        check(lib.jsgrad_hip_sync())
 
 
 def main():
@@ -333,6 +339,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle baseline")
     ap.add_argument("--traffic-probe", action="store_true", help="for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: one 512 MiB device-to-device copy "
                     "(a plain copy kernel of known size, to scale the counters) followed by 4 eager decode steps of --workload; prints nothing")
+    ap.add_argument("--traffic-batch", type=int, default=1, help="with --traffic-probe: also two batched decode steps of this many sequences")
     ap.add_argument("--fused-step", action="store_true", help="run each token as one persistent kernel (jsgrad_hip_decode_step) instead of one launch per fused op")
     ap.add_argument("--stream-step", action="store_true", help="run each token as one persistent kernel with streaming wavefronts (jsgrad_hip_stream_step)")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel eagerly instead of replaying a captured HIP graph "
@@ -348,7 +355,7 @@ def main():
     log(f"device: {dev.name}, {dev.cu_count} CUs")
 
     if args.traffic_probe:
-        traffic_probe(args.workload)
+        traffic_probe(args.workload, args.traffic_batch)
         return
     step_mode = "stream" if args.stream_step else args.fused_step
     llm, cfg, res = run_workload(args.workload, args.prompt, args.steps, args.warmup, use_graph=not args.no_graph, fused_step=step_mode)

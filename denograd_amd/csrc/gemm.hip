@@ -300,11 +300,11 @@ template <int KIND> struct SkFmt {
 constexpr int SK_THREADS = 320;
 constexpr int SK_KS = 4;                                      // wavefronts that split K
 constexpr int SK_XBUF = 4;                                    // x chunks in LDS: one being read, up to three on their way
-template <int KIND, int EPI> struct SkShape {
+template <int KIND, int EPI, int RTW> struct SkShape {
   static constexpr int NMAT = EPI == GEPI_SWIGLU ? 2 : 1;
   static constexpr int SPC = SkFmt<KIND>::KBC / SK_KS;        // k-blocks of a chunk one wavefront walks
   static constexpr int RS = 8;                                // k-blocks in the ring
-  static constexpr int BR = 16;                               // weight rows per block
+  static constexpr int BR = 16 * RTW;                         // weight rows per block: RTW tiles of 16
   static_assert(RS % SPC == 0, "chunk ends fall on fixed ring slots");
 };
 
@@ -314,12 +314,11 @@ template <int KIND, int EPI> struct SkShape {
 // its direct loads into LDS.
 __device__ __forceinline__ void sk_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-template <int KIND, int EPI, int MB>
+template <int KIND, int EPI, int MB, int RTW>
 __global__ __launch_bounds__(SK_THREADS, 2) void skinny_gemm_kernel(GemmArgs a) {
   static_assert(KIND == JSGRAD_W_F16 || KIND == JSGRAD_W_I8, "fp16 and int8 weights");
   typedef SkFmt<KIND> F;
-  typedef SkShape<KIND, EPI> S;
-  constexpr int KS = SK_KS, RTW = 1;
+  typedef SkShape<KIND, EPI, RTW> S;
   constexpr int NMAT = S::NMAT, SPC = S::SPC, RS = S::RS;
   constexpr int NMF = F::VEC / 8;                        // MFMAs per load
   constexpr int LS = F::KC + 8;                          // halves per LDS row of x (padded: rows start in different banks)
@@ -509,48 +508,56 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_gemm_kernel(GemmArgs a) 
     }
   };
 
-  // the four K parts, added in wavefront order; wavefront mb finishes row block mb
-  float *red = (float *)sk_lds;                          // [4][NMAT * MB][64 lanes] x 4 floats
+  // the four K parts, added in wavefront order; the (tile, row block) pairs are dealt to the wavefronts
+  constexpr int NACC = NMAT * RTW * MB;
+  float *red = (float *)sk_lds;                          // [4][NACC][64 lanes] x 4 floats
 #pragma unroll
   for (int q = 0; q < NMAT; q++)
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++) *(f4_t *)&red[((wave * NMAT * MB + q * MB + mb) * 64 + lane) * 4] = acc[q][0][mb];
+    for (int rt = 0; rt < RTW; rt++)
+#pragma unroll
+      for (int mb = 0; mb < MB; mb++) *(f4_t *)&red[((wave * NACC + (q * RTW + rt) * MB + mb) * 64 + lane) * 4] = acc[q][rt][mb];
   sk_barrier();
-  if (wave >= MB) return;
-  const int mb = wave;
-  f4_t tot[NMAT];
+  for (int item = wave; item < RTW * MB; item += 4) {
+    const int rt = item / MB, mb = item % MB;
+    f4_t tot[NMAT];
 #pragma unroll
-  for (int q = 0; q < NMAT; q++) {
-    tot[q] = *(const f4_t *)&red[((0 * NMAT * MB + q * MB + mb) * 64 + lane) * 4];
+    for (int q = 0; q < NMAT; q++) {
+      tot[q] = *(const f4_t *)&red[((0 * NACC + (q * RTW + rt) * MB + mb) * 64 + lane) * 4];
 #pragma unroll
-    for (int w = 1; w < 4; w++) tot[q] += *(const f4_t *)&red[((w * NMAT * MB + q * MB + mb) * 64 + lane) * 4];
+      for (int w = 1; w < 4; w++) tot[q] += *(const f4_t *)&red[((w * NACC + (q * RTW + rt) * MB + mb) * 64 + lane) * 4];
+    }
+    epilogue(tot, n_first + rt * 16, mb);
   }
-  epilogue(tot, n_first, mb);
 }
 
 // ---- host side ---------------------------------------------------------------------------------------------------
 
-template <int KIND, int EPI, int MB> static int launch_skinny(const GemmArgs &a, int prof_kind) {
+template <int KIND, int EPI, int MB, int RTW> static int launch_skinny(const GemmArgs &a, int prof_kind) {
   typedef SkFmt<KIND> F;
-  typedef SkShape<KIND, EPI> S;
+  typedef SkShape<KIND, EPI, RTW> S;
   constexpr size_t x_bytes = (size_t)SK_XBUF * MB * 16 * (F::KC + 8) * sizeof(_Float16);
-  constexpr size_t red_bytes = (size_t)4 * S::NMAT * MB * 64 * 4 * sizeof(float);
+  constexpr size_t red_bytes = (size_t)4 * S::NMAT * RTW * MB * 64 * 4 * sizeof(float);
   constexpr size_t lds = x_bytes > red_bytes ? x_bytes : red_bytes;
   if constexpr (lds > 64 * 1024) {
     static bool raised = false;   // one process, one device, one thread: set once per instantiation
     if (!raised) {
-      JSG_HIP(hipFuncSetAttribute((const void *)skinny_gemm_kernel<KIND, EPI, MB>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      JSG_HIP(hipFuncSetAttribute((const void *)skinny_gemm_kernel<KIND, EPI, MB, RTW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
       raised = true;
     }
   }
-  JSG_LAUNCH(prof_kind, (skinny_gemm_kernel<KIND, EPI, MB>), dim3(a.N / S::BR), dim3(SK_THREADS), lds, a);
+  JSG_LAUNCH(prof_kind, (skinny_gemm_kernel<KIND, EPI, MB, RTW>), dim3(a.N / S::BR), dim3(SK_THREADS), lds, a);
   return 0;
 }
-// Few rows: the weight-streaming kernel when K is whole chunks.
+// Few rows: the weight-streaming kernel when K is whole chunks.  Every block reads all of x; with two tiles of 16 weight
+// rows per block that is half as often, taken when the output is wide enough for two tiles per block to still fill the chip.
 template <int KIND, int EPI> static int dispatch_skinny(const GemmArgs &a, int prof_kind, bool *taken) {
   *taken = a.M <= 32 && a.K % SkFmt<KIND>::KC == 0 && a.K / SkFmt<KIND>::KC >= 2 && a.N % 16 == 0 && !getenv("JSG_GEMM_NO_SKINNY");
   if (!*taken) return 0;
-  return a.M <= 16 ? launch_skinny<KIND, EPI, 1>(a, prof_kind) : launch_skinny<KIND, EPI, 2>(a, prof_kind);
+  const char *pin = getenv("JSG_GEMM_SKINNY_TILES");     // "1" or "2": tests run small matrices through both
+  const bool two = a.N % 32 == 0 && (pin ? pin[0] == '2' : a.N / 32 >= 768);
+  if (a.M <= 16) return two ? launch_skinny<KIND, EPI, 1, 2>(a, prof_kind) : launch_skinny<KIND, EPI, 1, 1>(a, prof_kind);
+  return two ? launch_skinny<KIND, EPI, 2, 2>(a, prof_kind) : launch_skinny<KIND, EPI, 2, 1>(a, prof_kind);
 }
 
 template <int KIND, int EPI, int WGM, int WGN, int TM, int TN> static int launch_gemm(const GemmArgs &a, int prof_kind) {

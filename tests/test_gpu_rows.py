@@ -98,22 +98,38 @@ def test_gemm_rejects_bad_shapes(hip):
 
 
 def test_few_rows_streaming_kernel_equals_tiled_kernel(hip, monkeypatch):
-    """The two several-row kernels compute the same products; their float sums differ in order only."""
+    """The several-row kernels compute the same products; their float sums differ in order only.  The weight-streaming
+    kernel with one and with two tiles of 16 weight rows per block against the tiled kernel."""
     out_f, in_f = 256, 4096
     for kind in ("float16", "int8"):
         for rows in (16, 29):
             w, s = make_weight(kind, out_f, in_f)
             x = RNG.standard_normal((rows, in_f)).astype(np.float16)
             tw, ts = dev(w, s)
-            tx, ya, yb = Tensor(x), Tensor.empty((rows, out_f), "float16"), Tensor.empty((rows, out_f), "float16")
-            check(hip.jsgrad_hip_gemm(KINDS[kind], tw.ptr, sp(ts), out_f, in_f, tx.ptr, rows, ya.ptr, None))
-            monkeypatch.setenv("JSG_GEMM_NO_SKINNY", "1")
-            check(hip.jsgrad_hip_gemm(KINDS[kind], tw.ptr, sp(ts), out_f, in_f, tx.ptr, rows, yb.ptr, None))
-            monkeypatch.delenv("JSG_GEMM_NO_SKINNY")
-            a, b = ya.numpy().astype(np.float32), yb.numpy().astype(np.float32)
-            assert_close(a, orc.linear(w, s, x, out_f, in_f, True), True, f"streaming {kind} {rows} rows")
-            assert_close(a, b, True, f"streaming vs tiled {kind} {rows} rows")
-            assert (a == b).mean() > 0.97
+            tx = Tensor(x)
+            got = {}
+            for shape in ("1", "2", "tiled"):
+                monkeypatch.setenv("JSG_GEMM_NO_SKINNY", "1") if shape == "tiled" else monkeypatch.setenv("JSG_GEMM_SKINNY_TILES", shape)
+                y = Tensor.empty((rows, out_f), "float16")
+                check(hip.jsgrad_hip_gemm(KINDS[kind], tw.ptr, sp(ts), out_f, in_f, tx.ptr, rows, y.ptr, None))
+                got[shape] = y.numpy().astype(np.float32)
+                monkeypatch.delenv("JSG_GEMM_NO_SKINNY", raising=False)
+                monkeypatch.delenv("JSG_GEMM_SKINNY_TILES", raising=False)
+            ref = orc.linear(w, s, x, out_f, in_f, True)
+            for shape, y in got.items():
+                assert_close(y, ref, True, f"{shape} {kind} {rows} rows")
+            assert np.array_equal(got["1"], got["2"])     # same order of summation
+            assert (got["1"] == got["tiled"]).mean() > 0.97
+
+
+@pytest.mark.parametrize("tiles", ["1", "2"])
+def test_few_rows_fused_epilogues_with_one_and_two_tiles_per_block(hip, monkeypatch, tiles):
+    """SwiGLU and rotary / cache epilogues of the weight-streaming kernel, tiles per block pinned."""
+    monkeypatch.setenv("JSG_GEMM_SKINNY_TILES", tiles)
+    test_gemm_ffn_gate(hip, "int8", 16, 2048, 256)
+    test_gemm_ffn_gate(hip, "float16", 20, 1024, 128)
+    test_gemm_qkv_rope_writes_queries_and_cache(hip, "int8", 128, 16, 1, 2048)
+    test_gemm_qkv_rope_writes_queries_and_cache(hip, "float16", 64, 3, 9, 2048)
 
 
 @pytest.mark.parametrize("kind", ["float16", "int8", "nf4"])
