@@ -75,9 +75,20 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       }
     }
 
+    // The K and V rows of this thread's first NPRE iterations are requested together, before anything is computed: a chunk is
+    // usually that short, and the launch is a chain of round trips, so V must not wait for the softmax.
+    constexpr int NPRE = 2;
+    u4_t kpre[NPRE], vpre[NPRE];
+#pragma unroll
+    for (int i = 0; i < NPRE; i++) {
+      const int t = t0 + (wave + i * NW) * RPI + grp;
+      const size_t off = (size_t)(t < t1 ? t : t1 - 1) * row_stride;   // t1 > t0: the item exists
+      kpre[i] = *(const u4_t *)(kbase + off);
+      vpre[i] = *(const u4_t *)(vbase + off);
+    }
+
     // ---- phase 1: scores of the chunk
-    for (int t = t0 + wave * RPI + grp; t < t1; t += NW * RPI) {
-      u4_t raw = *(const u4_t *)(kbase + (size_t)t * row_stride);
+    auto score_row = [&](u4_t raw, int t) {
       float kf[EPL];
       if constexpr (sizeof(AT) == 2) {
 #pragma unroll
@@ -94,7 +105,13 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
         p = group_sum<G>(p);
         if (sub == 0) sm.sc[j][t - t0] = p * a.scale;
       }
+    };
+#pragma unroll
+    for (int i = 0; i < NPRE; i++) {
+      const int t = t0 + (wave + i * NW) * RPI + grp;
+      if (t < t1) score_row(kpre[i], t);
     }
+    for (int t = t0 + (wave + NPRE * NW) * RPI + grp; t < t1; t += NW * RPI) score_row(*(const u4_t *)(kbase + (size_t)t * row_stride), t);
     __syncthreads();
     // chunk maximum per head
     {
@@ -150,8 +167,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
     for (int j = 0; j < NREP; j++)
 #pragma unroll
       for (int e = 0; e < EPL; e++) of[j][e] = 0.0f;
-    for (int t = t0 + wave * RPI + grp; t < t1; t += NW * RPI) {
-      u4_t raw = *(const u4_t *)(vbase + (size_t)t * row_stride);
+    auto pv_row = [&](u4_t raw, int t) {
       float vf[EPL];
       if constexpr (sizeof(AT) == 2) {
 #pragma unroll
@@ -166,7 +182,13 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
 #pragma unroll
         for (int e = 0; e < EPL; e++) of[j][e] = fmaf(p, vf[e], of[j][e]);
       }
+    };
+#pragma unroll
+    for (int i = 0; i < NPRE; i++) {
+      const int t = t0 + (wave + i * NW) * RPI + grp;
+      if (t < t1) pv_row(vpre[i], t);
     }
+    for (int t = t0 + (wave + NPRE * NW) * RPI + grp; t < t1; t += NW * RPI) pv_row(*(const u4_t *)(vbase + (size_t)t * row_stride), t);
     // lanes with the same `sub` hold different rows: fold the RPI groups of the wavefront together
 #pragma unroll
     for (int j = 0; j < NREP; j++)
@@ -214,28 +236,50 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
     if (!sm.is_last) return;
     // merge: one wavefront per query head turns the per-chunk (m, l) into weights exp(m_s - M) and 1/L ...
     const float *base = a.partial + (size_t)g * a.nsplit * NREP * (HD + 2);
+    constexpr int MSL = ATT_CHUNK_MAX / 64;   // chunks per lane
     for (int j = wave; j < NREP; j += NW) {
+      float ms[MSL], ls[MSL];                  // (m, l) of this lane's chunks, all requested in one go
+#pragma unroll
+      for (int i = 0; i < MSL; i++) {
+        const int s_ = lane + i * 64;
+        if (i * 64 < n_active) {               // same for the whole wavefront
+          const float *ps = base + ((size_t)(s_ < n_active ? s_ : n_active - 1) * NREP + j) * (HD + 2);
+          ms[i] = ld_coherent(ps + HD);
+          ls[i] = ld_coherent(ps + HD + 1);
+        }
+      }
       float M = -INFINITY;
-      for (int s = lane; s < n_active; s += 64) M = fmaxf(M, ld_coherent(base + ((size_t)s * NREP + j) * (HD + 2) + HD));
+#pragma unroll
+      for (int i = 0; i < MSL; i++)
+        if (lane + i * 64 < n_active) M = fmaxf(M, ms[i]);
       M = wave_max(M);
       float L = 0.0f;
-      for (int s = lane; s < n_active; s += 64) {
-        const float *ps = base + ((size_t)s * NREP + j) * (HD + 2);
-        const float w = exp_f32(ld_coherent(ps + HD) - M);
-        sm.sc[j][s] = w;  // n_active <= nsplit <= ATT_CHUNK_MAX
-        L = fmaf(ld_coherent(ps + HD + 1), w, L);
+#pragma unroll
+      for (int i = 0; i < MSL; i++) {
+        const int s_ = lane + i * 64;
+        if (s_ < n_active) {
+          const float w = exp_f32(ms[i] - M);
+          sm.sc[j][s_] = w;  // n_active <= nsplit <= ATT_CHUNK_MAX
+          L = fmaf(ls[i], w, L);
+        }
       }
       L = wave_sum(L);
       if (lane == 0) sm.l_sh[j] = 1.0f / L;  // softmax normalisation is e * (1/sum) (tensor.ts:2211-2214)
     }
     __syncthreads();
-    // ... then every thread sums its output elements over the chunks; the loads are independent, so they pipeline
+    // ... then every thread sums its output elements over the chunks, 32 chunks per round trip, in chunk order
     for (int i = tid; i < NREP * HD; i += nthreads) {
       const int j = i / HD, d = i % HD;
       const float *po = base + (size_t)j * (HD + 2) + d;
       float O = 0.0f;
-#pragma unroll 8
-      for (int s = 0; s < n_active; s++) O = fmaf(ld_coherent(po + (size_t)s * NREP * (HD + 2)), sm.sc[j][s], O);
+      for (int s0 = 0; s0 < n_active; s0 += 32) {
+        float part[32];
+#pragma unroll
+        for (int u = 0; u < 32; u++) part[u] = ld_coherent(po + (size_t)(s0 + u < n_active ? s0 + u : n_active - 1) * NREP * (HD + 2));
+#pragma unroll
+        for (int u = 0; u < 32; u++)
+          if (s0 + u < n_active) O = fmaf(part[u], sm.sc[j][s0 + u], O);
+      }
       AT *dst = (AT *)a.out + (size_t)(g * NREP + j) * HD + d;
       const float r = Act<AT>::rn(O * sm.l_sh[j]);  // the cast of the P.V result
       if constexpr (COHERENT) st_coherent(dst, (AT)r);
