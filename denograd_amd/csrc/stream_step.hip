@@ -48,6 +48,7 @@ constexpr int SS_NORM_CHUNKS = 8;                // 16-byte chunks of the input 
 // workspace layout (bytes)
 constexpr size_t SS_WS_EPOCH = 0, SS_WS_ERR = 128, SS_WS_COUNTERS = 256, SS_WS_AMAX_VAL = 512, SS_WS_AMAX_IDX = 512 + 4096,
                  SS_WS_FLAGS = 16384, SS_WS_PARTIAL = SS_WS_FLAGS + (size_t)SS_MAX_BLOCKS * SS_FLAG_STRIDE * 4;
+constexpr int SS_TAG_DIM = SS_NORM_CHUNKS * 512, SS_TAG_HIDDEN = 65536;   // entries reserved for the tagged h / h2 rows and the g row
 
 struct SsLayer {   // = jsgrad_hip_layer_t
   const void *wq, *wk, *wv, *wo, *w1, *w2, *w3;
@@ -64,6 +65,8 @@ struct SsArgs {
   int32_t *state, *tokens_out;
   int tokens_cap;
   void *h, *h2, *q, *attn, *g, *logits;
+  // activation rows as they pass between blocks: one 32-bit word per element, fp16 value | version tag << 16
+  uint32_t *th, *th2, *tg, *tattn, *tq, *tkv;   // dim, dim, hidden, n_heads*hd, n_heads*hd, 2 * n_kv_heads*hd (k | v of this position)
   int *epoch, *err, *flags, *attn_counters;
   float *attn_partial;   // [n_kv_heads][SS_MAXCH][n_rep][HD + 2]
   float *amax_val;
@@ -135,6 +138,57 @@ __device__ __forceinline__ void st16_coherent(void *p, u4_t v) {
   __hip_atomic_store(q + 1, (uint64_t)v[2] | ((uint64_t)v[3] << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// ---- tagged rows: how activations pass from block to block ------------------------------------------------------------
+// An element of a row that other blocks read is one 32-bit word: the fp16 value below, the version of the phase that wrote
+// it above.  A reader asks for the words and takes them when every tag is the version it expects, else it asks again: the
+// data is its own flag, so a writer neither waits for its stores to be acknowledged nor raises a flag, and a reader needs
+// no round trip for a flag before the round trip for the data.  Nothing is overwritten too early: a block writes the
+// outputs of phase p + 1 only after it has seen every output of phase p, and whoever wrote those had finished reading
+// whatever it read in phases up to p.
+__device__ __forceinline__ uint32_t ss_tag(int version) { return (uint32_t)version % 65535u + 1u; }   // never 0: fresh memory matches nothing
+__device__ __forceinline__ uint32_t ss_tagged(uint32_t tag, float v) {
+  const _Float16 h = (_Float16)v;
+  return (tag << 16) | (uint32_t)__builtin_bit_cast(uint16_t, h);
+}
+__device__ __forceinline__ void st_tagged(uint32_t *p, uint32_t tag, float v) { st_coherent((int *)p, (int)ss_tagged(tag, v)); }
+__device__ __forceinline__ float ld_tagged_value(const uint32_t *p) {   // a word known to be there: its value
+  const uint32_t w = (uint32_t)ld_coherent((const int *)p);
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu));
+}
+// A tagged row as a buffer resource: 16-byte loads that are coherent across the device (sc1, like the agent-scope atomic
+// loads, which exist up to 64 bits only); a word is the unit that has to arrive whole, and every word carries its own tag.
+typedef __amdgpu_buffer_rsrc_t TagRow;
+__device__ __forceinline__ TagRow tag_row(const uint32_t *p, int n) {
+  return __builtin_amdgcn_make_buffer_rsrc((void *)(uintptr_t)uni64((uint64_t)(uintptr_t)p), 0, n * 4, 0x00020000);
+}
+// eight tagged words -> eight packed halves; ok: all eight carry `tag`
+__device__ __forceinline__ u4_t ss_untag8(u4_t a, u4_t b, uint32_t tag, bool &ok);
+// (words i .. i + 7 of a row given as a buffer resource: the few loads of an attention item)
+__device__ __forceinline__ u4_t ld8_tagged(TagRow row, int i, uint32_t tag, bool &ok) {
+  return ss_untag8(__builtin_amdgcn_raw_buffer_load_b128(row, i * 4, 0, 16), __builtin_amdgcn_raw_buffer_load_b128(row, i * 4 + 16, 0, 16), tag, ok);
+}
+// (32 bytes at p, as four 64-bit agent-scope loads: staging a whole row this way measured faster than with 16-byte loads)
+__device__ __forceinline__ u4_t ld8_tagged(const uint32_t *p, uint32_t tag, bool &ok) { return ss_untag8(ld16_coherent(p), ld16_coherent(p + 4), tag, ok); }
+__device__ __forceinline__ u4_t ss_untag8(u4_t a, u4_t b, uint32_t tag, bool &ok) {
+  const uint32_t e = tag << 16;
+  const uint32_t bad = ((a[0] ^ e) | (a[1] ^ e) | (a[2] ^ e) | (a[3] ^ e) | (b[0] ^ e) | (b[1] ^ e) | (b[2] ^ e) | (b[3] ^ e)) >> 16;
+  ok = ok && bad == 0;
+  return u4_t{(a[0] & 0xffffu) | (a[1] << 16), (a[2] & 0xffffu) | (a[3] << 16), (b[0] & 0xffffu) | (b[1] << 16), (b[2] & 0xffffu) | (b[3] << 16)};
+}
+
+// One more round of a wait on tagged rows; false: give up (the error word is set and nobody waits any more).
+__device__ __forceinline__ bool ss_poll_again(const SsArgs &s, SsCtl &ctl, int &it) {
+  if ((++it & 15) == 0) {
+    if (lds_ld(&ctl.abort) != 0) return false;
+    if (it > SS_SPIN_GLOBAL || ld_coherent(s.err) != 0) {
+      st_coherent(s.err, 1);
+      lds_st(&ctl.abort, 1);
+      return false;
+    }
+  }
+  return true;
+}
+
 // Wait until an LDS word reaches `target`.  Returns false when the wait was abandoned.
 __device__ __forceinline__ bool lds_wait(const SsArgs &s, SsCtl &ctl, const int *word, int target) {
   int it = 0;
@@ -204,19 +258,19 @@ __device__ __forceinline__ void ss_build_phase(const SsArgs &s, uint64_t *rec, i
   const int qdim = s.n_heads * s.head_dim, kvdim = s.n_kv_heads * s.head_dim;
   if (k == PH_QKV) {
     w0 = ldg(L + 0); w1 = ldg(L + 1); w2 = ldg(L + 2); s0 = ldg(L + 7); s1 = ldg(L + 8); s2 = ldg(L + 9);
-    rows0 = qdim; rows1 = kvdim; rows2 = kvdim; in_f = s.dim; src = (uint64_t)(uintptr_t)s.h; norm_w = ldg(L + 14);
+    rows0 = qdim; rows1 = kvdim; rows2 = kvdim; in_f = s.dim; src = (uint64_t)(uintptr_t)s.th; norm_w = ldg(L + 14);
   } else if (k == PH_WO) {
     w0 = ldg(L + 3); s0 = ldg(L + 10); rows0 = s.dim; in_f = qdim;
-    src = (uint64_t)(uintptr_t)s.attn; residual = (uint64_t)(uintptr_t)s.h; y = (uint64_t)(uintptr_t)s.h2;
+    src = (uint64_t)(uintptr_t)s.tattn; residual = (uint64_t)(uintptr_t)s.th; y = (uint64_t)(uintptr_t)s.th2;
   } else if (k == PH_FFN) {
     w0 = ldg(L + 4); w1 = ldg(L + 6); s0 = ldg(L + 11); s1 = ldg(L + 13); rows0 = s.hidden; in_f = s.dim; nm = 2;
-    src = (uint64_t)(uintptr_t)s.h2; norm_w = ldg(L + 15); y = (uint64_t)(uintptr_t)s.g;
+    src = (uint64_t)(uintptr_t)s.th2; norm_w = ldg(L + 15); y = (uint64_t)(uintptr_t)s.tg;
   } else if (k == PH_W2) {
     w0 = ldg(L + 5); s0 = ldg(L + 12); rows0 = s.dim; in_f = s.hidden;
-    src = (uint64_t)(uintptr_t)s.g; residual = (uint64_t)(uintptr_t)s.h2; y = (uint64_t)(uintptr_t)s.h;
+    src = (uint64_t)(uintptr_t)s.tg; residual = (uint64_t)(uintptr_t)s.th2; y = (uint64_t)(uintptr_t)s.th;
   } else if (k == PH_LM) {
     w0 = (uint64_t)(uintptr_t)s.out_w; s0 = (uint64_t)(uintptr_t)s.out_s; rows0 = s.vocab; in_f = s.dim;
-    src = (uint64_t)(uintptr_t)s.h; norm_w = (uint64_t)(uintptr_t)s.final_norm; y = (uint64_t)(uintptr_t)s.logits;
+    src = (uint64_t)(uintptr_t)s.th; norm_w = (uint64_t)(uintptr_t)s.final_norm; y = (uint64_t)(uintptr_t)s.logits;
   }
   rec[0] = w0; rec[1] = w1; rec[2] = w2; rec[3] = s0; rec[4] = s1; rec[5] = s2; rec[6] = src; rec[7] = norm_w; rec[8] = residual; rec[9] = y;
   rec[10] = (uint32_t)rows0 | ((uint64_t)(uint32_t)rows1 << 32);
@@ -558,7 +612,8 @@ template <int HD, int NREP> struct SsAttn {
       }
     }
   }
-  __device__ static void item(const SsArgs &s, const SsLayer &L, float *sc, int g, int c, int T, int chunk, int n_active) {
+  // tin: version of the queries and of this position's k / v rows; tout: version the output row gets
+  __device__ static void item(const SsArgs &s, SsCtl &ctl, const SsLayer &L, float *sc, int g, int c, int T, int chunk, int n_active, uint32_t tin, uint32_t tout) {
     typedef _Float16 AT;
     const int lane = threadIdx.x & 63, sub = lane % GL, grp = lane / GL;
     const int t0 = c * chunk, t1 = min(T, t0 + chunk), CH = t1 - t0;
@@ -579,19 +634,45 @@ template <int HD, int NREP> struct SsAttn {
     };
     load_batch(kraw, kbase, t0);
     load_batch(vraw, vbase, t0);
+    // The queries, and for the chunk that ends at this position its k and v rows (their cache rows are being written by
+    // other blocks right now, for later tokens to read), come as tagged rows.
+    const bool has_cur = t1 == T;
+    const int kvdim = s.n_kv_heads * HD;
     h2_t qh[NREP][4];
+    u4_t kcur = {0, 0, 0, 0}, vcur = {0, 0, 0, 0};
+    const TagRow rq = tag_row(s.tq, s.n_heads * HD), rkv = tag_row(s.tkv, 2 * kvdim);
+    for (int it = 0;;) {
+      bool ok = true;
 #pragma unroll
-    for (int j = 0; j < NREP; j++) {
-      const u4_t raw = ld16_coherent((const AT *)s.q + (size_t)(g * NREP + j) * HD + sub * 8);
+      for (int j = 0; j < NREP; j++) {
+        const u4_t raw = ld8_tagged(rq, (g * NREP + j) * HD + sub * 8, tin, ok);
 #pragma unroll
-      for (int e = 0; e < 4; e++) qh[j][e] = as_h2(raw[e]);
+        for (int e = 0; e < 4; e++) qh[j][e] = as_h2(raw[e]);
+      }
+      if (has_cur) {
+        kcur = ld8_tagged(rkv, g * HD + sub * 8, tin, ok);
+        vcur = ld8_tagged(rkv, kvdim + g * HD + sub * 8, tin, ok);
+      }
+      if (__all(ok) || !ss_poll_again(s, ctl, it)) break;
+    }
+    if (has_cur && T - 1 - t0 < BR) {   // the row sits in the first batch: replace what came from the cache
+#pragma unroll
+      for (int u = 0; u < NLD; u++)
+        if (t0 + u * RPI + grp == T - 1) { kraw[u] = kcur; vraw[u] = vcur; }
     }
     // scores of the chunk and their maximum
     float mx[NREP];
 #pragma unroll
     for (int j = 0; j < NREP; j++) mx[j] = -INFINITY;
     for (int tb = t0; tb < t1; tb += BR) {
-      if (tb != t0) load_batch(kraw, kbase, tb);
+      if (tb != t0) {
+        load_batch(kraw, kbase, tb);
+        if (has_cur) {
+#pragma unroll
+          for (int u = 0; u < NLD; u++)
+            if (tb + u * RPI + grp == T - 1) kraw[u] = kcur;
+        }
+      }
 #pragma unroll
       for (int u = 0; u < NLD; u++) {
         const int t = tb + u * RPI + grp;
@@ -630,7 +711,14 @@ template <int HD, int NREP> struct SsAttn {
 #pragma unroll
       for (int e = 0; e < 8; e++) of[j][e] = 0.0f;
     for (int tb = t0; tb < t1; tb += BR) {
-      if (tb != t0) load_batch(vraw, vbase, tb);
+      if (tb != t0) {
+        load_batch(vraw, vbase, tb);
+        if (has_cur) {
+#pragma unroll
+          for (int u = 0; u < NLD; u++)
+            if (tb + u * RPI + grp == T - 1) vraw[u] = vcur;
+        }
+      }
 #pragma unroll
       for (int u = 0; u < NLD; u++) {
         const int t = tb + u * RPI + grp;
@@ -676,6 +764,8 @@ template <int HD, int NREP> struct SsAttn {
     old = __builtin_amdgcn_readfirstlane(old);
     astamp(s, 5);
     if (old != n_active - 1) return;
+    // the counter is zero again long before the next layer counts on it (four hand-offs away)
+    if (lane == 0) __hip_atomic_store(&s.attn_counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
     // ---- merge the chunks of kv head g: weights exp(m_s - M), normalisation 1 / sum(l_s * w_s)
     const float *base = s.attn_partial + (size_t)g * SS_MAXCH * NREP * (HD + 2);
@@ -733,14 +823,13 @@ template <int HD, int NREP> struct SsAttn {
       float iv = inv[0];
 #pragma unroll
       for (int j = 1; j < NREP; j++) iv = jj[i] == j ? inv[j] : iv;
-      st_coherent((AT *)s.attn + (size_t)g * NREP * HD + i * 64 + lane, (AT)rn16(O[i] * iv));
+      st_tagged(s.tattn + (size_t)g * NREP * HD + i * 64 + lane, tout, rn16(O[i] * iv));
     }
-    if (lane == 0) __hip_atomic_store(&s.attn_counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     astamp(s, 6);
   }
 
   // the attention phase of layer l as the control wavefront of this block runs it: items block, block + G, ...
-  __device__ static __forceinline__ void phase(const SsArgs &s, const SsTabs &lt, SsCtl &ctl, float *sc, int l, int pos) {
+  __device__ static __forceinline__ void phase(const SsArgs &s, const SsTabs &lt, SsCtl &ctl, float *sc, int l, int pos, uint32_t tin, uint32_t tout) {
     const int G = gridDim.x;
     const bool pos_ok = pos >= 0 && pos < s.max_context;
     astamp(s, 1);
@@ -750,9 +839,8 @@ template <int HD, int NREP> struct SsAttn {
       const int n_active = (T + chunk - 1) / chunk;
       const SsLayer L = ss_layer(lt, l);
       for (int item_id = blockIdx.x; item_id < s.n_kv_heads * n_active; item_id += G)
-        item(s, L, sc, item_id / n_active, item_id % n_active, T, chunk, n_active);
+        item(s, ctl, L, sc, item_id / n_active, item_id % n_active, T, chunk, n_active, tin, tout);
     }
-    vm_drain();   // this wavefront's outputs are at the coherence point
     astamp(s, 7);
   }
 };
@@ -789,36 +877,49 @@ template <int KIND, int HD, int NREP> struct SsControl {
     }
   }
 
-  // 16-byte chunk c of the input row: written by other blocks in the activation dtype, or (EMB_I8) eight codes of an
-  // int8 embedding row, each becoming RN16(code * scale) (llama3.ts:71-77)
-  template <bool EMB_I8> __device__ static __forceinline__ u4_t fetch_x(const void *src, int c, float emb_scale) {
-    if constexpr (!EMB_I8) {
-      return ld16_coherent((const u4_t *)src + c);
-    } else {
-      const uint64_t raw = ldg((const uint64_t *)src + c);
-      u4_t o;
+  // where the input row of a phase comes from: a tagged row written by other blocks, or a row of the embedding table
+  enum { SRC_TAGGED = 0, SRC_EMB_F16 = 1, SRC_EMB_I8 = 2 };
+  // N chunks of 8 halves of the input row for this lane: chunks c_first + i * 64 + lane (lanes past the end re-read the last
+  // chunk: a load under a lane mask costs a full wait).  Tagged rows are asked for until every word carries `tag`.  An int8
+  // embedding row becomes RN16(code * scale) per element (llama3.ts:71-77).
+  template <int MODE, int N>
+  __device__ static __forceinline__ void fetch_chunks(const SsArgs &s, SsCtl &ctl, const void *src, int c_first, int nchunks, uint32_t tag, float emb_scale, u4_t (&out)[N]) {
+    const int lane = threadIdx.x & 63;
+    if constexpr (MODE == SRC_TAGGED) {
+      for (int it = 0;;) {
+        bool ok = true;
 #pragma unroll
-      for (int e = 0; e < 4; e++) {
-        h2_t y;
-        y[0] = mul_rn16((float)(int8_t)(raw >> (16 * e)), emb_scale);
-        y[1] = mul_rn16((float)(int8_t)(raw >> (16 * e + 8)), emb_scale);
-        o[e] = __builtin_bit_cast(uint32_t, y);
+        for (int i = 0; i < N; i++) {
+          const int c = c_first + i * 64 + lane;
+          out[i] = ld8_tagged((const uint32_t *)src + (size_t)(c < nchunks ? c : nchunks - 1) * 8, tag, ok);
+        }
+        if (__all(ok) || !ss_poll_again(s, ctl, it)) return;
       }
-      return o;
+    } else {
+#pragma unroll
+      for (int i = 0; i < N; i++) {
+        const int c = c_first + i * 64 + lane, cc = c < nchunks ? c : nchunks - 1;
+        if constexpr (MODE == SRC_EMB_F16) {
+          out[i] = ldg((const u4_t *)src + cc);
+        } else {
+          const uint64_t raw = ldg((const uint64_t *)src + cc);
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            h2_t y;
+            y[0] = mul_rn16((float)(int8_t)(raw >> (16 * e)), emb_scale);
+            y[1] = mul_rn16((float)(int8_t)(raw >> (16 * e + 8)), emb_scale);
+            out[i][e] = __builtin_bit_cast(uint32_t, y);
+          }
+        }
+      }
     }
   }
   // RMSNorm'ed row -> LDS (nn/index.ts:586-588); a lane keeps NR chunks between the sum of squares and the scaling.
-  // Loads are unconditional (lanes past the end re-read the last chunk): a load under a lane mask costs a full wait.
-  // mirror: where the raw row is left for later phases (block 0 and the embedding row only).
-  template <bool EMB_I8, int NR>
-  __device__ static __forceinline__ void stage_norm(const SsArgs &s, u4_t *xl, const void *src, const void *norm_w, int nchunks, float inv_d, float emb_scale, void *mirror) {
+  template <int MODE, int NR>
+  __device__ static __forceinline__ void stage_norm(const SsArgs &s, SsCtl &ctl, u4_t *xl, const void *src, const void *norm_w, int nchunks, float inv_d, uint32_t tag, float emb_scale) {
     const int lane = threadIdx.x & 63;
     u4_t xr[NR];
-#pragma unroll
-    for (int i = 0; i < NR; i++) {
-      const int c = i * 64 + lane;
-      xr[i] = fetch_x<EMB_I8>(src, c < nchunks ? c : nchunks - 1, emb_scale);
-    }
+    fetch_chunks<MODE, NR>(s, ctl, src, 0, nchunks, tag, emb_scale, xr);
     float ss = 0.0f;
 #pragma unroll
     for (int i = 0; i < NR; i++) {
@@ -831,7 +932,6 @@ template <int KIND, int HD, int NREP> struct SsControl {
         part = fmaf((float)h[1], (float)h[1], part);
       }
       ss = c < nchunks ? part : ss;
-      if (mirror != nullptr && c < nchunks) st16_coherent((u4_t *)mirror + c, xr[i]);
     }
     const float tot = wave_sum(ss);
     // sqrt(1 / (mean + eps)), mean = sum * float(1/d)  (nn/index.ts:586, tensor.ts:2944-2946)
@@ -861,24 +961,21 @@ template <int KIND, int HD, int NREP> struct SsControl {
       }
     }
   }
-  // Stage the input row of a weight phase in LDS.  src: in_f halves written by other blocks (or the embedding row);
-  // norm_w != nullptr applies RMSNorm.  The tail up to `padded` is zeroed.
-  template <bool EMB_I8>
-  __device__ static __forceinline__ void stage_x(const SsArgs &s, AT *xs, const void *src, const void *norm_w, int in_f, int padded, float inv_d, float emb_scale, void *mirror) {
+  // Stage the input row of a weight phase in LDS.  src: in_f elements (tagged words written by other blocks, or the embedding
+  // row); norm_w != nullptr applies RMSNorm.  The tail up to `padded` is zeroed.
+  template <int MODE>
+  __device__ static __forceinline__ void stage_x(const SsArgs &s, SsCtl &ctl, AT *xs, const void *src, const void *norm_w, int in_f, int padded, float inv_d, uint32_t tag, float emb_scale) {
     const int lane = threadIdx.x & 63;
     const int nchunks = in_f / 8;
     u4_t *xl = (u4_t *)xs;
     for (int c = nchunks + lane; c < padded / 8; c += 64) xl[c] = u4_t{0, 0, 0, 0};
     if (norm_w == nullptr) {
-      for (int c0 = 0; c0 < nchunks; c0 += 64 * 8) {
-        u4_t t[8];
+      constexpr int NB = 8;    // 32 loads of 8 bytes per lane and round trip
+      for (int c0 = 0; c0 < nchunks; c0 += 64 * NB) {
+        u4_t t[NB];
+        fetch_chunks<MODE, NB>(s, ctl, src, c0, nchunks, tag, emb_scale, t);
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-          const int c = c0 + i * 64 + lane;
-          t[i] = fetch_x<EMB_I8>(src, c < nchunks ? c : nchunks - 1, emb_scale);
-        }
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
+        for (int i = 0; i < NB; i++) {
           const int c = c0 + i * 64 + lane;
           if (c < nchunks) xl[c] = t[i];
         }
@@ -886,10 +983,10 @@ template <int KIND, int HD, int NREP> struct SsControl {
       return;
     }
     const int nr = (nchunks + 63) / 64;   // <= SS_NORM_CHUNKS (host)
-    if (nr <= 1) stage_norm<EMB_I8, 1>(s, xl, src, norm_w, nchunks, inv_d, emb_scale, mirror);
-    else if (nr <= 2) stage_norm<EMB_I8, 2>(s, xl, src, norm_w, nchunks, inv_d, emb_scale, mirror);
-    else if (nr <= 4) stage_norm<EMB_I8, 4>(s, xl, src, norm_w, nchunks, inv_d, emb_scale, mirror);
-    else stage_norm<EMB_I8, 8>(s, xl, src, norm_w, nchunks, inv_d, emb_scale, mirror);
+    if (nr <= 1) stage_norm<MODE, 1>(s, ctl, xl, src, norm_w, nchunks, inv_d, tag, emb_scale);
+    else if (nr <= 2) stage_norm<MODE, 2>(s, ctl, xl, src, norm_w, nchunks, inv_d, tag, emb_scale);
+    else if (nr <= 4) stage_norm<MODE, 4>(s, ctl, xl, src, norm_w, nchunks, inv_d, tag, emb_scale);
+    else stage_norm<MODE, 8>(s, ctl, xl, src, norm_w, nchunks, inv_d, tag, emb_scale);
   }
 
   // what the epilogue of one 64-slot pass needs besides the sums
@@ -906,6 +1003,11 @@ template <int KIND, int HD, int NREP> struct SsControl {
     SsLayer L;
     int pos;
     bool pos_ok;
+    uint32_t tout;          // version tag of the rows this phase writes
+    // layer 0: the residual of wo is the embedding row itself (every block reads it from the table)
+    const void *emb_row;    // null: the residual is a tagged row
+    bool emb_i8;
+    float emb_scale;
   };
   // slot -> stacked row of the phase (or -1): slot = 2 * (local group of this block) + row of the pair
   __device__ static __forceinline__ int slot_row(const EpiCtx &e, int slot) {
@@ -938,7 +1040,10 @@ template <int KIND, int HD, int NREP> struct SsControl {
         o.e1 = (float)ldg(tp + 1);
       }
     } else if (e.residual != nullptr) {
-      o.e0 = (float)ld_coherent((const AT *)e.residual + row);
+      // a tagged row this block has already seen complete (it staged all of it one or two phases ago)
+      if (e.emb_row == nullptr) o.e0 = ld_tagged_value((const uint32_t *)e.residual + row);
+      else if (e.emb_i8) o.e0 = mul_rn16((float)ldg((const int8_t *)e.emb_row + row), e.emb_scale);
+      else o.e0 = (float)ldg((const AT *)e.emb_row + row);
     }
     return o;
   }
@@ -964,21 +1069,27 @@ template <int KIND, int HD, int NREP> struct SsControl {
       int m, rr;
       locate(e.d, row, m, rr);
       if (m == 2) {
-        st_coherent((AT *)e.L.cache_v + (size_t)e.pos * e.d.rows2 + rr, (AT)v0);
+        st_coherent((AT *)e.L.cache_v + (size_t)e.pos * e.d.rows2 + rr, (AT)v0);   // for later tokens
+        st_tagged(s.tkv + e.d.rows1 + rr, e.tout, v0);                              // for this token's attention
       } else {
         // interleaved pairs (llama.ts:17-32): (a, b) -> (a cos - b sin, a sin + b cos), unfused as in plain C
         const float c = o.e0, d = o.e1;
         const float out = (row & 1) ? rn16(partner * d + v0 * c) : rn16(v0 * c - partner * d);
-        AT *dst = m == 0 ? (AT *)s.q : (AT *)e.L.cache_k + (size_t)e.pos * e.d.rows1;
-        st_coherent(dst + rr, (AT)out);
+        if (m == 0) st_tagged(s.tq + rr, e.tout, out);
+        else {
+          st_coherent((AT *)e.L.cache_k + (size_t)e.pos * e.d.rows1 + rr, (AT)out);
+          st_tagged(s.tkv + rr, e.tout, out);
+        }
       }
     } else if (e.kind == PH_FFN) {
-      st_coherent((AT *)e.y + row, (AT)rn16(silu_act<AT>(v0) * v1));
+      st_tagged((uint32_t *)e.y + row, e.tout, rn16(silu_act<AT>(v0) * v1));
+    } else if (e.kind == PH_LM) {
+      st_coherent((AT *)e.y + row, (AT)v0);
+      if (v0 > best || (v0 == best && row < best_i)) { best = v0; best_i = row; }
     } else {
       float v = v0;
       if (e.residual != nullptr) v = rn16(o.e0 + v);
-      st_coherent((AT *)e.y + row, (AT)v);
-      if (e.kind == PH_LM && (v > best || (v == best && row < best_i))) { best = v; best_i = row; }
+      st_tagged((uint32_t *)e.y + row, e.tout, v);
     }
   }
 
@@ -993,13 +1104,14 @@ template <int KIND, int HD, int NREP> struct SsControl {
     stamp();
     float best = -INFINITY;
     int best_i = 0x7fffffff;
+    if (!pos_ok && lane == 0) lds_st(&ctl.abort, 1);   // nothing will be written for such a position: nobody waits
     for (int p = 0; p < nph; p++) {
       const int kind = ss_kind(s, p);
-      if (p > 0) wait_flags(s, ctl, base + p);
+      const uint32_t tin = ss_tag(base + p), tout = ss_tag(base + p + 1);   // versions of what the phase reads and writes
       stamp();
       if (kind == PH_ATTN) {
         stamp();
-        SsAttn<HD, NREP>::phase(s, lt, ctl, att_sc, p / 5, pos);
+        SsAttn<HD, NREP>::phase(s, lt, ctl, att_sc, p / 5, pos, tin, tout);
         stamp();
       } else {
         EpiCtx e;
@@ -1009,23 +1121,24 @@ template <int KIND, int HD, int NREP> struct SsControl {
         e.nb = F::nbatch(e.d);
         e.pos = pos;
         e.pos_ok = pos_ok;
+        e.tout = tout;
         e.L = ss_layer(lt, kind == PH_LM ? 0 : p / 5);
         e.residual = e.d.residual;
         e.y = e.d.y;
-        const void *src = e.d.src, *norm_w = e.d.norm_w;
-        bool emb_i8 = false;
+        // the embedding row (Embedding.call: a row gather) is the input of the first phase and the residual of the first wo
+        const bool emb_i8 = s.embed_kind == JSGRAD_W_I8;
+        const void *emb_row = (const char *)s.tok_emb + (size_t)tok * s.dim * (emb_i8 ? 1 : 2);
         float emb_scale = 1.0f;
-        void *mirror = nullptr;
-        if (p == 0) {   // the embedding row is the first input (Embedding.call: a row gather); block 0 also leaves it in h
-          emb_i8 = s.embed_kind == JSGRAD_W_I8;
-          src = (const char *)s.tok_emb + (size_t)tok * s.dim * (emb_i8 ? 1 : 2);
-          if (emb_i8) emb_scale = (float)ldg((const _Float16 *)s.tok_scale + tok);
-          if (blockIdx.x == 0) mirror = s.h;
-        }
+        if (emb_i8 && p < 5) emb_scale = (float)ldg((const _Float16 *)s.tok_scale + tok);
+        e.emb_row = p == PH_WO ? emb_row : nullptr;
+        e.emb_i8 = emb_i8;
+        e.emb_scale = emb_scale;
+        const void *src = e.d.src, *norm_w = e.d.norm_w;
         const int padded = F::nbatch(e.d) * F::unroll(e.d.nm) * F::STEP;
         const float inv_d = (float)(1.0 / (double)e.d.in_f);
-        if (emb_i8) stage_x<true>(s, xs, src, norm_w, e.d.in_f, padded, inv_d, emb_scale, mirror);
-        else stage_x<false>(s, xs, src, norm_w, e.d.in_f, padded, inv_d, emb_scale, mirror);
+        if (p != 0) stage_x<SRC_TAGGED>(s, ctl, xs, src, norm_w, e.d.in_f, padded, inv_d, tin, 1.0f);
+        else if (emb_i8) stage_x<SRC_EMB_I8>(s, ctl, xs, emb_row, norm_w, e.d.in_f, padded, inv_d, tin, emb_scale);
+        else stage_x<SRC_EMB_F16>(s, ctl, xs, emb_row, norm_w, e.d.in_f, padded, inv_d, tin, emb_scale);
         lds_fence();
         lds_st(&ctl.x_ready, ss_wordinal(s, p) + 1);
         stamp();
@@ -1047,11 +1160,12 @@ template <int KIND, int HD, int NREP> struct SsControl {
             if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
           }
           if (lane == 0) { st_coherent(&s.amax_val[blockIdx.x], best); st_coherent(&s.amax_idx[blockIdx.x], best_i); }
+          // the one flag of the step: this block's logits and arg-max partial are at the coherence point
+          vm_drain();
+          if (lane == 0) st_coherent(&s.flags[blockIdx.x * SS_FLAG_STRIDE], base + nph);
         }
-        vm_drain();   // every store of this phase is at the coherence point
         stamp();
       }
-      if (lane == 0) st_coherent(&s.flags[blockIdx.x * SS_FLAG_STRIDE], base + p + 1);
     }
     if (blockIdx.x != 0) return;
     // ---- greedy arg-max over the blocks' partials (Tensor.argmax: lowest index among the maxima), state update
@@ -1130,8 +1244,10 @@ using namespace jsg;
 extern "C" {
 
 size_t jsgrad_hip_stream_workspace_bytes(int n_heads, int n_kv_heads, int head_dim) {
-  (void)n_kv_heads;
-  return SS_WS_PARTIAL + (size_t)n_heads * SS_MAXCH * (head_dim + 2) * sizeof(float);
+  // flags and counters | attention partials | tagged rows: h, h2 (SS_TAG_DIM each), g (SS_TAG_HIDDEN), attn, q, k | v of the position
+  const size_t partial = (size_t)n_heads * SS_MAXCH * (head_dim + 2) * sizeof(float);
+  const size_t tagged = ((size_t)2 * SS_TAG_DIM + SS_TAG_HIDDEN + (size_t)2 * n_heads * head_dim + (size_t)2 * n_kv_heads * head_dim) * sizeof(uint32_t);
+  return SS_WS_PARTIAL + partial + tagged;
 }
 
 int jsgrad_hip_stream_step(const jsgrad_hip_step_t *d) {
@@ -1151,6 +1267,8 @@ int jsgrad_hip_stream_step(const jsgrad_hip_step_t *d) {
   JSG_REQUIRE(d->dim % vec == 0 && d->hidden % vec == 0 && qdim % vec == 0, "%s: feature sizes must be multiples of %d", who, vec);
   JSG_REQUIRE(d->dim % 2 == 0 && d->hidden % 2 == 0 && d->vocab % 2 == 0, "%s: row counts must be even", who);
   JSG_REQUIRE(d->dim <= SS_NORM_CHUNKS * 64 * 8, "%s: dim %d exceeds the fused RMSNorm limit of %d", who, d->dim, SS_NORM_CHUNKS * 64 * 8);
+  JSG_REQUIRE(d->dim <= SS_TAG_DIM && d->hidden <= SS_TAG_HIDDEN, "%s: dim %d / hidden %d exceed the workspace rows of %d / %d", who, d->dim, d->hidden, SS_TAG_DIM, SS_TAG_HIDDEN);
+  JSG_REQUIRE(d->dim % 8 == 0 && d->hidden % 8 == 0 && qdim % 8 == 0, "%s: feature sizes must be multiples of 8", who);
   JSG_REQUIRE(d->kind == JSGRAD_W_F16 || d->out_s, "%s: quantised lm_head needs a scale", who);
   JSG_REQUIRE(d->max_context <= SS_MAXCH * SS_CHUNK, "%s: max_context %d exceeds %d", who, d->max_context, SS_MAXCH * SS_CHUNK);
   const int grid = state().cu_count;   // one block per CU: every block is resident, which the flags need
@@ -1189,6 +1307,12 @@ int jsgrad_hip_stream_step(const jsgrad_hip_step_t *d) {
   s.amax_idx = (int *)(ws + SS_WS_AMAX_IDX);
   s.flags = (int *)(ws + SS_WS_FLAGS);
   s.attn_partial = (float *)(ws + SS_WS_PARTIAL);
+  s.th = (uint32_t *)(ws + SS_WS_PARTIAL + (size_t)d->n_heads * SS_MAXCH * (d->head_dim + 2) * sizeof(float));
+  s.th2 = s.th + SS_TAG_DIM;
+  s.tg = s.th2 + SS_TAG_DIM;
+  s.tattn = s.tg + SS_TAG_HIDDEN;
+  s.tq = s.tattn + (size_t)d->n_heads * d->head_dim;
+  s.tkv = s.tq + (size_t)d->n_heads * d->head_dim;
   s.trace = d->trace;
   s.x_bytes = (int)x_bytes;
   s.grid = grid;
