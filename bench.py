@@ -48,8 +48,9 @@ def linear_bytes(cfg, out_f, in_f):
     return out_f * in_f * 2
 
 
-def kernel_bytes(cfg, T):
-    """algorithmic HBM bytes per decode step of each kernel family at T visible positions"""
+def kernel_bytes(cfg, T, attn_wo=False):
+    """algorithmic HBM bytes per decode step of each kernel family at T visible positions; attn_wo: attention and wo of a
+    layer are one launch (their bytes move from `attn_decode` and `linear` to `attn_wo`)"""
     from denograd_amd import synthetic
     d, V, L = cfg["dim"], cfg["vocab_size"], cfg["n_layers"]
     shp = synthetic.linear_shapes(cfg)
@@ -57,12 +58,16 @@ def kernel_bytes(cfg, T):
     head_q = "int8" if cfg["quantize"] == "int8" else None
     head = (V * d + V * 2) if head_q == "int8" else V * d * 2
     act = 2
-    return {
+    out = {
         "qkv_rope": L * (lb("attention.wq") + lb("attention.wk") + lb("attention.wv") + d * act),
         "attn_decode": synthetic.kv_bytes_per_position(cfg) * T,
         "linear": L * (lb("attention.wo") + lb("feed_forward.w2")) + head + d * act,
         "ffn_gate": L * (lb("feed_forward.w1") + lb("feed_forward.w3") + d * act),
     }
+    if attn_wo:
+        out["attn_wo"] = out.pop("attn_decode") + L * lb("attention.wo")
+        out["linear"] -= L * lb("attention.wo")
+    return out
 
 
 def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=True, blocker_steps=40, per_op_steps=64, fused_step=False):
@@ -147,7 +152,7 @@ def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=Tru
         if m.forward_jit is not None:
             m.forward_jit.reset()
     fam = per_op if fused else kinds
-    kb = kernel_bytes(cfg, llm.start_pos)
+    kb = kernel_bytes(cfg, llm.start_pos, attn_wo="attn_wo" in fam)
     for kname, b_ in kb.items():
         k = fam[kname]
         k["bytes_per_step"] = int(b_)
@@ -164,7 +169,7 @@ def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=Tru
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get((name, "decode_step")),
                 "bytes_per_launch": int(bytes_now), "avg_us_per_launch": round(step_ms * 1e3, 2)}
     else:
-        dom = "linear"   # wo, w2 and the lm_head: the weight-streaming family with the most launches and (with ffn_gate) the most time
+        dom = "linear"   # w2 and the lm_head (and wo, when it is a launch of its own): the weight-streaming family with the most launches
         achieved = fam[dom]["GBps"]
         roof = {"bound": "hbm", "kernel": f"gemv_kernel ({dom})", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get((name, dom)),

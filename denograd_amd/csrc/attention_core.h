@@ -28,6 +28,9 @@ struct AttnArgs {
   // several sequences at the same position (grid z): distance between consecutive sequences, in bytes (q, out, caches)
   // and in elements (counters, partial); zero for a single sequence
   size_t q_bstride = 0, cache_bstride = 0, partial_bstride = 0;
+  // when set, the merged output goes here as tagged words (value | out_tag << 16) for other blocks of the same launch
+  uint32_t *out_tagged = nullptr;
+  uint32_t out_tag = 0;
 };
 
 template <int G> __device__ __forceinline__ float group_sum(float v) {
@@ -282,7 +285,8 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       }
       AT *dst = (AT *)a.out + (size_t)(g * NREP + j) * HD + d;
       const float r = Act<AT>::rn(O * sm.l_sh[j]);  // the cast of the P.V result
-      if constexpr (COHERENT) st_coherent(dst, (AT)r);
+      if (a.out_tagged != nullptr) tw_store(a.out_tagged + (size_t)(g * NREP + j) * HD + d, a.out_tag, r);
+      else if constexpr (COHERENT) st_coherent(dst, (AT)r);
       else *dst = (AT)r;
     }
     if (tid == 0) __hip_atomic_store(&a.counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -1,0 +1,141 @@
+// Decode attention and the wo projection of one layer in ONE launch.
+//
+// As two launches the pair costs a chain of latencies: the attention kernel ends (its last block merges the chunks of a kv
+// head), the wo kernel starts, requests its weights, stages x, and only then computes; wo of a small model is little more
+// than that ramp.  Here every wavefront requests its first wo item (8 KiB of weights) before the attention items run, the
+// blocks that have an attention item run it, and the merged attention row travels to all blocks as tagged words (value |
+// version tag, common.h): the wo part of a block asks for the row until every word carries the tag of this launch, then
+// multiplies with weights that are already in registers.
+//
+// Deadlock freedom: only the wo part waits, and only for the blocks with attention items, which have the lowest block ids
+// and are dispatched first; those never wait for anyone (the last block of a kv head to arrive merges, nobody waits for
+// that).  The wait is bounded all the same and reports through an error word.
+//
+// Reference: models/llama.ts:89-96 (repeat_kv + scaled_dot_product_attention + wo) and :125 (the residual add).
+#include "attention_core.h"
+#include "gemv_core.h"
+
+namespace jsg {
+
+constexpr int AW_THREADS = 256;
+
+template <int KIND, int HD, int NREP>
+__global__ __launch_bounds__(AW_THREADS) void attn_wo_kernel(AttnArgs at, GemvArgs a, int layer) {
+  typedef _Float16 AT;
+  typedef Attn<AT, HD, NREP, AW_THREADS / 64, false> A;
+  typedef Gemv<KIND, AT, EPI_STORE, 2, 4, false> G;
+  extern __shared__ __align__(16) unsigned char smem[];   // the staged input row of wo
+  __shared__ typename A::Smem sm;
+  __shared__ float red[8];
+  __shared__ float lut[16];
+
+  const int pos = at.st[1];
+  // the version of this launch: no other launch that writes the same tagged row has it (another layer, or another
+  // position of the same layer; a model has at least two layers here)
+  const uint32_t tag = tw_tag(pos * 128 + layer);
+  at.out_tag = tag;
+  a.x_tag = tag;
+
+  // this wavefront's first wo item, requested before anything else
+  GemvBuf buf;
+  const int wave = threadIdx.x >> 6, grp = blockIdx.x * (AW_THREADS / 64) + wave;
+  const bool preloaded = grp < G::ngroups(a);
+  if (preloaded) G::load_item(a, buf, grp, 0, 0);
+
+  if (pos >= 0 && pos < at.max_context) {
+    const int T = pos + 1;
+    const int chunk = (T + at.nsplit - 1) / at.nsplit;   // <= ATT_CHUNK_MAX, checked on the host against max_context
+    const int n_active = (T + chunk - 1) / chunk;
+    const int id = blockIdx.x;
+    if (id < at.n_kv_heads * n_active) A::item(at, sm, id % at.n_kv_heads, id / at.n_kv_heads, T, chunk, n_active);
+  } else if (blockIdx.x == 0 && threadIdx.x == 0) {
+    st_coherent(a.err, 1);   // no attention row will come for such a position
+  }
+  __syncthreads();   // the LDS of the attention item is done with
+  G::run(a, (AT *)smem, red, lut, buf, preloaded, 0);
+}
+
+static int aw_nsplit(int max_context) {
+  int by_lds = (max_context + ATT_CHUNK_MAX - 1) / ATT_CHUNK_MAX;
+  int wanted = (max_context + 31) / 32;
+  if (wanted > 64) wanted = 64;
+  return by_lds > wanted ? by_lds : wanted;
+}
+
+template <int KIND, int HD> static int launch_attn_wo(const AttnArgs &at, const GemvArgs &a, int n_rep, int layer, int out_f) {
+  const int ngroups = (out_f + 1) / 2, need = (ngroups + 3) / 4;
+  const int cap = state().cu_count * 4;
+  int blocks = need < cap ? need : cap;
+  const int items = at.n_kv_heads * at.nsplit;
+  if (blocks < items) blocks = items;
+  const size_t lds = (size_t)Gemv<KIND, _Float16, EPI_STORE, 2, 4, false>::x_elems(a.in_f) * sizeof(_Float16);
+#define JSG_REP(N)                                                                                                   \
+  case N:                                                                                                            \
+    JSG_LAUNCH(PROF_ATTN_WO, (attn_wo_kernel<KIND, HD, N>), dim3(blocks), dim3(AW_THREADS), lds, at, a, layer);       \
+    break;
+  switch (n_rep) {
+    JSG_REP(1) JSG_REP(2) JSG_REP(4)
+    default: return fail("jsgrad_hip_attn_wo: n_heads/n_kv_heads = %d is not one of 1,2,4", n_rep);
+  }
+#undef JSG_REP
+  return 0;
+}
+
+}  // namespace jsg
+
+using namespace jsg;
+
+extern "C" {
+
+size_t jsgrad_hip_attn_wo_workspace_bytes(int n_heads, int n_kv_heads, int head_dim) {
+  // [0, 256): chunk counters per kv head; [256, 512): error word; attention partials; the tagged attention row
+  (void)n_kv_heads;
+  return 512 + (size_t)n_heads * 256 * (head_dim + 2) * sizeof(float) + (size_t)n_heads * head_dim * sizeof(uint32_t);
+}
+
+int jsgrad_hip_attn_wo(const void *q, const void *cache_k, const void *cache_v, const int32_t *st, void *workspace, int n_heads, int n_kv_heads,
+                       int head_dim, int max_context, int kind, const void *wo, const void *so, int dim, const void *residual, void *y, int layer) {
+  JSG_READY();
+  JSG_REQUIRE(q && cache_k && cache_v && st && workspace && wo && y, "jsgrad_hip_attn_wo: null pointer argument");
+  JSG_REQUIRE(kind == JSGRAD_W_F16 || kind == JSGRAD_W_I8, "jsgrad_hip_attn_wo: weight kind %d (fp16 and int8 are built)", kind);
+  JSG_REQUIRE(kind == JSGRAD_W_F16 || so, "jsgrad_hip_attn_wo: quantised weight needs a scale");
+  JSG_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_kv_heads <= 64 && n_heads % n_kv_heads == 0, "jsgrad_hip_attn_wo: n_heads %d / n_kv_heads %d", n_heads, n_kv_heads);
+  JSG_REQUIRE(head_dim == 64 || head_dim == 128, "jsgrad_hip_attn_wo: head_dim %d (64 and 128 are built)", head_dim);
+  JSG_REQUIRE(max_context > 0 && max_context <= 64 * ATT_CHUNK_MAX, "jsgrad_hip_attn_wo: max_context %d exceeds %d", max_context, 64 * ATT_CHUNK_MAX);
+  JSG_REQUIRE(layer >= 0 && layer < 128, "jsgrad_hip_attn_wo: layer index %d", layer);
+  const int qdim = n_heads * head_dim;
+  JSG_REQUIRE(dim > 0 && dim % 2 == 0 && qdim % 16 == 0 && (size_t)qdim * 2 <= 64 * 1024, "jsgrad_hip_attn_wo: dim %d / n_heads*head_dim %d", dim, qdim);
+  char *ws = (char *)workspace;
+  AttnArgs at;
+  at.q = q; at.cache_k = cache_k; at.cache_v = cache_v; at.st = st; at.out = nullptr;
+  at.counters = (int *)ws;
+  at.partial = (float *)(ws + 512);
+  at.n_kv_heads = n_kv_heads; at.nsplit = aw_nsplit(max_context); at.max_context = max_context;
+  at.scale = (float)(1.0 / sqrt((double)head_dim));
+  at.out_tagged = (uint32_t *)(ws + 512 + (size_t)n_heads * 256 * (head_dim + 2) * sizeof(float));
+  GemvArgs a = {};
+  a.w0 = wo; a.s0 = so; a.rows0 = dim; a.in_f = qdim; a.x = nullptr; a.norm_w = nullptr; a.eps = 0.0f;
+  a.inv_d = (float)(1.0 / (double)qdim); a.y = y; a.residual = residual;
+  a.x_tagged = at.out_tagged;
+  a.err = (int *)(ws + 256);
+  const int n_rep = n_heads / n_kv_heads;
+#define JSG_KIND(K) \
+  case K: return head_dim == 64 ? launch_attn_wo<K, 64>(at, a, n_rep, layer, dim) : launch_attn_wo<K, 128>(at, a, n_rep, layer, dim);
+  switch (kind) {
+    JSG_KIND(JSGRAD_W_F16)
+    JSG_KIND(JSGRAD_W_I8)
+  }
+#undef JSG_KIND
+  return fail("jsgrad_hip_attn_wo: weight kind %d", kind);
+}
+
+int jsgrad_hip_attn_wo_status(const void *workspace, int *host_out_error) {
+  JSG_READY();
+  JSG_REQUIRE(workspace && host_out_error, "jsgrad_hip_attn_wo_status: null pointer");
+  JSG_REQUIRE(!state().capturing, "jsgrad_hip_attn_wo_status during graph capture");
+  JSG_HIP(hipMemcpyAsync(host_out_error, (const char *)workspace + 256, sizeof(int), hipMemcpyDeviceToHost, state().stream));
+  JSG_HIP(hipStreamSynchronize(state().stream));
+  return 0;
+}
+
+}  // extern "C"

@@ -23,7 +23,7 @@ int fail(const char *fmt, ...);
 int fail_hip(hipError_t e, const char *what);
 
 // per-kernel timing with HIP events on the library stream (off unless jsgrad_hip_profile(1))
-enum { PROF_EMBED = 0, PROF_RMSNORM, PROF_LINEAR, PROF_QKV_ROPE, PROF_ATTN, PROF_FFN_GATE, PROF_ARGMAX, PROF_STEP, PROF_GEMM, PROF_ATTN_PREFILL, PROF_KINDS };
+enum { PROF_EMBED = 0, PROF_RMSNORM, PROF_LINEAR, PROF_QKV_ROPE, PROF_ATTN, PROF_FFN_GATE, PROF_ARGMAX, PROF_STEP, PROF_GEMM, PROF_ATTN_PREFILL, PROF_ATTN_WO, PROF_KINDS };
 // Event pair for the next launch of `kind`, or false when profiling is off (or capturing, or out of slots).  The pair
 // is handed to hipExtLaunchKernelGGL, which stamps it with the dispatch's own begin/end times, so the elapsed time is
 // the kernel alone: no marker packets, no launch latency.
@@ -147,6 +147,30 @@ __device__ __forceinline__ float row8_sum(float v) {
   v += dpp_f<0x4E>(v);
   v += dpp_f<0x141>(v);
   return v;
+}
+
+// ---------------------------------------------------------------- tagged words: data that is its own flag
+// A row that blocks of one launch hand to each other: one 32-bit word per element, the fp16 value below, a version tag
+// above.  A reader asks for the words and takes them once every tag is the one it expects: no flag, and the writer does
+// not have to wait for its stores to be acknowledged before anything.
+__device__ __forceinline__ uint32_t tw_tag(int version) { return (uint32_t)version % 65535u + 1u; }   // never 0: fresh memory matches nothing
+__device__ __forceinline__ void tw_store(uint32_t *p, uint32_t tag, float v) {
+  const _Float16 h = (_Float16)v;
+  st_coherent((int *)p, (int)((tag << 16) | (uint32_t)__builtin_bit_cast(uint16_t, h)));
+}
+// eight tagged words at p -> eight packed halves; ok: all eight carry `tag`
+__device__ __forceinline__ u4_t tw_load8(const uint32_t *p, uint32_t tag, bool &ok) {
+  const JSG_GLOBAL uint64_t *q = as_global<uint64_t>(p);
+  uint64_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) w[i] = __hip_atomic_load(q + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const uint64_t e = ((uint64_t)tag << 16) | ((uint64_t)tag << 48);
+  const uint64_t bad = ((w[0] ^ e) | (w[1] ^ e) | (w[2] ^ e) | (w[3] ^ e)) & 0xffff0000ffff0000ull;
+  ok = ok && bad == 0;
+  u4_t o;
+#pragma unroll
+  for (int i = 0; i < 4; i++) o[i] = (uint32_t)(w[i] & 0xffffu) | ((uint32_t)(w[i] >> 32) << 16);
+  return o;
 }
 
 // ---------------------------------------------------------------- jsgrad's polynomial exp2 / sin

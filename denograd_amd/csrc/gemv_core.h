@@ -29,6 +29,11 @@ struct GemvArgs {
   const int32_t *st;      // device {token, start_pos}
   void *cache_k, *cache_v;
   int head_dim, max_context;
+  // when set, the input row is read from here instead of x: tagged words (fp16 value | x_tag << 16) that other blocks of
+  // the same launch are writing; err: set when the wait for them ran out
+  const uint32_t *x_tagged = nullptr;
+  uint32_t x_tag = 0;
+  int *err = nullptr;
 };
 
 // ---- weight formats: VEC elements per 16-byte load --------------------------------------------
@@ -155,6 +160,18 @@ template <typename AT, bool COHERENT> __device__ __forceinline__ void stage_x(co
   const u4_t *xg = (const u4_t *)a.x;
   u4_t *xl = (u4_t *)xs;
   auto ldx = [&](int c) -> u4_t {
+    if constexpr (sizeof(AT) == 2) {
+      if (a.x_tagged != nullptr) {   // ask until the eight words of the chunk carry the tag of this launch
+        u4_t v;
+        for (int it = 0;; it++) {
+          bool ok = true;
+          v = tw_load8(a.x_tagged + (size_t)c * 8, a.x_tag, ok);
+          if (ok) break;
+          if (it > (1 << 18)) { st_coherent(a.err, 1); break; }
+        }
+        return v;
+      }
+    }
     if constexpr (COHERENT) {
       const uint32_t *p = (const uint32_t *)(xg + c);
       u4_t v;
@@ -166,7 +183,43 @@ template <typename AT, bool COHERENT> __device__ __forceinline__ void stage_x(co
     }
   };
   if (a.norm_w == nullptr) {
-    for (int c = tid; c < nchunks; c += nt) xl[c] = ldx(c);
+    if (sizeof(AT) == 2 && a.x_tagged != nullptr) {
+      // Waiting cheaply first: a block that asked for the whole row over and over would take memory bandwidth from the
+      // blocks that are still producing it.  Eight words spread over the row are watched by one wavefront until they carry
+      // the tag (a hint that the row is about there); what decides is the check of every word below.
+      if (tid < 64) {
+        const int probe = (tid & 7) * (n / 8);
+        for (int it = 0; it < (1 << 18); it++) {
+          const uint32_t w = (uint32_t)ld_coherent((const int *)a.x_tagged + probe);
+          if (__all((w >> 16) == a.x_tag)) break;
+          __builtin_amdgcn_s_sleep(8);
+        }
+      }
+      __syncthreads();
+      // all chunks of a thread are asked for together, again and again until every one carries the tag: one round trip
+      // when the row is there, instead of one per chunk
+      constexpr int NCH = 2;
+      for (int c0 = tid; c0 < nchunks; c0 += NCH * nt) {
+        u4_t v[NCH];
+        for (int it = 0;; it++) {
+          bool ok = true;
+#pragma unroll
+          for (int i = 0; i < NCH; i++) {
+            const int c = c0 + i * nt;
+            v[i] = tw_load8(a.x_tagged + (size_t)(c < nchunks ? c : c0) * 8, a.x_tag, ok);   // past the end: its own first chunk again
+          }
+          if (ok) break;
+          if (it > (1 << 18)) { st_coherent(a.err, 1); break; }
+        }
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+          const int c = c0 + i * nt;
+          if (c < nchunks) xl[c] = v[i];
+        }
+      }
+    } else {
+      for (int c = tid; c < nchunks; c += nt) xl[c] = ldx(c);
+    }
     __syncthreads();
     return;
   }

@@ -40,6 +40,7 @@ class Attention:
         self.wv = linear(dim, self.n_kv_heads * self.head_dim, False)
         self.wo = linear(self.n_heads * self.head_dim, dim, False)
         self.cache_kv: Tensor | None = None
+        self.layer_id: int | None = None   # set by Transformer: which layer of the model this is
 
     def _ensure_cache(self, dtype: str, device: str, bsz: int = 1) -> None:
         # Tensor.zeros([2, bsz, max_context, n_kv_heads, head_dim]) (llama.ts:78-80); created for the batch size of the
@@ -76,6 +77,11 @@ class Attention:
         check(lib.jsgrad_hip_qkv_rope(self.wq.kind, self.wq.weight.ptr, sp(self.wq), self.wk.weight.ptr, sp(self.wk), self.wv.weight.ptr, sp(self.wv),
                                       x.ptr, norm.weight.ptr, norm.eps, freqs_cis.ptr, state.ptr, ctx.q.ptr, ck, cv,
                                       self.dim, self.n_heads, self.n_kv_heads, self.head_dim, self.max_context, act))
+        if ctx.fuse_attn_wo and self.layer_id is not None:
+            # attention and wo as one launch: the wo weights are on their way while the attention items run
+            check(lib.jsgrad_hip_attn_wo(ctx.q.ptr, ck, cv, state.ptr, ctx.attn_wo_ws.ptr, self.n_heads, self.n_kv_heads, self.head_dim, self.max_context,
+                                         self.wo.kind, self.wo.weight.ptr, sp(self.wo), self.dim, x.ptr, ctx.h2.ptr, self.layer_id))
+            return ctx.h2
         check(lib.jsgrad_hip_attn_decode(ctx.q.ptr, ck, cv, state.ptr, ctx.attn.ptr, ctx.workspace.ptr,
                                          self.n_heads, self.n_kv_heads, self.head_dim, self.max_context, act))
         return self.wo.call(ctx.attn, out=ctx.h2, residual=x)
@@ -136,6 +142,14 @@ class _Scratch:
         self.logits = Tensor.empty((vocab,), dtype, device)
         nbytes = ffi.load().jsgrad_hip_attn_workspace_bytes(n_heads, n_kv_heads, head_dim)
         self.workspace = Tensor.zeros((nbytes,), "uint8", device)
+        # attention + wo as one launch (set up by Transformer._prepare when the model qualifies)
+        self.fuse_attn_wo = False
+        self.attn_wo_ws: Tensor | None = None
+
+    def enable_attn_wo(self, n_heads: int, n_kv_heads: int, head_dim: int, device: str) -> None:
+        nbytes = ffi.load().jsgrad_hip_attn_wo_workspace_bytes(n_heads, n_kv_heads, head_dim)
+        self.attn_wo_ws = Tensor.zeros((nbytes,), "uint8", device)
+        self.fuse_attn_wo = True
 
 
 class _RowScratch:
@@ -248,7 +262,7 @@ class TinyJit:
 class Transformer:
     def __init__(self, dim: int, hidden_dim: int, n_heads: int, n_layers: int, norm_eps: float, vocab_size: int, linear=Linear, embedding=Embedding,
                  n_kv_heads: int | None = None, rope_theta: float = 10000, max_context: int = 1024, jit: bool = True, feed_forward=FeedForward, device: str = "HIP",
-                 fused_step: bool = False):
+                 fused_step: bool = False, fuse_attn_wo: bool = True):
         self.dim, self.hidden_dim, self.n_heads, self.vocab_size, self.max_context = dim, hidden_dim, n_heads, vocab_size, max_context
         self.n_kv_heads = n_kv_heads if n_kv_heads is not None else n_heads
         self.rope_theta, self.device = rope_theta, device
@@ -266,8 +280,17 @@ class Transformer:
         self._pos = 0                                                        # host mirror of state[1]
         # False: one launch per fused op (the faster of the two today); True: the whole step as one persistent kernel
         self.fused_step = fused_step
+        self.fuse_attn_wo = fuse_attn_wo   # attention and wo of a layer as one launch, where the model qualifies
         self._fused: _FusedStep | None = None
         self._rows: _RowScratch | None = None
+
+    def attn_wo_error(self) -> int:
+        """1 if a bounded wait inside a fused attention + wo launch ever ran out (its result is then not to be trusted)."""
+        if self._ctx is None or self._ctx.attn_wo_ws is None:
+            return 0
+        e = C.c_int(0)
+        check(ffi.load().jsgrad_hip_attn_wo_status(self._ctx.attn_wo_ws.ptr, C.byref(e)))
+        return e.value
 
     # ---- plumbing
     @property
@@ -282,8 +305,13 @@ class Transformer:
             hd = self.dim // self.n_heads
             self._ctx = _Scratch(self.dim, self.hidden_dim, self.n_heads, self.n_kv_heads, hd, self.vocab_size, self.dtype, self.device)
             self.freqs_cis = precompute_freqs_cis(hd, self.max_context * 2, self.rope_theta, self.dtype, self.device)
-            for layer in self.layers:
+            for i, layer in enumerate(self.layers):
                 layer.attention._ensure_cache(self.dtype, self.device)
+                layer.attention.layer_id = i
+            wo = self.layers[0].attention.wo
+            if (self.fuse_attn_wo and self.dtype == "float16" and wo.kind in (ffi.W_F16, ffi.W_I8) and 2 <= len(self.layers) <= 128 and hd in (64, 128)
+                    and self.n_heads // self.n_kv_heads in (1, 2, 4) and self.max_context <= 64 * 256 and self.n_heads * hd * 2 <= 64 * 1024):
+                self._ctx.enable_attn_wo(self.n_heads, self.n_kv_heads, hd, self.device)
             if self.fused_step:
                 self._fused = _FusedStep(self, self._ctx, self._fused_mode())      # raises NotImplementedError for models it was not built for
         return self._ctx

@@ -85,3 +85,30 @@ def test_fused_step_rejects_what_it_was_not_built_for(mode):
     auto = Llama3.from_config(cfg).load_weights(sd, quantized=True)      # default: falls back to one launch per op
     auto._call(1)
     assert auto.model._fused is None
+
+
+@pytest.mark.parametrize("name", ["tiny-f16", "small-int8", "small-f16-hd128"])
+def test_attention_and_wo_in_one_launch_is_bit_identical_to_two(name):
+    """jsgrad_hip_attn_wo runs the same arithmetic in the same order as jsgrad_hip_attn_decode + jsgrad_hip_linear(wo)."""
+    cfg = dict(CASES[name], max_context=640)
+    sd = quantize_state(cfg, synthetic.random_state_dict(cfg, seed=0, std=0.02))
+    one = Llama3.from_config(cfg).load_weights(sd, quantized=True)
+    two = Llama3.from_config(cfg).load_weights(sd, quantized=True)
+    two.model.fuse_attn_wo = False
+    toks = [int(t) for t in synthetic.random_prompt(cfg, 300, seed=6)]
+    for pos, t in enumerate(toks):
+        ta = one._call(t); one.start_pos += 1
+        tb = two._call(t); two.start_pos += 1
+        assert ta == tb, f"position {pos}"
+        if pos in (0, 1, 31, 32, 33, 255, 256, 299):
+            assert np.array_equal(one.model.logits.numpy(), two.model.logits.numpy()), f"position {pos}"
+    assert one.model._ctx.fuse_attn_wo and not two.model._ctx.fuse_attn_wo
+    assert one.model.attn_wo_error() == 0
+    # graph replay of the fused launch: positions advance on the device
+    p0 = one.start_pos
+    one.model.generate(24)
+    two.model.generate(24)
+    ta, tb = one.model.tokens_out.numpy()[p0:p0 + 24], two.model.tokens_out.numpy()[p0:p0 + 24]
+    assert np.array_equal(ta, tb)
+    assert np.array_equal(one.model.logits.numpy(), two.model.logits.numpy())
+    assert one.model.attn_wo_error() == 0
