@@ -389,12 +389,14 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_gemm_kernel(GemmArgs a) 
       if constexpr (KIND == JSGRAD_W_I8) { const _Float16 sv = sc[row]; wscale[rt][q] = h2_t{sv, sv}; }
     }
   // Step s of this wavefront is k-block ks * SPC + s % SPC of chunk s / SPC: its SPC k-blocks of a chunk are neighbours, so
-  // that the halves of a 128-byte line of a weight row are asked for by one wavefront, back to back.  Byte offset of the step inside a weight row;
-  // past the end: the first k-block again (a few re-reads of bytes that are in L2 keep the number of loads in flight the
-  // same on every path).
+  // that the halves of a 128-byte line of a weight row are asked for by one wavefront, back to back.  Byte offset of the
+  // step inside a weight row.  Past the end the last k-block is asked for again: the refills of the last RS steps keep the
+  // number of loads in flight the same on every path, and a line that was fetched a moment ago costs no HBM traffic (the
+  // first k-block of the row, read at the start, has long left the caches by then: that was 1.2-1.5x the bytes).
   const int nsteps = nchunks * SPC;
   auto woff = [&](int s) -> uint32_t {
-    const int kb = s < nsteps ? (s / SPC) * F::KBC + ks * SPC + s % SPC : ks * SPC;
+    const int sc = s < nsteps ? s : nsteps - 1;
+    const int kb = (sc / SPC) * F::KBC + ks * SPC + sc % SPC;
     return (uint32_t)(kb * 4) * 16u;
   };
 
