@@ -31,7 +31,11 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the `linear` kernel family (average over wo, w2 and the lm_head of one step), from two
 # `rocprofv3 --pmc` runs of `bench.py --traffic-probe` (FETCH_SIZE, then WRITE_SIZE), each scaled by what the counter
 # reads for the 512 MiB copy in the same run (factors 2.000 and 1.000).  Counters cannot be read from inside this process.
-MEASURED_TRAFFIC = {("1B", "linear"): 36.49e6, ("8B-int8", "linear"): 45.72e6, ("1B", "ffn_gate"): 67.31e6, ("8B-int8", "ffn_gate"): 118.3e6}
+# HBM bytes per launch of the dominant kernel family from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised under
+# profiles/ (average over the launches of one step).  "linear" is w2 + lm_head when attention and wo share a launch
+# (the default for fp16 activations), else wo + w2 + lm_head.
+MEASURED_TRAFFIC = {("1B", "linear", True): 62.78e6, ("8B-int8", "linear", True): 73.45e6,
+                    ("1B", "linear", False): 36.49e6, ("8B-int8", "linear", False): 45.72e6}
 
 
 def log(*a):
@@ -166,13 +170,13 @@ def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=Tru
         achieved = bytes_now / (step_ms * 1e-3) / 1e9
         kern = "stream_step_kernel" if m._fused.mode == "stream" else "decode_step_kernel"
         roof = {"bound": "hbm", "kernel": f"{kern} (whole token: embedding, 5 phases x layers, lm_head, argmax)", "achieved": round(achieved, 1),
-                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get((name, "decode_step")),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                 "bytes_per_launch": int(bytes_now), "avg_us_per_launch": round(step_ms * 1e3, 2)}
     else:
         dom = "linear"   # w2 and the lm_head (and wo, when it is a launch of its own): the weight-streaming family with the most launches
         achieved = fam[dom]["GBps"]
         roof = {"bound": "hbm", "kernel": f"gemv_kernel ({dom})", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get((name, dom)),
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get((name, dom, "attn_wo" in fam)),
                 "bytes_per_launch": int(kb[dom] / fam[dom]["launches_per_step"]), "avg_us_per_launch": round(fam[dom]["avg_us_per_launch"], 2)}
     rnd = lambda d: {k: {kk: (round(vv, 3) if isinstance(vv, float) else vv) for kk, vv in v.items()} for k, v in d.items()}
     res = {

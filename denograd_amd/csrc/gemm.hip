@@ -552,12 +552,13 @@ template <int KIND, int EPI, int MB, int RTW> static int launch_skinny(const Gem
   return 0;
 }
 // Few rows: the weight-streaming kernel when K is whole chunks.  Every block reads all of x; with two tiles of 16 weight
-// rows per block that is half as often, taken when the output is wide enough for two tiles per block to still fill the chip.
+// rows per block that is half as often.  Measured on the lm_head (8016 tiles) the two-tile shape is no faster and moves
+// more HBM bytes (1.5x the weights against 1.24x), so it is only taken when pinned.
 template <int KIND, int EPI> static int dispatch_skinny(const GemmArgs &a, int prof_kind, bool *taken) {
   *taken = a.M <= 32 && a.K % SkFmt<KIND>::KC == 0 && a.K / SkFmt<KIND>::KC >= 2 && a.N % 16 == 0 && !getenv("JSG_GEMM_NO_SKINNY");
   if (!*taken) return 0;
   const char *pin = getenv("JSG_GEMM_SKINNY_TILES");     // "1" or "2": tests run small matrices through both
-  const bool two = a.N % 32 == 0 && (pin ? pin[0] == '2' : a.N / 32 >= 768);
+  const bool two = a.N % 32 == 0 && pin && pin[0] == '2';
   if (a.M <= 16) return two ? launch_skinny<KIND, EPI, 1, 2>(a, prof_kind) : launch_skinny<KIND, EPI, 1, 1>(a, prof_kind);
   return two ? launch_skinny<KIND, EPI, 2, 2>(a, prof_kind) : launch_skinny<KIND, EPI, 2, 1>(a, prof_kind);
 }
