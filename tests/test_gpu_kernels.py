@@ -261,7 +261,8 @@ def attn_oracle(q, K, V, H, KV, hd, T, act16):
 
 
 @pytest.mark.parametrize("dt,H,KV,hd,ctx", [("float32", 4, 2, 64, 64), ("float16", 32, 8, 64, 1024), ("float16", 24, 8, 128, 600), ("float16", 8, 8, 128, 300),
-                                             ("float16", 8, 1, 64, 2100), ("float32", 6, 2, 128, 96)])
+                                             ("float16", 8, 1, 64, 2100), ("float32", 6, 2, 128, 96),
+                                             ("float16", 8, 2, 128, 4096)])   # 64-row chunks: more iterations than the rows requested up front
 def test_attention_decode(hip, dt, H, KV, hd, ctx):
     """GQA decode attention over the cache for several T, including T=1, chunk boundaries and the full cache;
     repeated launches share one workspace (the merging block must leave the counters at zero)."""
@@ -280,3 +281,37 @@ def test_attention_decode(hip, dt, H, KV, hd, ctx):
         assert np.max(np.abs(f32(out) - ref)) <= tol * max(1.0, np.abs(ref).max()), f"T={T}"
         assert np.mean(np.abs(f32(out) - ref) <= np.abs(ref) * (2.0 ** -8 if act16 else 2.0 ** -16) + 2e-4) > 0.99, f"T={T}"
     assert np.all(ws.numpy()[:256] == 0)
+
+
+@pytest.mark.parametrize("kind,H,KV,hd,ctx", [("f16", 32, 8, 64, 1024), ("i8", 8, 2, 128, 4096), ("f16", 4, 4, 64, 96)])
+def test_attention_and_wo_in_one_launch(hip, kind, H, KV, hd, ctx):
+    """jsgrad_hip_attn_wo == jsgrad_hip_attn_decode followed by jsgrad_hip_linear(wo, residual), bit for bit, for several T,
+    two layers sharing one workspace (the version tag tells their rows apart), and no bounded wait ever running out."""
+    dim, qdim = 256, H * hd
+    K = (RNG.standard_normal((ctx, KV, hd)) * 0.7).astype(np.float16)
+    V = RNG.standard_normal((ctx, KV, hd)).astype(np.float16)
+    q = (RNG.standard_normal(qdim) * 0.7).astype(np.float16)
+    res = RNG.standard_normal(dim).astype(np.float16)
+    w = (RNG.standard_normal((dim, qdim)) * 0.05).astype(np.float32)
+    if kind == "i8":
+        wq, sc = orc.int8_quantize(w)
+        tw, ts, code = Tensor(wq), Tensor(sc), ffi.W_I8
+    else:
+        tw, ts, code = Tensor(w.astype(np.float16)), None, ffi.W_F16
+    tK, tV, tq, tres = Tensor(K), Tensor(V), Tensor(q), Tensor(res)
+    attn, y_two, y_one = Tensor.empty((qdim,), "float16"), Tensor.empty((dim,), "float16"), Tensor.empty((dim,), "float16")
+    ws2 = Tensor.zeros((hip.jsgrad_hip_attn_workspace_bytes(H, KV, hd),), "uint8")
+    ws1 = Tensor.zeros((hip.jsgrad_hip_attn_wo_workspace_bytes(H, KV, hd),), "uint8")
+    sp_ = ts.ptr if ts is not None else None
+    for T in sorted(t for t in {1, 2, 33, 65, ctx // 2 + 1, ctx} if t <= ctx):
+        st = Tensor(np.int32([0, T - 1]))
+        check(hip.jsgrad_hip_attn_decode(tq.ptr, tK.ptr, tV.ptr, st.ptr, attn.ptr, ws2.ptr, H, KV, hd, ctx, ffi.F16))
+        check(hip.jsgrad_hip_linear(code, tw.ptr, sp_, dim, qdim, attn.ptr, y_two.ptr, None, 0.0, tres.ptr, ffi.F16))
+        for layer in (0, 1):
+            check(hip.jsgrad_hip_memset(y_one.ptr, 0, y_one.nbytes))
+            check(hip.jsgrad_hip_attn_wo(tq.ptr, tK.ptr, tV.ptr, st.ptr, ws1.ptr, H, KV, hd, ctx, code, tw.ptr, sp_, dim, tres.ptr, y_one.ptr, layer))
+            assert np.array_equal(y_one.numpy(), y_two.numpy()), f"T={T} layer={layer}"
+    e = C.c_int(0)
+    check(hip.jsgrad_hip_attn_wo_status(ws1.ptr, C.byref(e)))
+    assert e.value == 0
+    assert np.all(ws1.numpy()[:256] == 0)      # the chunk counters are left at zero
