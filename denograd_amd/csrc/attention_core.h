@@ -114,7 +114,22 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       const int t = t0 + (wave + i * NW) * RPI + grp;
       if (t < t1) score_row(kpre[i], t);
     }
-    for (int t = t0 + (wave + NPRE * NW) * RPI + grp; t < t1; t += NW * RPI) score_row(*(const u4_t *)(kbase + (size_t)t * row_stride), t);
+    // longer chunks (several sequences per launch, long contexts): the remaining rows in batches of NBATCH requests, so that
+    // an iteration does not wait a round trip of its own
+    constexpr int NBATCH = 8;
+    for (int tb = t0 + (wave + NPRE * NW) * RPI + grp; tb < t1; tb += NBATCH * NW * RPI) {
+      u4_t raw[NBATCH];
+#pragma unroll
+      for (int i = 0; i < NBATCH; i++) {
+        const int t = tb + i * NW * RPI;
+        raw[i] = *(const u4_t *)(kbase + (size_t)(t < t1 ? t : t1 - 1) * row_stride);
+      }
+#pragma unroll
+      for (int i = 0; i < NBATCH; i++) {
+        const int t = tb + i * NW * RPI;
+        if (t < t1) score_row(raw[i], t);
+      }
+    }
     __syncthreads();
     // chunk maximum per head
     {
@@ -191,7 +206,19 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       const int t = t0 + (wave + i * NW) * RPI + grp;
       if (t < t1) pv_row(vpre[i], t);
     }
-    for (int t = t0 + (wave + NPRE * NW) * RPI + grp; t < t1; t += NW * RPI) pv_row(*(const u4_t *)(vbase + (size_t)t * row_stride), t);
+    for (int tb = t0 + (wave + NPRE * NW) * RPI + grp; tb < t1; tb += NBATCH * NW * RPI) {
+      u4_t raw[NBATCH];
+#pragma unroll
+      for (int i = 0; i < NBATCH; i++) {
+        const int t = tb + i * NW * RPI;
+        raw[i] = *(const u4_t *)(vbase + (size_t)(t < t1 ? t : t1 - 1) * row_stride);
+      }
+#pragma unroll
+      for (int i = 0; i < NBATCH; i++) {
+        const int t = tb + i * NW * RPI;
+        if (t < t1) pv_row(raw[i], t);
+      }
+    }
     // lanes with the same `sub` hold different rows: fold the RPI groups of the wavefront together
 #pragma unroll
     for (int j = 0; j < NREP; j++)
