@@ -74,6 +74,52 @@ def kernel_bytes(cfg, T, attn_wo=False):
     return out
 
 
+def read_only_launches(lib, cfg, T, attn_wo, reps=12):
+    """Time jsgrad_hip_read_probe at the byte count of every weight-streaming launch of one decode step (cold data: the
+    source window moves through 1 GiB).  Returns ms per step per kernel family, their sum, and the per-size table."""
+    from denograd_amd import ffi, synthetic
+    from denograd_amd.ffi import check
+    from denograd_amd.tensor import Tensor
+
+    L, d, V = cfg["n_layers"], cfg["dim"], cfg["vocab_size"]
+    shp = synthetic.linear_shapes(cfg)
+    lb = lambda name: linear_bytes(cfg, *shp[name])
+    head = (V * d + V * 2) if cfg["quantize"] == "int8" else V * d * 2
+    kv = synthetic.kv_bytes_per_position(cfg) * T // L
+    launches = {   # family -> [(count per step, bytes)]
+        "qkv_rope": [(L, lb("attention.wq") + lb("attention.wk") + lb("attention.wv"))],
+        "ffn_gate": [(L, lb("feed_forward.w1") + lb("feed_forward.w3"))],
+        "linear": [(L, lb("feed_forward.w2")), (1, head)],
+    }
+    if attn_wo:
+        launches["attn_wo"] = [(L, lb("attention.wo") + kv)]
+    else:
+        launches["linear"].append((L, lb("attention.wo")))
+        launches["attn_decode"] = [(L, kv)]
+    span = 1 << 30
+    src, sink = Tensor.empty((span,), "uint8"), Tensor.zeros((4,), "uint8")
+    check(lib.jsgrad_hip_memset(src.ptr, 1, span))
+    kid = ffi.PROF_KINDS["read_probe"]
+    cache, off = {}, 0
+
+    def probe(nbytes):
+        nonlocal off
+        nbytes = max(16, nbytes // 16 * 16)
+        if nbytes not in cache:
+            check(lib.jsgrad_hip_profile(1))
+            for _ in range(reps + 2):
+                off = (off + nbytes + (64 << 20)) % (span - nbytes) // 256 * 256
+                check(lib.jsgrad_hip_read_probe(src.ptr + off, nbytes, sink.ptr))
+            n, tot = C.c_int(), C.c_double()
+            check(lib.jsgrad_hip_profile_read(kid, C.byref(n), C.byref(tot)))
+            check(lib.jsgrad_hip_profile(0))
+            cache[nbytes] = tot.value / n.value
+        return cache[nbytes]
+
+    fams = {k: sum(c * probe(b) for c, b in v) for k, v in launches.items()}
+    return {"families": fams, "step_ms": sum(fams.values()), "sizes_us": {str(b): round(1e3 * t, 2) for b, t in sorted(cache.items())}}
+
+
 def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=True, blocker_steps=40, per_op_steps=64, fused_step=False):
     from denograd_amd import ffi, synthetic
     from denograd_amd.ffi import check
@@ -163,6 +209,12 @@ def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=Tru
         k["avg_us_per_launch"] = 1e3 * k["ms_per_step"] / k["launches_per_step"]
         k["GBps"] = b_ / (k["ms_per_step"] * 1e-3) / 1e9
     bytes_tok = synthetic.weight_bytes_per_token(cfg) + synthetic.kv_bytes_per_position(cfg) * t_avg
+    # The measuring stick: a launch that only reads as many bytes as each weight-streaming launch of the step moves (cold
+    # data, same event timing).  What the step would take if its launches did nothing but read.
+    read_only = read_only_launches(lib, cfg, llm.start_pos, "attn_wo" in fam)
+    for kname, r in read_only["families"].items():
+        if kname in fam:
+            fam[kname]["read_only_ms_per_step"] = r
     if fused:
         # one launch = one token: the step kernel is the dominant (only) kernel
         step_ms = kinds["decode_step"]["ms_per_step"]
@@ -177,13 +229,16 @@ def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=Tru
         achieved = fam[dom]["GBps"]
         roof = {"bound": "hbm", "kernel": f"gemv_kernel ({dom})", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get((name, dom, "attn_wo" in fam)),
-                "bytes_per_launch": int(kb[dom] / fam[dom]["launches_per_step"]), "avg_us_per_launch": round(fam[dom]["avg_us_per_launch"], 2)}
+                "bytes_per_launch": int(kb[dom] / fam[dom]["launches_per_step"]), "avg_us_per_launch": round(fam[dom]["avg_us_per_launch"], 2),
+                # the same launches as read-only kernels of the same sizes: the rate a launch of this size can reach at all
+                "read_only_GBps": round(kb[dom] / (read_only["families"][dom] * 1e-3) / 1e9, 1)}
     rnd = lambda d: {k: {kk: (round(vv, 3) if isinstance(vv, float) else vv) for kk, vv in v.items()} for k, v in d.items()}
     res = {
         "name": name, "tok_s": tok_s, "ms_per_step": 1e3 * wall / steps, "event_ms_per_step": ms.value / steps,
         "roofline": roof,
         "step_roofline": {"bytes_per_token": int(bytes_tok), "achieved": round(bytes_tok * tok_s / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": round(bytes_tok * tok_s / 1e9 / HBM_PEAK_GBS, 4)},
+                          "frac": round(bytes_tok * tok_s / 1e9 / HBM_PEAK_GBS, 4),
+                          "read_only_launches_ms": round(read_only["step_ms"], 4), "read_only_sizes_us": read_only["sizes_us"]},
         "kernels": rnd(kinds),
         "config": {"workload": f"Llama-3 decode bs=1, {name}-shaped random init ({cfg['quantize']}), {prompt_len}-token prompt, {steps} greedy tokens",
                    "prompt": prompt_len, "decode": steps, "avg_visible_positions": t_avg, "max_context": ctx,

@@ -22,7 +22,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_decode_kernel(AttnArgs a) {
   const int pos = a.st[1];
   if (pos < 0 || pos >= a.max_context) return;
   const int T = pos + 1;
-  const int chunk = (T + a.nsplit - 1) / a.nsplit;  // <= ATT_CHUNK_MAX, checked on the host against max_context
+  const int chunk = att_chunk_rows(T, a.nsplit);  // <= ATT_CHUNK_MAX, checked on the host against max_context
   const int n_active = (T + chunk - 1) / chunk;
   if (split >= n_active) return;
   A::item(a, sm, g, split, T, chunk, n_active);

@@ -16,6 +16,15 @@
 namespace jsg {
 
 constexpr int ATT_CHUNK_MAX = 256;  // positions per item held in LDS; also the most chunks the merge can index
+constexpr int ATT_CHUNK_MIN = 32;   // a block covers this many rows with the requests it sends before anything else (one
+                                    // iteration at head_dim 64, two at 128), so shorter chunks finish no sooner and only
+                                    // add partial results for the merge to fetch
+
+// rows per chunk when T visible positions are cut into at most nsplit chunks
+__host__ __device__ __forceinline__ int att_chunk_rows(int T, int nsplit) {
+  const int c = (T + nsplit - 1) / nsplit;
+  return c < ATT_CHUNK_MIN ? ATT_CHUNK_MIN : c;
+}
 
 struct AttnArgs {
   const void *q, *cache_k, *cache_v;

@@ -44,7 +44,7 @@ __global__ __launch_bounds__(AW_THREADS) void attn_wo_kernel(AttnArgs at, GemvAr
 
   if (pos >= 0 && pos < at.max_context) {
     const int T = pos + 1;
-    const int chunk = (T + at.nsplit - 1) / at.nsplit;   // <= ATT_CHUNK_MAX, checked on the host against max_context
+    const int chunk = att_chunk_rows(T, at.nsplit);   // <= ATT_CHUNK_MAX, checked on the host against max_context
     const int n_active = (T + chunk - 1) / chunk;
     const int id = blockIdx.x;
     if (id < at.n_kv_heads * n_active) A::item(at, sm, id % at.n_kv_heads, id / at.n_kv_heads, T, chunk, n_active);
@@ -114,9 +114,10 @@ int jsgrad_hip_attn_wo(const void *q, const void *cache_k, const void *cache_v, 
   at.scale = (float)(1.0 / sqrt((double)head_dim));
   at.out_tagged = (uint32_t *)(ws + 512 + (size_t)n_heads * 256 * (head_dim + 2) * sizeof(float));
   GemvArgs a = {};
-  a.w0 = wo; a.s0 = so; a.rows0 = dim; a.in_f = qdim; a.x = nullptr; a.norm_w = nullptr; a.eps = 0.0f;
+  a.w0 = wo; a.s0 = so; a.rows0 = dim; a.in_f = qdim; a.norm_w = nullptr; a.eps = 0.0f;
   a.inv_d = (float)(1.0 / (double)qdim); a.y = y; a.residual = residual;
   a.x_tagged = at.out_tagged;
+  a.x = at.out_tagged;   // never read as the input; a readable address for the load that stands in for a missing residual
   a.err = (int *)(ws + 256);
   const int n_rep = n_heads / n_kv_heads;
 #define JSG_KIND(K) \

@@ -259,7 +259,33 @@ template <typename T> __global__ void randn_kernel(T *out, size_t n, uint64_t se
 
 using namespace jsg;
 
+// ---------------------------------------------------------------- read probe
+// Reads n 16-byte vectors and keeps nothing: every thread has eight streaming loads in flight, grid-stride.  The compare
+// at the end keeps the loads alive (a match only writes a word nobody reads).
+__global__ __launch_bounds__(256) void read_probe_kernel(const u4_t *p, size_t n, uint32_t *sink) {
+  u4_t acc = {0, 0, 0, 0};
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += 8 * stride) {
+    u4_t v[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      const size_t k = i + u * stride;
+      v[u] = ldg_stream16(p + (k < n ? k : i));
+    }
+#pragma unroll
+    for (int u = 0; u < 8; u++) acc ^= v[u];
+  }
+  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u) *sink = 1;
+}
+
 extern "C" {
+
+int jsgrad_hip_read_probe(const void *src, size_t nbytes, void *sink) {
+  JSG_READY();
+  JSG_REQUIRE(src && sink && nbytes >= 16 && nbytes % 16 == 0 && (uintptr_t)src % 16 == 0, "jsgrad_hip_read_probe: bad argument");
+  JSG_LAUNCH(PROF_READ, read_probe_kernel, dim3(state().cu_count * 2), dim3(256), 0, (const u4_t *)src, nbytes / 16, (uint32_t *)sink);
+  return 0;
+}
 
 int jsgrad_hip_memset(void *dst, int byte, size_t nbytes) {
   JSG_READY();

@@ -79,9 +79,15 @@ int jsgrad_hip_event_destroy(void *event);
 /* Per-kernel statistics (DEBUG>=2 of engine/realize.ts:168-178; ProfileRangeEvent, runtime/allocator.ts:147-151):
  * while enabled, every Llama kernel launched outside a graph capture is bracketed by an event pair.  `read` waits
  * for the stream and returns launch count and summed milliseconds of one kind since profiling was enabled. */
-enum { JSGRAD_PROF_EMBED = 0, JSGRAD_PROF_RMSNORM, JSGRAD_PROF_LINEAR, JSGRAD_PROF_QKV_ROPE, JSGRAD_PROF_ATTN, JSGRAD_PROF_FFN_GATE, JSGRAD_PROF_ARGMAX, JSGRAD_PROF_STEP, JSGRAD_PROF_GEMM, JSGRAD_PROF_ATTN_PREFILL };
+enum { JSGRAD_PROF_EMBED = 0, JSGRAD_PROF_RMSNORM, JSGRAD_PROF_LINEAR, JSGRAD_PROF_QKV_ROPE, JSGRAD_PROF_ATTN, JSGRAD_PROF_FFN_GATE, JSGRAD_PROF_ARGMAX, JSGRAD_PROF_STEP, JSGRAD_PROF_GEMM, JSGRAD_PROF_ATTN_PREFILL, JSGRAD_PROF_ATTN_WO, JSGRAD_PROF_READ };
 int jsgrad_hip_profile(int enable);
 int jsgrad_hip_profile_read(int kind, int *host_out_count, double *host_out_total_ms);
+
+/* A measuring stick, with no counterpart in the reference: one launch that reads nbytes (a multiple of 16) of device memory
+ * at src through registers and keeps nothing (two blocks per CU, eight 16-byte streaming loads in flight per thread).  Its
+ * duration (kind JSGRAD_PROF_READ of the statistics above) is what a launch that only had to read that many bytes takes
+ * on this device: the ceiling for a one-launch linear layer of that size.  sink: 4 writable bytes of device memory. */
+int jsgrad_hip_read_probe(const void *src, size_t nbytes, void *sink);
 
 /* TinyJit capture / replay as a device graph (engine/jit.ts:14-69 apply_graph_to_jit, :71 GraphRunner,
  * `Compiled.graph` allocator.ts:176): everything queued between begin and end becomes one HIP graph. */

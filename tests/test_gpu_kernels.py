@@ -311,6 +311,12 @@ def test_attention_and_wo_in_one_launch(hip, kind, H, KV, hd, ctx):
             check(hip.jsgrad_hip_memset(y_one.ptr, 0, y_one.nbytes))
             check(hip.jsgrad_hip_attn_wo(tq.ptr, tK.ptr, tV.ptr, st.ptr, ws1.ptr, H, KV, hd, ctx, code, tw.ptr, sp_, dim, tres.ptr, y_one.ptr, layer))
             assert np.array_equal(y_one.numpy(), y_two.numpy()), f"T={T} layer={layer}"
+    # without a residual (T is the last one of the loop; layer 0 again, another position would do as well)
+    st = Tensor(np.int32([0, max(ctx // 4, 1) - 1]))
+    check(hip.jsgrad_hip_attn_decode(tq.ptr, tK.ptr, tV.ptr, st.ptr, attn.ptr, ws2.ptr, H, KV, hd, ctx, ffi.F16))
+    check(hip.jsgrad_hip_linear(code, tw.ptr, sp_, dim, qdim, attn.ptr, y_two.ptr, None, 0.0, None, ffi.F16))
+    check(hip.jsgrad_hip_attn_wo(tq.ptr, tK.ptr, tV.ptr, st.ptr, ws1.ptr, H, KV, hd, ctx, code, tw.ptr, sp_, dim, None, y_one.ptr, 0))
+    assert np.array_equal(y_one.numpy(), y_two.numpy()), "no residual"
     e = C.c_int(0)
     check(hip.jsgrad_hip_attn_wo_status(ws1.ptr, C.byref(e)))
     assert e.value == 0
