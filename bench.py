@@ -387,6 +387,45 @@ def traffic_probe(name, batch=1):
         check(lib.jsgrad_hip_sync())
 
 
+def run_formats(reps=5):
+    """Load-time kernels of the checkpoint path, each on one lm_head-sized tensor (128256 x 2048 elements): GGML Q6_K ->
+    float32, bfloat16 -> float16, and the q_proj row permutation.  HBM-bound byte work: bytes read + written per second."""
+    from denograd_amd import ffi
+    from denograd_amd.ffi import check
+    from denograd_amd.tensor import Tensor
+
+    lib = ffi.load()
+    rows, cols = 128256, 2048
+    n = rows * cols
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    check(lib.jsgrad_hip_event_create(C.byref(e0)))
+    check(lib.jsgrad_hip_event_create(C.byref(e1)))
+
+    def timed(fn, nbytes):
+        fn()
+        check(lib.jsgrad_hip_event_record(e0))
+        for _ in range(reps):
+            fn()
+        check(lib.jsgrad_hip_event_record(e1))
+        ms = C.c_float()
+        check(lib.jsgrad_hip_event_elapsed_ms(e0, e1, C.byref(ms)))
+        us = 1e3 * ms.value / reps
+        return {"bytes": int(nbytes), "us": round(us, 1), "GBps": round(nbytes / us / 1e3, 1), "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+
+    out = {}
+    nb = lib.jsgrad_hip_ggml_nbytes(14, n)
+    blocks = Tensor.empty((nb,), "uint8")
+    check(lib.jsgrad_hip_memset(blocks.ptr, 0x11, nb))
+    f32 = Tensor.empty((n,), "float32")
+    out["ggml_q6k_dequant"] = timed(lambda: check(lib.jsgrad_hip_ggml_dequant(14, blocks.ptr, n, f32.ptr)), nb + 4 * n)
+    h = Tensor.empty((rows, cols), "float16")
+    out["bf16_to_f16"] = timed(lambda: check(lib.jsgrad_hip_cast(f32.ptr, ffi.BF16, h.ptr, ffi.F16, n)), 4 * n)
+    h2 = Tensor.empty((rows, cols), "float16")
+    out["hf_permute"] = timed(lambda: check(lib.jsgrad_hip_hf_permute(h.ptr, h2.ptr, rows, cols * 2, rows // 64)), 4 * n)
+    out["tensor"] = f"{rows} x {cols} elements"
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -445,6 +484,7 @@ def main():
                             "step_roofline": secondary["step_roofline"], "kernels": secondary["kernels"], "per_op_path": secondary.get("per_op_path")}
     if args.batched:
         out["batched"] = run_batched(args.batched, args.batch, args.batch_prompt, args.batch_steps)
+    out["formats"] = run_formats()
     print(json.dumps(out), flush=True)
 
 

@@ -20,7 +20,9 @@ from . import ffi
 from .ffi import HipError, check
 
 DTYPES = {"float32": (np.float32, ffi.F32), "float16": (np.float16, ffi.F16), "int8": (np.int8, None), "uint8": (np.uint8, None),
-          "int32": (np.int32, None)}
+          "int32": (np.int32, None), "int16": (np.int16, None),
+          # bfloat16 has no numpy type: the 16 bits travel as uint16 and only jsgrad_hip_cast ever interprets them
+          "bfloat16": (np.uint16, ffi.BF16)}
 
 
 def itemsize(dtype: str) -> int:

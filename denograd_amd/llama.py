@@ -470,3 +470,66 @@ class Transformer:
             raise ValueError(f"{n_steps} steps from position {self._pos} overrun the KV cache of {self.max_context} positions")
         for _ in range(n_steps):
             self.forward_jit.call()
+
+
+# *** helpers (llama.ts:222-279) ***
+
+def convert_from_huggingface(weights: dict, n_layers: int, n_heads: int, n_kv_heads: int, permute_layers: bool = True, device: str = "HIP") -> dict[str, Tensor]:
+    """models/llama.ts:224-253: Hugging Face key names -> the model's, and q_proj / k_proj rows permuted from the
+    rotate-half layout to the interleaved pairs that apply_rotary_emb rotates (on the device, jsgrad_hip_hf_permute).
+    `weights`: host arrays (as safe_load returns them) or device Tensors; the result holds device Tensors.
+
+    The reference's key map writes `{l}` instead of `${l}` in the entries for `post_attention_layernorm` and the biases
+    (llama.ts:234-235), so there a real checkpoint's ffn_norm weights land under the key `undefined`; here they are mapped
+    to `layers.N.ffn_norm.weight`, as every other line of the map (and the function it was translated from) does."""
+    from .state import to_device
+    lib = ffi.load()
+    keymap = {"model.embed_tokens.weight": "tok_embeddings.weight", "model.norm.weight": "norm.weight", "lm_head.weight": "output.weight"}
+    for l in range(n_layers):
+        keymap[f"model.layers.{l}.input_layernorm.weight"] = f"layers.{l}.attention_norm.weight"
+        keymap[f"model.layers.{l}.post_attention_layernorm.weight"] = f"layers.{l}.ffn_norm.weight"
+        for x in "qkvo":
+            keymap[f"model.layers.{l}.self_attn.{x}_proj.weight"] = f"layers.{l}.attention.w{x}.weight"
+            keymap[f"model.layers.{l}.self_attn.{x}_proj.bias"] = f"layers.{l}.attention.w{x}.bias"
+        for x, y in (("gate", "1"), ("down", "2"), ("up", "3")):
+            keymap[f"model.layers.{l}.mlp.{x}_proj.weight"] = f"layers.{l}.feed_forward.w{y}.weight"
+    sd: dict[str, Tensor] = {}
+    for k, v in weights.items():
+        if ".rotary_emb." in k:
+            continue
+        if k not in keymap:
+            raise KeyError(f"{k} is not a key of a Hugging Face Llama checkpoint with {n_layers} layers")
+        t = to_device(v, device)
+        if "model.layers" in k and permute_layers and ("q_proj" in k or "k_proj" in k):
+            heads = n_heads if "q_proj" in k else n_kv_heads
+            if t.ndim != 2:
+                raise ValueError(f"{k}: expected a matrix, got shape {t.shape}")
+            out = Tensor.empty(t.shape, t.dtype, device)
+            check(lib.jsgrad_hip_hf_permute(t.ptr, out.ptr, t.shape[0], t.nbytes // t.shape[0], heads))
+            t = out
+        sd[keymap[k]] = t
+    return sd
+
+
+def convert_from_gguf(weights: dict[str, Tensor], n_layers: int) -> dict[str, Tensor]:
+    """models/llama.ts:255-270: GGUF tensor names -> the model's; the lm_head is the embedding table."""
+    keymap = {"token_embd.weight": "tok_embeddings.weight", "output_norm.weight": "norm.weight", "rope_freqs.weight": "rope_freqs.weight"}
+    for l in range(n_layers):
+        keymap[f"blk.{l}.attn_norm.weight"] = f"layers.{l}.attention_norm.weight"
+        keymap[f"blk.{l}.ffn_norm.weight"] = f"layers.{l}.ffn_norm.weight"
+        keymap[f"blk.{l}.attn_output.weight"] = f"layers.{l}.attention.wo.weight"
+        for x in "qkv":
+            keymap[f"blk.{l}.attn_{x}.weight"] = f"layers.{l}.attention.w{x}.weight"
+        for x, y in (("gate", "1"), ("down", "2"), ("up", "3")):
+            keymap[f"blk.{l}.ffn_{x}.weight"] = f"layers.{l}.feed_forward.w{y}.weight"
+    for k in weights:
+        if k not in keymap:
+            raise KeyError(f"{k} is not a tensor of a GGUF Llama checkpoint with {n_layers} layers")
+    sd = {keymap[k]: v for k, v in weights.items()}
+    sd["output.weight"] = weights["token_embd.weight"]
+    return sd
+
+
+def fix_bf16(weights: dict[str, Tensor]) -> dict[str, Tensor]:
+    """models/llama.ts:272-279: bfloat16 tensors become float16 by way of float32."""
+    return {k: (v.cast("float16") if v.dtype == "bfloat16" else v) for k, v in weights.items()}

@@ -6,10 +6,12 @@ row; two 4-bit codes per byte + one fp16 scale per 64 elements) and its quantise
 dequantising GEMV.  Llama3 drives a Transformer the way the reference does: token-serial prefill, greedy
 decode, per-token `.item()`; `generate` is the free-running variant that keeps the token on the device.
 Downloading checkpoints and the tokenizer are out of scope here: a model is built from a state dict
-(host arrays, a .safetensors file, or seeded random-init weights made on the device).
+(host arrays), a checkpoint file (.safetensors in the model's or in Hugging Face names, a .safetensors.index.json, a
+.gguf with F32 / F16 / Q4_0 / Q4_1 / Q8_0 / Q6_K tensors), or seeded random-init weights made on the device.
 """
 from __future__ import annotations
 
+import os
 import time
 
 import numpy as np
@@ -17,9 +19,9 @@ import numpy as np
 from . import ffi, synthetic
 from .device import DTYPES
 from .ffi import check
-from .llama import Transformer
+from .llama import Transformer, convert_from_gguf, convert_from_huggingface, fix_bf16
 from .nn import Embedding, Linear, act_code
-from .state import load_state_dict, safe_load
+from .state import gguf_load, load_state_dict, safe_load, to_device
 from .tensor import Tensor
 
 
@@ -115,6 +117,9 @@ class Llama3:
 
     def __init__(self, size: str | None = None, quantize: str | None = None, device: str = "HIP", max_context: int = 8192, temperature: float = 0.0,
                  top_k: int = 0, top_p: float = 0.0, alpha_f: float = 0.0, alpha_p: float = 0.0, args: dict | None = None, fused_step: bool = False):
+        # quantize: None (tensors as loaded), "float16" (every tensor cast to float16, llama3.ts:234), "int8", "nf4"
+        self.cast_float16 = quantize == "float16"
+        quantize = None if quantize == "float16" else quantize
         self.size, self.quantize, self.device, self.max_context = size, quantize, device, max_context
         self.temperature, self.top_k, self.top_p, self.alpha_f, self.alpha_p = temperature, top_k, top_p, alpha_f, alpha_p
         self.linear, self.embedding, self.quantize_embeds = _classes(quantize)
@@ -148,8 +153,38 @@ class Llama3:
         load_state_dict(self.model, dev, strict=False)
         return self
 
+    def _load(self, fn: str) -> dict:
+        """llama3.ts:201-213: a `.safetensors` file, a `.safetensors.index.json` that names several, or a `.gguf` file."""
+        if fn.endswith(".index.json"):
+            import json
+            with open(fn) as f:
+                weight_map = json.load(f)["weight_map"]
+            base = os.path.dirname(fn)
+            parts = {n: self._load(os.path.join(base, n)) for n in sorted(set(weight_map.values()))}
+            return {k: parts[n][k] for k, n in weight_map.items()}
+        if fn.endswith(".gguf"):
+            return gguf_load(fn, self.device)[1]
+        if fn.endswith(".safetensors"):
+            return safe_load(fn)
+        raise ValueError("invalid file")
+
     def load(self, fn: str) -> "Llama3":
-        return self.load_weights(safe_load(fn))
+        """llama3.ts:215-255 from the file on: read, rename (Hugging Face or GGUF names, told apart by their embedding
+        key), bfloat16 -> float16, then `quantize == float16` casts every tensor to float16 and the quantised modes
+        quantise; tensors of a file already in the model's own names and dtype load as they are."""
+        p = self.params
+        weights = self._load(fn)
+        if "model.embed_tokens.weight" in weights:
+            weights = convert_from_huggingface(weights, p["n_layers"], p["n_heads"], p.get("n_kv_heads") or p["n_heads"], device=self.device)
+        elif "token_embd.weight" in weights:
+            weights = convert_from_gguf(weights, p["n_layers"])
+            weights.pop("rope_freqs.weight", None)   # carried through by the reference's map, not a tensor of the model
+        weights = fix_bf16({k: to_device(v, self.device) for k, v in weights.items()})
+        if self.cast_float16 or self.quantize is not None:
+            # the quantisers start from float16 (`v.cast(scale_dtype)`, llama3.ts:42,103); the tensors they leave alone (norms,
+            # an unquantised embedding) are cast as well, so that the model has one activation dtype on this device
+            weights = {k: (v.cast("float16") if v.dtype == "float32" else v) for k, v in weights.items()}
+        return self.load_weights(weights)
 
     def random_init(self, seed: int = 0, std: float = 0.02, tied: bool = True) -> "Llama3":
         """Seeded N(0, std) weights generated on the device in fp16 (fp32 for a float32 model is not offered here),

@@ -31,6 +31,15 @@ class Tensor:
             self.lazydata, self.shape, self.dtype = buffer, tuple(shape), dtype or buffer.dtype
             return
         arr = np.asarray(data)
+        if dtype == "bfloat16":
+            if arr.dtype != np.uint16:
+                raise TypeError("bfloat16 data is passed as its 16-bit patterns (uint16)")
+            self.dtype, self.shape = "bfloat16", tuple(arr.shape)
+            self.lazydata = Buffer(self.device, max(1, arr.size), "bfloat16")
+            self.lazydata.allocate()
+            if arr.size:
+                self.lazydata.copyin(np.ascontiguousarray(arr))
+            return
         if dtype is not None:
             arr = arr.astype(DTYPES[dtype][0])
         elif arr.dtype == np.float64:
@@ -113,6 +122,17 @@ class Tensor:
         if int(np.prod(shape)) != self.numel:
             raise ValueError(f"size mismatch, can't reshape {self.shape} -> {shape}")
         return Tensor(buffer=self.lazydata, shape=shape, dtype=self.dtype, device=self.device)
+
+    def cast(self, dtype: str) -> "Tensor":
+        """Tensor.cast (tensor.ts:4141-4148) between float32 / float16, and from bfloat16 (through float32, which is what
+        fix_bf16 spells out, models/llama.ts:275).  Same dtype: the tensor itself."""
+        if dtype == self.dtype:
+            return self
+        if self.dtype not in ("float32", "float16", "bfloat16") or dtype not in ("float32", "float16"):
+            raise NotImplementedError(f"cast {self.dtype} -> {dtype} is not built on this device")
+        out = Tensor.empty(self.shape, dtype, self.device)
+        check(ffi.load().jsgrad_hip_cast(self.ptr, DTYPES[self.dtype][1], out.ptr, DTYPES[dtype][1], self.numel))
+        return out
 
     def __repr__(self) -> str:
         return f"<Tensor {self.shape} {self.dtype} on {self.device}>"

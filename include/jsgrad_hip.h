@@ -268,6 +268,20 @@ int jsgrad_hip_int8_dequant(const int8_t *codes, const void *scale_f16, int out_
 /* NF4Linear(64).quantize / the dequantisation of NF4Linear.call for n elements (llama3.ts:91-96,98-114). */
 int jsgrad_hip_nf4_quantize(const void *w, size_t n, uint8_t *packed, void *scale_f16, int act);
 int jsgrad_hip_nf4_dequant(const uint8_t *packed, const void *scale_f16, size_t n, void *w16);
+/* Checkpoint formats on the way into the model.
+ * ggml_dequant: ggml_data_to_tensor (nn/state.ts:192-223) for the quantised GGML types Q4_0 (2), Q4_1 (3), Q8_0 (8) and
+ *   Q6_K (14): n elements (whole blocks) from the block bytes at `blocks` (2-byte aligned) to float32.
+ *   ggml_nbytes: bytes that n elements of a type occupy (0 for a type that is not one of the four).
+ * cast: n elements between JSGRAD_F32 / JSGRAD_F16, and from JSGRAD_BF16 (fix_bf16, models/llama.ts:272-279: bfloat16 ->
+ *   float32 -> float16; `v.cast(float16)`, models/llama3.ts:234).
+ * hf_permute: the q_proj / k_proj row permutation of convert_from_huggingface (models/llama.ts:225-227),
+ *   dst = src.reshape(n_heads, 2, rows/n_heads/2, row).transpose(1, 2), rows of row_bytes bytes (a multiple of 16). */
+enum { JSGRAD_BF16 = 2 };
+size_t jsgrad_hip_ggml_nbytes(int ggml_type, size_t n);
+int jsgrad_hip_ggml_dequant(int ggml_type, const void *blocks, size_t n, void *out_f32);
+int jsgrad_hip_cast(const void *src, int src_dtype, void *dst, int dst_dtype, size_t n);
+int jsgrad_hip_hf_permute(const void *src, void *dst, int rows, int row_bytes, int n_heads);
+
 /* Random-init weights ~ N(0, std) in the given dtype (the role of Tensor.randn / Linear's random
  * initialisation, nn/index.ts:406-409, for synthetic models); counter-based, reproducible from seed. */
 int jsgrad_hip_randn(void *out, size_t n, int dtype, uint64_t seed, float std);
