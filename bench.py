@@ -126,7 +126,7 @@ def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=Tru
     from denograd_amd.llama3 import Llama3
 
     lib = ffi.load()
-    ctx = prompt_len + warmup + steps + 2 * (profile_steps + blocker_steps) + per_op_steps + 16
+    ctx = prompt_len + warmup + steps + 3 * (profile_steps + blocker_steps) + 2 * per_op_steps + 32
     cfg = synthetic.config(name, max_context=ctx)
     t0 = time.perf_counter()
     llm = Llama3.from_config(cfg, fused_step=fused_step).random_init(seed=0, tied=cfg["tied"])
@@ -183,6 +183,23 @@ def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=Tru
 
     fused = m._fused is not None
     kinds = profiled(profile_steps)
+    sampled = None
+    if not fused:
+        # the same steps ending in the reference's default sampler (temperature 0.95, whole-vocabulary draw, llama3.ts:192)
+        # instead of the greedy argmax: four small launches more per token
+        m._set_sampling(0.95, 0, 0.0, 0.0, 0.0)
+        m._step(); m._step(); m.generate(4)
+        llm.start_pos += 6
+        check(lib.jsgrad_hip_sync())
+        w1 = time.perf_counter()
+        m.generate(per_op_steps)
+        check(lib.jsgrad_hip_sync())
+        s_ms = 1e3 * (time.perf_counter() - w1) / per_op_steps
+        llm.start_pos += per_op_steps
+        sk = profiled(2).get("sample", {})
+        sampled = {"temperature": 0.95, "tok_s": round(1e3 / s_ms, 2), "ms_per_step": round(s_ms, 4), "sampler_launches_per_step": sk.get("launches_per_step"),
+                   "sampler_ms_per_step": round(sk.get("ms_per_step", 0.0), 4)}
+        m._set_sampling(0.0, 0, 0.0, 0.0, 0.0)
     per_op = None
     if fused:
         # the same model through the one-launch-per-op path, for the per-family table and as a second data point
@@ -244,6 +261,8 @@ def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=Tru
                    "prompt": prompt_len, "decode": steps, "avg_visible_positions": t_avg, "max_context": ctx,
                    "launch": ("one persistent kernel per token" if fused else "one launch per fused op") + (", replayed as a HIP graph" if use_graph else ", eager")},
     }
+    if sampled is not None:
+        res["sampled"] = sampled
     if per_op is not None:
         res["per_op_path"] = {"tok_s": round(1e3 / per_op_ms, 2), "ms_per_step": round(per_op_ms, 4), "kernels": rnd(per_op)}
     return llm, cfg, res
@@ -476,12 +495,13 @@ def main():
         "dtype": "f16", "data": "synthetic", "config": res["config"],
         "roofline": res["roofline"], "cpu_baseline": cpu,
         "step_roofline": res["step_roofline"], "kernels": res["kernels"], "event_ms_per_step": round(res["event_ms_per_step"], 4),
-        "launch_mode": "eager" if args.no_graph else "hip_graph", "per_op_path": res.get("per_op_path"),
+        "launch_mode": "eager" if args.no_graph else "hip_graph", "per_op_path": res.get("per_op_path"), "sampled": res.get("sampled"),
     }
     if secondary:
         out["secondary"] = {"value": round(secondary["tok_s"], 2), "unit": "tok/s", "steps": args.secondary_steps, "ms_per_step": round(secondary["ms_per_step"], 4),
                             "dtype": "i8 weights, f16 activations", "config": secondary["config"], "roofline": secondary["roofline"],
-                            "step_roofline": secondary["step_roofline"], "kernels": secondary["kernels"], "per_op_path": secondary.get("per_op_path")}
+                            "step_roofline": secondary["step_roofline"], "kernels": secondary["kernels"], "per_op_path": secondary.get("per_op_path"),
+                            "sampled": secondary.get("sampled")}
     if args.batched:
         out["batched"] = run_batched(args.batched, args.batch, args.batch_prompt, args.batch_steps)
     out["formats"] = run_formats()

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libjsgrad_hip.so")
 
 F32, F16, BF16 = 0, 1, 2
 W_F32, W_F16, W_I8, W_NF4 = 0, 1, 2, 3
-PROF_KINDS = {"embed": 0, "rmsnorm": 1, "linear": 2, "qkv_rope": 3, "attn_decode": 4, "ffn_gate": 5, "argmax": 6, "decode_step": 7, "gemm": 8, "attn_prefill": 9, "attn_wo": 10, "read_probe": 11}
+PROF_KINDS = {"embed": 0, "rmsnorm": 1, "linear": 2, "qkv_rope": 3, "attn_decode": 4, "ffn_gate": 5, "argmax": 6, "decode_step": 7, "gemm": 8, "attn_prefill": 9, "attn_wo": 10, "read_probe": 11, "sample": 12}
 
 
 class HipError(RuntimeError):
@@ -79,6 +79,8 @@ SIGNATURES: dict[str, tuple[list, object]] = {
     "jsgrad_hip_stream_step": ([_vp], _i32),
     "jsgrad_hip_stream_status": ([_vp, C.POINTER(_i32)], _i32),
     "jsgrad_hip_read_probe": ([_vp, _sz, _vp], _i32),
+    "jsgrad_hip_sample_workspace_bytes": ([_i32], _sz),
+    "jsgrad_hip_sample": ([_vp, _i32, _i32, C.c_double, _i32, C.c_double, C.c_double, C.c_double, _vp, _vp, _vp, _vp, _i32, _i32, _vp], _i32),
     "jsgrad_hip_ggml_nbytes": ([_i32, _sz], _sz),
     "jsgrad_hip_ggml_dequant": ([_i32, _vp, _sz, _vp], _i32),
     "jsgrad_hip_cast": ([_vp, _i32, _vp, _i32, _sz], _i32),

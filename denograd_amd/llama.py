@@ -283,6 +283,10 @@ class Transformer:
         self.fuse_attn_wo = fuse_attn_wo   # attention and wo of a layer as one launch, where the model qualifies
         self._fused: _FusedStep | None = None
         self._rows: _RowScratch | None = None
+        # sampling (llama.ts:131-185): (temperature, top_k, top_p, alpha_f, alpha_p) of the current calls; greedy until told otherwise
+        self._sampling = (0.0, 0, 0.0, 0.0, 0.0)
+        self.alpha_counter: Tensor | None = None      # llama.ts:130: created on the first call with alpha_f or alpha_p (module-wide in the reference)
+        self._sample_ws: Tensor | None = None
 
     def attn_wo_error(self) -> int:
         """1 if a bounded wait inside a fused attention + wo launch ever ran out (its result is then not to be trusted)."""
@@ -330,8 +334,40 @@ class Transformer:
         for layer in self.layers:
             h = layer.call(h, self.state, self.freqs_cis, ctx)
         self.output.call(h, out=ctx.logits, norm=self.norm)
-        check(ffi.load().jsgrad_hip_argmax(ctx.logits.ptr, self.vocab_size, self.state.ptr, self.tokens_out.ptr, self.max_context, 1, act_code(self.dtype)))
+        self._pick_token(ctx.logits)
         return Tensor(buffer=self.state.lazydata.view(1, "int32", 0), shape=(), dtype="int32", device=self.device)
+
+    def _pick_token(self, logits: Tensor) -> None:
+        """`sample(logits.flatten(), ...)` (llama.ts:212): the token goes to state[0], the position advances."""
+        lib = ffi.load()
+        temp, k, p, af, ap = self._sampling
+        if temp < 1e-6:
+            check(lib.jsgrad_hip_argmax(logits.ptr, self.vocab_size, self.state.ptr, self.tokens_out.ptr, self.max_context, 1, act_code(self.dtype)))
+            return
+        if self._sample_ws is None:
+            self._sample_ws = Tensor.zeros((lib.jsgrad_hip_sample_workspace_bytes(self.vocab_size),), "uint8", self.device)
+        if (af or ap) and self.alpha_counter is None:
+            self.alpha_counter = Tensor.zeros((self.vocab_size,), "int32", self.device)
+        check(lib.jsgrad_hip_sample(logits.ptr, self.vocab_size, act_code(self.dtype), temp, k, p, af, ap,
+                                    self.alpha_counter.ptr if self.alpha_counter is not None else None, rng_state(self.device).ptr,
+                                    self.state.ptr, self.tokens_out.ptr, self.max_context, 1, self._sample_ws.ptr))
+
+    def _set_sampling(self, temperature: float, top_k: int, top_p: float, alpha_f: float, alpha_p: float) -> None:
+        """Argument checks of `sample` (llama.ts:132-134); a change of parameters drops the captured graph, which has them baked in."""
+        if temperature >= 1e-6:
+            if not 0 <= top_p <= 1:
+                raise ValueError("p must be between 0 and 1")
+            if not 0 <= top_k <= self.vocab_size:
+                raise ValueError("k must be between 0 and numel")
+            if self.fused_step:
+                raise NotImplementedError("the whole-step kernels end in the greedy argmax; sampling runs on the per-op path")
+            new = (float(temperature), int(top_k), float(top_p), float(alpha_f), float(alpha_p))
+        else:
+            new = (0.0, 0, 0.0, 0.0, 0.0)
+        if new != self._sampling:
+            self._sampling = new
+            if self.forward_jit is not None:
+                self.forward_jit.reset()
 
     def _advance_host_pos(self) -> None:
         self._pos += 1
@@ -352,9 +388,9 @@ class Transformer:
     # ---- the reference's entry points
     def forward(self, tokens, start_pos: int, temperature: float = 0.0, top_k: int = 0, top_p: float = 0.8, alpha_f: float = 0.0, alpha_p: float = 0.0) -> Tensor:
         """llama.ts:201-213 for one sequence.  Several tokens are fed position by position (the reference's own
-        prefill is token-serial, models/llama3.ts:307-311); the returned tensor is the greedy token of the last one."""
-        if temperature >= 1e-6:
-            raise NotImplementedError("only greedy decoding (temperature 0 -> argmax, llama.ts:137) is built on this device")
+        prefill is token-serial, models/llama3.ts:307-311); the returned tensor is the token picked after the last one
+        (every position draws, as in the reference: each one advances the random counter and the alpha counter)."""
+        self._set_sampling(temperature, top_k, top_p, alpha_f, alpha_p)
         toks = np.asarray(tokens.numpy() if isinstance(tokens, Tensor) else tokens, np.int32)
         if toks.ndim != 2 or toks.shape[0] != 1:
             raise ValueError(f"tokens must have shape [1, seqlen], got {toks.shape}; several sequences go through forward_rows")
@@ -451,8 +487,7 @@ class Transformer:
         """llama.ts:214-220: single-token calls past position 0 go through the jit (a captured graph)."""
         toks = np.asarray(tokens.numpy() if isinstance(tokens, Tensor) else tokens, np.int32)
         if toks.shape == (1, 1) and self.forward_jit is not None and start_pos != 0:
-            if temperature >= 1e-6:
-                raise NotImplementedError("only greedy decoding (temperature 0 -> argmax, llama.ts:137) is built on this device")
+            self._set_sampling(temperature, top_k, top_p, alpha_f, alpha_p)
             self.set_state(int(toks[0, 0]), start_pos)
             return self.forward_jit.call()
         return self.forward(toks, start_pos, temperature, top_k, top_p, alpha_f, alpha_p)
@@ -470,6 +505,29 @@ class Transformer:
             raise ValueError(f"{n_steps} steps from position {self._pos} overrun the KV cache of {self.max_context} positions")
         for _ in range(n_steps):
             self.forward_jit.call()
+
+
+# *** random numbers of the sampler (tensor.ts:773-843) ***
+_SEED = [0]
+_RNG: dict[str, Tensor] = {}
+
+
+def manual_seed(seed: int = 0) -> None:
+    """Tensor.manual_seed (tensor.ts:773-775): the seed of the next draws; every device starts over at counter 0."""
+    _SEED[0] = int(seed) & 0xFFFFFFFF
+    _RNG.clear()
+
+
+def rng_state(device: str = "HIP") -> Tensor:
+    """The device words Tensor.rand works from: {sha256(number of devices seeded before this one) mod 2^32, seed, counter}
+    (tensor.ts:813-819), as int32 storage; jsgrad_hip_sample reads them and advances the counter."""
+    from .device import Device
+    device = Device.canonicalize(device)
+    if device not in _RNG:
+        import hashlib
+        key0 = int.from_bytes(hashlib.sha256(len(_RNG).to_bytes(4, "big")).digest(), "big") % 2 ** 32
+        _RNG[device] = Tensor(np.array([key0, _SEED[0], 0], np.uint32).view(np.int32), device=device)
+    return _RNG[device]
 
 
 # *** helpers (llama.ts:222-279) ***

@@ -18,7 +18,7 @@ def get_state_dict(obj, prefix: str = "") -> dict[str, Tensor]:
         return out
     if hasattr(obj, "__dict__"):
         for k, v in vars(obj).items():
-            if k.startswith("_") or k in ("state", "tokens_out", "freqs_cis", "cache_kv", "forward_jit"):
+            if k.startswith("_") or k in ("state", "tokens_out", "freqs_cis", "cache_kv", "forward_jit", "alpha_counter"):
                 continue
             if isinstance(v, (Tensor, list, tuple)) or (hasattr(v, "__dict__") and not callable(v)):
                 out.update(get_state_dict(v, f"{prefix}{k}."))
@@ -34,6 +34,8 @@ def _slots(obj, prefix: str = ""):
     for k, v in vars(obj).items():
         if k in ("weight", "scale"):
             yield f"{prefix}{k}", obj, k
+        elif k.startswith("_"):
+            continue
         elif isinstance(v, (list, tuple)) or (hasattr(v, "__dict__") and not isinstance(v, Tensor) and not callable(v) and not k.startswith("_") and k not in ("forward_jit",)):
             yield from _slots(v, f"{prefix}{k}.")
 

@@ -79,7 +79,7 @@ int jsgrad_hip_event_destroy(void *event);
 /* Per-kernel statistics (DEBUG>=2 of engine/realize.ts:168-178; ProfileRangeEvent, runtime/allocator.ts:147-151):
  * while enabled, every Llama kernel launched outside a graph capture is bracketed by an event pair.  `read` waits
  * for the stream and returns launch count and summed milliseconds of one kind since profiling was enabled. */
-enum { JSGRAD_PROF_EMBED = 0, JSGRAD_PROF_RMSNORM, JSGRAD_PROF_LINEAR, JSGRAD_PROF_QKV_ROPE, JSGRAD_PROF_ATTN, JSGRAD_PROF_FFN_GATE, JSGRAD_PROF_ARGMAX, JSGRAD_PROF_STEP, JSGRAD_PROF_GEMM, JSGRAD_PROF_ATTN_PREFILL, JSGRAD_PROF_ATTN_WO, JSGRAD_PROF_READ };
+enum { JSGRAD_PROF_EMBED = 0, JSGRAD_PROF_RMSNORM, JSGRAD_PROF_LINEAR, JSGRAD_PROF_QKV_ROPE, JSGRAD_PROF_ATTN, JSGRAD_PROF_FFN_GATE, JSGRAD_PROF_ARGMAX, JSGRAD_PROF_STEP, JSGRAD_PROF_GEMM, JSGRAD_PROF_ATTN_PREFILL, JSGRAD_PROF_ATTN_WO, JSGRAD_PROF_READ, JSGRAD_PROF_SAMPLE };
 int jsgrad_hip_profile(int enable);
 int jsgrad_hip_profile_read(int kind, int *host_out_count, double *host_out_total_ms);
 
@@ -268,6 +268,19 @@ int jsgrad_hip_int8_dequant(const int8_t *codes, const void *scale_f16, int out_
 /* NF4Linear(64).quantize / the dequantisation of NF4Linear.call for n elements (llama3.ts:91-96,98-114). */
 int jsgrad_hip_nf4_quantize(const void *w, size_t n, uint8_t *packed, void *scale_f16, int act);
 int jsgrad_hip_nf4_dequant(const uint8_t *packed, const void *scale_f16, size_t n, void *w16);
+/* `sample` (models/llama.ts:131-185) on the logits of one position: alpha penalties with their counter, NaN -> -inf,
+ * softmax(logits / temp), then Tensor.multinomial (tensor.ts:1164-1172) over the whole vocabulary (k == 0) or over the k
+ * largest after the top-p mask; temp < 1e-6 is the greedy jsgrad_hip_argmax.  The uniform number is the float32 that
+ * Tensor.rand([1,1,1]) draws (tensor.ts:798-843): Threefry-2x32-20 under the key rng[0] (sha256 of the device count, see
+ * Tensor._device_seeds), rng[1] (the seed of Tensor.manual_seed) at the counter rng[2], which the call advances by one.
+ * The token goes to state[0] (and tokens_out[state[1]]), state[1] advances when `advance` is set, alpha_counter[token]
+ * grows by one when af or ap is set (may be NULL otherwise).  Everything is device memory and the call only queues
+ * kernels, so it can sit inside a captured graph.  workspace: jsgrad_hip_sample_workspace_bytes(n) bytes, zero-filled once
+ * before first use.  n: more than 512 and at most 1048576 logits; k <= 256. */
+size_t jsgrad_hip_sample_workspace_bytes(int n);
+int jsgrad_hip_sample(const void *logits, int n, int act, double temp, int k, double p, double af, double ap, int32_t *alpha_counter, uint32_t *rng,
+                      int32_t *state, int32_t *tokens_out, int tokens_cap, int advance, void *workspace);
+
 /* Checkpoint formats on the way into the model.
  * ggml_dequant: ggml_data_to_tensor (nn/state.ts:192-223) for the quantised GGML types Q4_0 (2), Q4_1 (3), Q8_0 (8) and
  *   Q6_K (14): n elements (whole blocks) from the block bytes at `blocks` (2-byte aligned) to float32.
