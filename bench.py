@@ -464,6 +464,7 @@ def main():
     ap.add_argument("--traffic-batch", type=int, default=1, help="with --traffic-probe: also two batched decode steps of this many sequences")
     ap.add_argument("--fused-step", action="store_true", help="run each token as one persistent kernel (jsgrad_hip_decode_step) instead of one launch per fused op")
     ap.add_argument("--stream-step", action="store_true", help="run each token as one persistent kernel with streaming wavefronts (jsgrad_hip_stream_step)")
+    ap.add_argument("--formats-only", action="store_true", help="only the load-time kernels of the checkpoint path (GGML dequantisation, casts, row permutation); prints their JSON")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel eagerly instead of replaying a captured HIP graph "
                     "(rocprofv3 --kernel-trace on this image crashes inside hipGraphLaunch, so profiles are taken this way)")
     args = ap.parse_args()
@@ -478,6 +479,9 @@ def main():
 
     if args.traffic_probe:
         traffic_probe(args.workload, args.traffic_batch)
+        return
+    if args.formats_only:
+        print(json.dumps({"formats": run_formats()}), flush=True)
         return
     step_mode = "stream" if args.stream_step else args.fused_step
     llm, cfg, res = run_workload(args.workload, args.prompt, args.steps, args.warmup, use_graph=not args.no_graph, fused_step=step_mode)

@@ -14,8 +14,8 @@
 //   prep  y = (logit - penalty, NaN -> -inf) * (1/temp); chunk maxima
 //   exp   e = exp(y - max); chunk sums
 //   cdf   t = e * (1 / sum); running sums inside the chunk; chunk totals
-//   pick  cdf = (running sum + totals before) * (1 / grand total); count of cdf entries <= u; the last block to finish
-//         writes the token, advances the position, the alpha counter and the random counter
+//   pick  (one block) cdf = (running sum + totals before) * (1 / grand total); count of cdf entries <= u, found in the one
+//         chunk where the cdf passes u; writes the token, advances the position, the alpha counter and the random counter
 // With top_k > 0 the last launch is one block instead: k times (largest value, lowest index among equals, zero it), the
 // top-p mask over those k, and the draw among them.
 #include "common.h"
@@ -37,7 +37,6 @@ struct SampleArgs {
   int32_t *st, *tokens_out;
   int tokens_cap, advance;
   float *y, *prefix, *cmax, *csum, *ctot;   // workspace: [nch*256] x 2, [nch] x 3
-  int *counters;                  // {blocks finished, count}, zero between calls
 };
 
 __device__ __forceinline__ void threefry2x32(uint32_t &x0, uint32_t &x1, uint32_t k0, uint32_t k1) {
@@ -105,7 +104,16 @@ __device__ __forceinline__ float sample_seq_sum(const float *v, int n, int mark,
   float s = 0.0f;
   before = 0.0f;
   if (threadIdx.x == 0) {
-    for (int c = 0; c < n; c++) {
+    int c = 0;
+    for (; c + 4 <= n; c += 4) {           // four values per LDS read; only the additions depend on each other
+      const f4_t t = *(const f4_t *)&stage[c];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        if (c + e == mark) before = s;
+        s = s + t[e];
+      }
+    }
+    for (; c < n; c++) {
       if (c == mark) before = s;
       s = s + stage[c];
     }
@@ -116,7 +124,7 @@ __device__ __forceinline__ float sample_seq_sum(const float *v, int n, int mark,
 
 __global__ __launch_bounds__(SM_CHUNK) void sample_exp_kernel(SampleArgs a) {
   __shared__ float red[SM_CHUNK / 64];
-  __shared__ float e_sh[SM_CHUNK];
+  __shared__ __align__(16) float e_sh[SM_CHUNK];
   const int slot = blockIdx.x * SM_CHUNK + threadIdx.x;
   const float M = sample_global_max(a, red);
   const float e = exp_f32(a.y[slot] - M);
@@ -125,7 +133,10 @@ __global__ __launch_bounds__(SM_CHUNK) void sample_exp_kernel(SampleArgs a) {
   __syncthreads();
   if (threadIdx.x == 0) {
     float s = 0.0f;
-    for (int l = 0; l < SM_CHUNK; l++) s = s + e_sh[l];
+    for (int l = 0; l < SM_CHUNK; l += 4) {
+      const f4_t t = *(const f4_t *)&e_sh[l];
+      s = s + t[0]; s = s + t[1]; s = s + t[2]; s = s + t[3];
+    }
     a.csum[blockIdx.x] = s;
   }
 }
@@ -133,7 +144,7 @@ __global__ __launch_bounds__(SM_CHUNK) void sample_exp_kernel(SampleArgs a) {
 // WITH_PREFIX: also the running sums inside the chunk and the chunk total (the whole-vocabulary draw); without, only t
 template <bool WITH_PREFIX> __global__ __launch_bounds__(SM_CHUNK) void sample_cdf_kernel(SampleArgs a) {
   __shared__ float t_sh[SM_CHUNK];
-  __shared__ float stage[SM_MAXCH];
+  __shared__ __align__(16) float stage[SM_MAXCH];
   __shared__ float rs_sh;
   const int slot = blockIdx.x * SM_CHUNK + threadIdx.x;
   float unused;
@@ -162,36 +173,55 @@ __device__ __forceinline__ void sample_finish(const SampleArgs &a, int token) {
   a.rng[2] = a.rng[2] + 1u;                                              // the next Tensor.rand of one number (tensor.ts:819)
 }
 
+// One block.  The cdf never decreases (running sums of non-negative weights, float addition and the multiplication by a
+// positive number are monotone), and the last cdf entry of a chunk is (chunk total + totals before) * inv, which the chunk
+// totals alone give.  So: thread 0 turns the totals into the totals BEFORE each chunk and the grand total; the threads
+// look for the first chunk whose last entry is above u; only that chunk's running sums are read and compared.  Every
+// chunk before it counts whole, every chunk after it not at all - the same count as comparing all entries.
 __global__ __launch_bounds__(SM_CHUNK) void sample_pick_kernel(SampleArgs a) {
-  __shared__ float base_sh, inv_sh, u_sh;
-  __shared__ float stage[SM_MAXCH];
-  __shared__ int cnt_sh[SM_CHUNK / 64];
-  const int slot = blockIdx.x * SM_CHUNK + threadIdx.x, i = slot - a.pad;
-  float before;
-  const float total = sample_seq_sum(a.ctot, a.nch, blockIdx.x, before, stage);
-  if (threadIdx.x == 0) {
-    base_sh = before;
-    inv_sh = 1.0f / total;
+  __shared__ __align__(16) float tot_sh[SM_MAXCH], base_sh[SM_MAXCH];
+  __shared__ float inv_sh, u_sh;
+  __shared__ int red_sh[SM_CHUNK / 64];
+  const int tid = threadIdx.x;
+  for (int c = tid; c < a.nch; c += SM_CHUNK) tot_sh[c] = a.ctot[c];
+  __syncthreads();
+  if (tid == 0) {
+    // reads of one array, writes to another: only the additions depend on each other
+    float s = 0.0f;
+    int c = 0;
+    for (; c + 4 <= a.nch; c += 4) {
+      const f4_t t = *(const f4_t *)&tot_sh[c];
+      f4_t b;
+      b[0] = s; s = s + t[0];
+      b[1] = s; s = s + t[1];
+      b[2] = s; s = s + t[2];
+      b[3] = s; s = s + t[3];
+      *(f4_t *)&base_sh[c] = b;
+    }
+    for (; c < a.nch; c++) { base_sh[c] = s; s = s + tot_sh[c]; }
+    inv_sh = 1.0f / s;
     u_sh = sample_uniform(a.rng);
   }
   __syncthreads();
-  const float cdf = (a.prefix[slot] + base_sh) * inv_sh;
-  const bool hit = i >= 0 && i < a.n && u_sh >= cdf;
-  const int c = __popcll(__ballot(hit));
-  if ((threadIdx.x & 63) == 0) cnt_sh[threadIdx.x >> 6] = c;
+  const float inv = inv_sh, u = u_sh;
+  int first = a.nch;                                    // first chunk that is not counted whole
+  for (int c = tid; c < a.nch; c += SM_CHUNK)
+    if (!(u >= (tot_sh[c] + base_sh[c]) * inv)) { first = c; break; }
+  for (int off = 32; off > 0; off >>= 1) first = min(first, __shfl_xor(first, off));
+  if ((tid & 63) == 0) red_sh[tid >> 6] = first;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    const int mine = cnt_sh[0] + cnt_sh[1] + cnt_sh[2] + cnt_sh[3];
-    if (mine) __hip_atomic_fetch_add(&a.counters[1], mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __builtin_amdgcn_s_waitcnt(0);   // the count has arrived before this block reports in
-    const int done = __hip_atomic_fetch_add(&a.counters[0], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (done == (int)gridDim.x - 1) {
-      const int token = __hip_atomic_load(&a.counters[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      sample_finish(a, token);
-      __hip_atomic_store(&a.counters[0], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(&a.counters[1], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
+  first = min(min(red_sh[0], red_sh[1]), min(red_sh[2], red_sh[3]));
+  __syncthreads();
+  int token = a.n;                                      // u >= every entry (possible when the last entry rounds below 1)
+  if (first < a.nch) {
+    const int slot = first * SM_CHUNK + tid, i = slot - a.pad;
+    const bool hit = i >= 0 && i < a.n && u >= (a.prefix[slot] + base_sh[first]) * inv;
+    const int c = __popcll(__ballot(hit));
+    if ((tid & 63) == 0) red_sh[tid >> 6] = c;
+    __syncthreads();
+    token = (first > 0 ? first * SM_CHUNK - a.pad : 0) + red_sh[0] + red_sh[1] + red_sh[2] + red_sh[3];
   }
+  if (tid == 0) sample_finish(a, token);
 }
 
 // top_k > 0: one block over t (in a.y, the padding holds zeros)
@@ -290,7 +320,6 @@ int jsgrad_hip_sample(const void *logits, int n, int act, double temp, int k, do
   a.use_alpha = alpha; a.k = k; a.alpha = alpha_counter; a.rng = rng;
   a.st = st; a.tokens_out = tokens_out; a.tokens_cap = tokens_cap; a.advance = advance;
   char *ws = (char *)workspace;
-  a.counters = (int *)ws;
   a.y = (float *)(ws + 256);
   a.prefix = a.y + (size_t)a.nch * SM_CHUNK;
   const size_t nchp = ((size_t)a.nch + 63) / 64 * 64;
@@ -303,7 +332,7 @@ int jsgrad_hip_sample(const void *logits, int n, int act, double temp, int k, do
   JSG_LAUNCH(PROF_SAMPLE, sample_exp_kernel, grid, block, 0, a);
   if (k == 0) {
     JSG_LAUNCH(PROF_SAMPLE, sample_cdf_kernel<true>, grid, block, 0, a);
-    JSG_LAUNCH(PROF_SAMPLE, sample_pick_kernel, grid, block, 0, a);
+    JSG_LAUNCH(PROF_SAMPLE, sample_pick_kernel, dim3(1), dim3(SM_CHUNK), 0, a);
   } else {
     JSG_LAUNCH(PROF_SAMPLE, sample_cdf_kernel<false>, grid, block, 0, a);
     JSG_LAUNCH(PROF_SAMPLE, sample_topk_kernel, dim3(1), dim3(SM_TOPK_THREADS), 0, a);
