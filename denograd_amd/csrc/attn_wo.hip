@@ -74,8 +74,8 @@ template <int KIND, int HD> static int launch_attn_wo(const AttnArgs &at, const 
     JSG_LAUNCH(PROF_ATTN_WO, (attn_wo_kernel<KIND, HD, N>), dim3(blocks), dim3(AW_THREADS), lds, at, a, layer);       \
     break;
   switch (n_rep) {
-    JSG_REP(1) JSG_REP(2) JSG_REP(4)
-    default: return fail("jsgrad_hip_attn_wo: n_heads/n_kv_heads = %d is not one of 1,2,4", n_rep);
+    JSG_REP(1) JSG_REP(2) JSG_REP(3) JSG_REP(4)
+    default: return fail("jsgrad_hip_attn_wo: n_heads/n_kv_heads = %d is not one of 1,2,3,4", n_rep);
   }
 #undef JSG_REP
   return 0;

@@ -9,7 +9,7 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL>
 __global__ __launch_bounds__(256) void gemv_kernel(GemvArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   __shared__ float red[8];
-  __shared__ float lut[16];
+  __shared__ float lut[KIND == JSGRAD_W_NF4 ? NF4_LUT_WORDS : 16];
   typedef Gemv<KIND, AT, EPI, ROWS, UNROLL, false> G;
   // read the position now, not in the epilogue: the load then overlaps the weight stream instead of ending the kernel
   const int pos = EPI == EPI_ROPE_KV ? a.st[1] : 0;

@@ -145,6 +145,27 @@ template <> struct Dot<JSGRAD_W_I8, _Float16> {
   }
 };
 
+// fp16 activations x NF4 weights.  One byte holds two codes (element 2j in the high nibble, llama3.ts:92-94,105), and the
+// lane's x fragment holds the two activations they meet as one packed pair: a 256-entry LDS table indexed by the byte gives
+// both code values as a packed fp16 pair, ready for the packed dot.  The block scale (one per 64 elements, so one per
+// 16-byte vector) multiplies the sum of the 32 products once: code * scale is exact in float either way, the sums differ
+// from the generic path's in the last float bits only.  lut: 16 floats (the generic table), then the 256 pairs.
+constexpr int NF4_LUT_WORDS = 16 + 256;
+template <> struct Dot<JSGRAD_W_NF4, _Float16> {
+  static constexpr int VEC = 32;
+  __device__ static __forceinline__ float run(u4_t wv, const XFrag<_Float16, 32> &xf, float acc, float blk_scale, const float *lut) {
+    const uint32_t *pairs = (const uint32_t *)lut + 16;
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t d = wv[i];
+#pragma unroll
+      for (int b = 0; b < 4; b++) s = __builtin_amdgcn_fdot2(as_h2(pairs[(d >> (8 * b)) & 0xffu]), xf.v[4 * i + b], s, false);
+    }
+    return acc + s * blk_scale;
+  }
+};
+
 // Stage x (optionally RMSNorm'ed) into LDS in the activation dtype.  Every thread moves 16-byte chunks; with a
 // norm the chunks stay in registers between the sum of squares and the scaling, so x is read from memory once and
 // the whole prologue costs one round of loads and two barriers.  Ends with a barrier.
@@ -289,6 +310,7 @@ struct GemvBuf {
   // where they are used: any arithmetic at load time, even a zero-extension, waits for the load, and loads complete in
   // order, so it would wait for the weight vectors issued before it as well.
   _Float16 scale[4];    // [j][r] flattened: the int8 row scale
+  _Float16 nscale[8];   // NF4: the block scale of each of the 8 vectors (one per 64 elements), fetched with them
   _Float16 extra_h[2];  // fp16 activations - EPI_STORE: residual[row]; EPI_ROPE_KV: cos or sin of the rotary pair
   float extra_f[2];     // the same for float32 activations
 };
@@ -357,6 +379,7 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
           const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;  // tail rows reload the last row, never stored
           const char *p = (const char *)wbase(a, w.m, j) + (((size_t)row * in_f + (size_t)k) * BITS) / 8;
           buf.w[wi(u, j, r)] = ldg_stream16(p);
+          if constexpr (KIND == JSGRAD_W_NF4) buf.nscale[wi(u, j, r)] = ldg((const _Float16 *)sbase(a, w.m, j) + (((size_t)row * in_f + (size_t)k) >> 6));
         }
     }
     if (b != nbatch(a) - 1) return;
@@ -448,11 +471,7 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
 #pragma unroll
         for (int r = 0; r < ROWS; r++) {
           float bs = 1.0f;
-          if constexpr (KIND == JSGRAD_W_NF4) {
-            const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;
-            const int kc = k < in_f ? k : in_f - VEC;
-            bs = (float)ldg((const _Float16 *)sbase(a, w.m, j) + (((size_t)row * in_f + kc) >> 6));
-          }
+          if constexpr (KIND == JSGRAD_W_NF4) bs = (float)buf.nscale[wi(u, j, r)];
           // every 16-byte vector is summed on its own and then added: eight short dependent chains per item
           // instead of two long ones
           acc[j][r] += Dot<KIND, AT>::run(buf.w[wi(u, j, r)], xf, 0.0f, bs, lut);
@@ -506,11 +525,20 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
     }
   }
 
-  // xs: LDS for in_f activations; red: LDS float[blockDim/64]; lut: LDS float[16] (NF4 code book, written here)
+  // xs: LDS for in_f activations; red: LDS float[blockDim/64]; lut: LDS float[16] (NF4 code book, written here), and for
+  // NF4 weights with fp16 activations NF4_LUT_WORDS words (the table of code pairs behind it)
   __device__ static __forceinline__ void run(const GemvArgs &a, AT *xs, float *red, float *lut, Buf &bufA, bool preloaded, int pos) {
     const int wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     const int ng = ngroups(a), nb = nbatch(a), gstride = gridDim.x * nw;
-    if (KIND == JSGRAD_W_NF4 && threadIdx.x < 16) lut[threadIdx.x] = NF4_CODE[threadIdx.x];
+    if constexpr (KIND == JSGRAD_W_NF4) {
+      if (threadIdx.x < 16) lut[threadIdx.x] = NF4_CODE[threadIdx.x];
+      if constexpr (sizeof(AT) == 2) {   // the table of code pairs, one entry per byte value (lut has NF4_LUT_WORDS words then)
+        for (int e = threadIdx.x; e < 256; e += blockDim.x) {
+          const h2_t pr = {(_Float16)NF4_CODE[e >> 4], (_Float16)NF4_CODE[e & 15]};
+          ((uint32_t *)lut)[16 + e] = __builtin_bit_cast(uint32_t, pr);
+        }
+      }
+    }
     int grp = blockIdx.x * nw + wave, b = 0;
     if (!preloaded && grp < ng) load_item(a, bufA, grp, 0, pos);
     auto advance = [&](int &g, int &bb) {

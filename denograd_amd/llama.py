@@ -314,7 +314,7 @@ class Transformer:
                 layer.attention.layer_id = i
             wo = self.layers[0].attention.wo
             if (self.fuse_attn_wo and self.dtype == "float16" and wo.kind in (ffi.W_F16, ffi.W_I8) and 2 <= len(self.layers) <= 128 and hd in (64, 128)
-                    and self.n_heads // self.n_kv_heads in (1, 2, 4) and self.max_context <= 64 * 256 and self.n_heads * hd * 2 <= 64 * 1024):
+                    and self.n_heads // self.n_kv_heads in (1, 2, 3, 4) and self.max_context <= 64 * 256 and self.n_heads * hd * 2 <= 64 * 1024):
                 self._ctx.enable_attn_wo(self.n_heads, self.n_kv_heads, hd, self.device)
             if self.fused_step:
                 self._fused = _FusedStep(self, self._ctx, self._fused_mode())      # raises NotImplementedError for models it was not built for
