@@ -57,6 +57,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
   static constexpr int EPL = 16 / sizeof(AT);  // elements per lane per 128-bit load
   static constexpr int G = HD / EPL;           // lanes per cache row
   static constexpr int RPI = 64 / G;           // rows per wavefront iteration
+  static_assert(G == 8 || G == 16 || G == 32, "the fold over row groups is written for 8, 16 or 32 lanes per row");
   struct Smem {
     float sc[NREP][ATT_CHUNK_MAX];
     float red[NREP][NW];
@@ -140,6 +141,19 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       }
     }
     __syncthreads();
+    if (CH <= 64 && NREP <= NW) {
+      // A short chunk (the usual case for one sequence): the scores of a head fit one wavefront, lane i holding row i, so
+      // wavefront j does the whole softmax of head j by itself - maximum, exp, sum - with no barrier in between.
+      if (wave < NREP) {
+        const int j = wave;
+        const float s = lane < CH ? sm.sc[j][lane] : -INFINITY;
+        const float m = wave_max(s);
+        const float e = lane < CH ? exp_f32(s - m) : 0.0f;
+        if (lane < CH) sm.sc[j][lane] = e;
+        const float l = wave_sum(e);
+        if (lane == 0) { sm.m_sh[j] = m; sm.l_sh[j] = l; }
+      }
+    } else {
     // chunk maximum per head
     {
       float mx[NREP];
@@ -185,6 +199,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
         sm.l_sh[tid] = w;
       }
       // the barrier below also orders the in-place exp writes before phase 2 reads them
+    }
     }
     __syncthreads();
 
@@ -234,8 +249,9 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
 #pragma unroll
       for (int e = 0; e < EPL; e++) {
         float v = of[j][e];
-#pragma unroll
-        for (int off = G; off < 64; off <<= 1) v += __shfl_xor(v, off);
+        if constexpr (G <= 8) v += dpp_f<0x128>(v);    // row_ror:8: lane l ^ 8 of the same 16-lane row
+        if constexpr (G <= 16) v = add_xor16(v);
+        v = add_xor32(v);
         of[j][e] = v;
       }
     // wavefronts fold into (at most) four LDS slots, four at a time

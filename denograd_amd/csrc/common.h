@@ -133,6 +133,19 @@ __device__ __forceinline__ float wave_max(float v) {
   v = fmaxf(v, dpp_f<0x140>(v));
   return fmaxf(fmaxf(readlane_f(v, 0), readlane_f(v, 16)), fmaxf(readlane_f(v, 32), readlane_f(v, 48)));
 }
+// v[l] + v[l ^ 16] and v[l] + v[l ^ 32] for every lane, in the vector ALU (v_permlane16_swap / v_permlane32_swap exchange
+// the odd 16-lane rows, or the upper half, of one operand with the even rows, or the lower half, of the other; given the
+// same value twice, the two results added hold the pair sum in both places).  A shuffle through the LDS crossbar does the
+// same and queues behind every other LDS access of the CU.
+__device__ __forceinline__ float add_xor16(float v) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float add_xor32(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // sum over aligned groups of 16 lanes (one DPP row); every lane of the group gets the group total
 __device__ __forceinline__ float row16_sum(float v) {
   v += dpp_f<0xB1>(v);
