@@ -322,24 +322,55 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       if (lane == 0) sm.l_sh[j] = 1.0f / L;  // softmax normalisation is e * (1/sum) (tensor.ts:2211-2214)
     }
     __syncthreads();
-    // ... then every thread sums its output elements over the chunks, 32 chunks per round trip, in chunk order
-    for (int i = tid; i < NREP * HD; i += nthreads) {
+    // ... then every thread sums its output elements over the chunks in chunk order.  Two elements at a time: the first 32
+    // chunks of both are requested together (one round trip where there would be two; few chunks is the usual case)
+    auto finish = [&](int i, float O) {
       const int j = i / HD, d = i % HD;
-      const float *po = base + (size_t)j * (HD + 2) + d;
-      float O = 0.0f;
-      for (int s0 = 0; s0 < n_active; s0 += 32) {
-        float part[32];
-#pragma unroll
-        for (int u = 0; u < 32; u++) part[u] = ld_coherent(po + (size_t)(s0 + u < n_active ? s0 + u : n_active - 1) * NREP * (HD + 2));
-#pragma unroll
-        for (int u = 0; u < 32; u++)
-          if (s0 + u < n_active) O = fmaf(part[u], sm.sc[j][s0 + u], O);
-      }
       AT *dst = (AT *)a.out + (size_t)(g * NREP + j) * HD + d;
       const float r = Act<AT>::rn(O * sm.l_sh[j]);  // the cast of the P.V result
       if (a.out_tagged != nullptr) tw_store(a.out_tagged + (size_t)(g * NREP + j) * HD + d, a.out_tag, r);
       else if constexpr (COHERENT) st_coherent(dst, (AT)r);
       else *dst = (AT)r;
+    };
+    auto ld_part = [&](const float *po, int s) { return ld_coherent(po + (size_t)(s < n_active ? s : n_active - 1) * NREP * (HD + 2)); };
+    constexpr bool PAIRS = NREP * HD > NW * 64;              // more elements than threads: a thread has at least two
+    for (int i0 = tid; i0 < NREP * HD; i0 += (PAIRS ? 2 : 1) * nthreads) {
+      const int i1 = i0 + nthreads;
+      const bool two = PAIRS && i1 < NREP * HD;
+      const int ja = i0 / HD, jb = (two ? i1 : i0) / HD;
+      const float *pa = base + (size_t)ja * (HD + 2) + i0 % HD, *pb = base + (size_t)jb * (HD + 2) + (two ? i1 : i0) % HD;
+      float parta[32], partb[32];
+#pragma unroll
+      for (int u = 0; u < 32; u++) parta[u] = ld_part(pa, u);
+      if constexpr (PAIRS) {
+#pragma unroll
+        for (int u = 0; u < 32; u++) partb[u] = ld_part(pb, u);
+      }
+      float Oa = 0.0f, Ob = 0.0f;
+#pragma unroll
+      for (int u = 0; u < 32; u++)
+        if (u < n_active) Oa = fmaf(parta[u], sm.sc[ja][u], Oa);
+      if constexpr (PAIRS) {
+#pragma unroll
+        for (int u = 0; u < 32; u++)
+          if (u < n_active) Ob = fmaf(partb[u], sm.sc[jb][u], Ob);
+      }
+      for (int s0 = 32; s0 < n_active; s0 += 32) {           // more than 32 chunks: the rest in batches, element by element
+#pragma unroll
+        for (int u = 0; u < 32; u++) parta[u] = ld_part(pa, s0 + u);
+#pragma unroll
+        for (int u = 0; u < 32; u++)
+          if (s0 + u < n_active) Oa = fmaf(parta[u], sm.sc[ja][s0 + u], Oa);
+        if constexpr (PAIRS) {
+#pragma unroll
+          for (int u = 0; u < 32; u++) partb[u] = ld_part(pb, s0 + u);
+#pragma unroll
+          for (int u = 0; u < 32; u++)
+            if (s0 + u < n_active) Ob = fmaf(partb[u], sm.sc[jb][s0 + u], Ob);
+        }
+      }
+      finish(i0, Oa);
+      if (two) finish(i1, Ob);
     }
     if (tid == 0) __hip_atomic_store(&a.counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }

@@ -29,18 +29,20 @@ __global__ __launch_bounds__(AW_THREADS) void attn_wo_kernel(AttnArgs at, GemvAr
   __shared__ float red[8];
   __shared__ float lut[16];
 
-  const int pos = at.st[1];
-  // the version of this launch: no other launch that writes the same tagged row has it (another layer, or another
-  // position of the same layer; a model has at least two layers here)
-  const uint32_t tag = tw_tag(pos * 128 + layer);
-  at.out_tag = tag;
-  a.x_tag = tag;
+  const int pos = at.st[1];   // asked for first, waited for after the weight requests below are out
 
   // this wavefront's first wo item, requested before anything else
   GemvBuf buf;
   const int wave = threadIdx.x >> 6, grp = blockIdx.x * (AW_THREADS / 64) + wave;
   const bool preloaded = grp < G::ngroups(a);
   if (preloaded) G::load_item(a, buf, grp, 0, 0);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // the version of this launch: no other launch that writes the same tagged row has it (another layer, or another
+  // position of the same layer; a model has at least two layers here)
+  const uint32_t tag = tw_tag(pos * 128 + layer);
+  at.out_tag = tag;
+  a.x_tag = tag;
 
   if (pos >= 0 && pos < at.max_context) {
     const int T = pos + 1;
