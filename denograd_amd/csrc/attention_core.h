@@ -140,17 +140,46 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
         if (t < t1) score_row(raw[i], t);
       }
     }
-    __syncthreads();
-    if (CH <= 64 && NREP <= NW) {
-      // A short chunk (the usual case for one sequence): the scores of a head fit one wavefront, lane i holding row i, so
-      // wavefront j does the whole softmax of head j by itself - maximum, exp, sum - with no barrier in between.
+    // A chunk with more rows than the requests sent up front cover (several sequences, long contexts): the first batch of V
+    // rows is requested now, so that it travels while the softmax is computed.  The two barriers around the softmax wait
+    // for LDS traffic only; __syncthreads() would also wait for these requests.
+    const int tb_v = t0 + (wave + NPRE * NW) * RPI + grp;
+    const bool more_v = CH > NPRE * NW * RPI;              // the same for the whole block
+    u4_t vbat[NBATCH];
+    if (more_v) {
+#pragma unroll
+      for (int i = 0; i < NBATCH; i++) {
+        const int t = tb_v + i * NW * RPI;
+        vbat[i] = *(const u4_t *)(vbase + (size_t)(t < t1 ? t : t1 - 1) * row_stride);
+      }
+    }
+    lds_barrier();
+    if (NREP <= NW) {
+      // Wavefront j does the whole softmax of head j by itself - maximum, exp, sum - with no barrier in between: lane i holds
+      // rows i, i + 64, ... of the chunk (one row per lane for the short chunks of a single sequence).
       if (wave < NREP) {
         const int j = wave;
-        const float s = lane < CH ? sm.sc[j][lane] : -INFINITY;
-        const float m = wave_max(s);
-        const float e = lane < CH ? exp_f32(s - m) : 0.0f;
-        if (lane < CH) sm.sc[j][lane] = e;
-        const float l = wave_sum(e);
+        constexpr int PL = ATT_CHUNK_MAX / 64;
+        float sv[PL];
+        float m = -INFINITY;
+#pragma unroll
+        for (int q = 0; q < PL; q++) {
+          const int i = lane + 64 * q;
+          sv[q] = (q * 64 < CH && i < CH) ? sm.sc[j][i] : -INFINITY;
+          m = fmaxf(m, sv[q]);
+        }
+        m = wave_max(m);
+        float l = 0.0f;
+#pragma unroll
+        for (int q = 0; q < PL; q++) {
+          const int i = lane + 64 * q;
+          if (q * 64 < CH) {      // the same for the whole wavefront
+            const float e = i < CH ? exp_f32(sv[q] - m) : 0.0f;
+            if (i < CH) sm.sc[j][i] = e;
+            l += e;
+          }
+        }
+        l = wave_sum(l);
         if (lane == 0) { sm.m_sh[j] = m; sm.l_sh[j] = l; }
       }
     } else {
@@ -201,7 +230,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       // the barrier below also orders the in-place exp writes before phase 2 reads them
     }
     }
-    __syncthreads();
+    lds_barrier();
 
     // ---- phase 2: o[j][d] = sum_t p[j][t] * V[t][d]
     float of[NREP][EPL];
@@ -230,7 +259,14 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       const int t = t0 + (wave + i * NW) * RPI + grp;
       if (t < t1) pv_row(vpre[i], t);
     }
-    for (int tb = t0 + (wave + NPRE * NW) * RPI + grp; tb < t1; tb += NBATCH * NW * RPI) {
+    if (more_v) {
+#pragma unroll
+      for (int i = 0; i < NBATCH; i++) {
+        const int t = tb_v + i * NW * RPI;
+        if (t < t1) pv_row(vbat[i], t);
+      }
+    }
+    for (int tb = tb_v + NBATCH * NW * RPI; tb < t1; tb += NBATCH * NW * RPI) {
       u4_t raw[NBATCH];
 #pragma unroll
       for (int i = 0; i < NBATCH; i++) {

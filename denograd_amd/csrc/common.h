@@ -112,6 +112,11 @@ __device__ __forceinline__ _Float16 ld_coherent(const _Float16 *p) {
 __device__ __forceinline__ float ld_coherent(const float *p) { return __hip_atomic_load(as_global<float>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ int ld_coherent(const int *p) { return __hip_atomic_load(as_global<int>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
+// A block barrier that waits for the wavefront's LDS traffic only.  __syncthreads() also waits for every global load the
+// wavefront has in flight (the counter that tracks loads tracks stores too, and a barrier publishes stores), which ends
+// any prefetch at the barrier.  Use where only LDS contents must be agreed on.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // DPP cross-lane moves inside a 64-lane wavefront
 template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
