@@ -119,15 +119,34 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
         if (sub == 0) sm.sc[j][t - t0] = p * a.scale;
       }
     };
+    // a chunk with more rows than the up-front requests cover: its first batch of K rows is asked for before the first
+    // scores are computed
+    const int tb_v = t0 + (wave + NPRE * NW) * RPI + grp;
+    const bool more_v = CH > NPRE * NW * RPI;              // the same for the whole block
+    constexpr int NBATCH = 8;
+    u4_t kbat[NBATCH];
+    if (more_v) {
+#pragma unroll
+      for (int i = 0; i < NBATCH; i++) {
+        const int t = tb_v + i * NW * RPI;
+        kbat[i] = *(const u4_t *)(kbase + (size_t)(t < t1 ? t : t1 - 1) * row_stride);
+      }
+    }
 #pragma unroll
     for (int i = 0; i < NPRE; i++) {
       const int t = t0 + (wave + i * NW) * RPI + grp;
       if (t < t1) score_row(kpre[i], t);
     }
-    // longer chunks (several sequences per launch, long contexts): the remaining rows in batches of NBATCH requests, so that
-    // an iteration does not wait a round trip of its own
-    constexpr int NBATCH = 8;
-    for (int tb = t0 + (wave + NPRE * NW) * RPI + grp; tb < t1; tb += NBATCH * NW * RPI) {
+    if (more_v) {
+#pragma unroll
+      for (int i = 0; i < NBATCH; i++) {
+        const int t = tb_v + i * NW * RPI;
+        if (t < t1) score_row(kbat[i], t);
+      }
+    }
+    // still longer chunks: the remaining rows in batches of NBATCH requests, so that an iteration does not wait a round trip
+    // of its own
+    for (int tb = tb_v + NBATCH * NW * RPI; tb < t1; tb += NBATCH * NW * RPI) {
       u4_t raw[NBATCH];
 #pragma unroll
       for (int i = 0; i < NBATCH; i++) {
@@ -143,8 +162,6 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
     // A chunk with more rows than the requests sent up front cover (several sequences, long contexts): the first batch of V
     // rows is requested now, so that it travels while the softmax is computed.  The two barriers around the softmax wait
     // for LDS traffic only; __syncthreads() would also wait for these requests.
-    const int tb_v = t0 + (wave + NPRE * NW) * RPI + grp;
-    const bool more_v = CH > NPRE * NW * RPI;              // the same for the whole block
     u4_t vbat[NBATCH];
     if (more_v) {
 #pragma unroll
