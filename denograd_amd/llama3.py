@@ -5,7 +5,7 @@ Int8Linear / Int8Embedding / NF4Linear keep the reference's storage (int8 codes 
 row; two 4-bit codes per byte + one fp16 scale per 64 elements) and its quantisers; `call` runs the fused
 dequantising GEMV.  Llama3 drives a Transformer the way the reference does: token-serial prefill, greedy
 decode, per-token `.item()`; `generate` is the free-running variant that keeps the token on the device.
-Downloading checkpoints and the tokenizer are out of scope here: a model is built from a state dict
+Downloading checkpoints is out of scope here: a model is built from a state dict
 (host arrays), a checkpoint file (.safetensors in the model's or in Hugging Face names, a .safetensors.index.json, a
 .gguf with F32 / F16 / Q4_0 / Q4_1 / Q8_0 / Q6_K tensors), or seeded random-init weights made on the device.
 """
@@ -129,6 +129,7 @@ class Llama3:
                                  self.linear, self.embedding, params.get("n_kv_heads"), params["rope_theta"], self.max_context, True, device=device,
                                  fused_step=fused_step)
         self.start_pos = 0
+        self.tokenizer = None                  # set by load_tokenizer
         self.last_seen_toks: list[int] = []
         # False: prompts are fed one token per call, as the reference does (llama3.ts:307-311).  True: the prompt is one
         # several-position call (matrix-core GEMMs + causal attention), the reference's Transformer.forward on [1, S]
@@ -243,6 +244,44 @@ class Llama3:
         for tok in toks:
             self._call(tok)
             self.start_pos += 1
+
+    # ---- text in, text out (llama3.ts:257-296)
+    def load_tokenizer(self, path: str) -> "Llama3":
+        """llama3.ts:257: the `tokenizer.model` next to the checkpoint."""
+        from .tokenizer import Tokenizer
+        self.tokenizer = Tokenizer.llama(path)
+        return self
+
+    def _system(self, msg: str = "You are an helpful assistant.") -> None:
+        """llama3.ts:266-269: begin_of_text and the system message, fed once; a later chat continues from there."""
+        self._prefill([self.tokenizer.bos_id, *self.tokenizer.encode_message("system", msg)])
+
+    def chat(self, messages: list[dict], on_token=None, max_new_tokens: int | None = None) -> dict:
+        """llama3.ts:270-296: frame the messages, prefill all but the last prompt token, then decode token by token (with the
+        sampler settings of this Llama3) until a stop token.  `max_new_tokens` (not in the reference, which only stops at a
+        stop token) bounds the loop; it also stops when the KV cache is full.  Returns the reference's response fields."""
+        tk = self.tokenizer
+        toks = [t for m in messages for t in tk.encode_message(m["role"], m["content"])] + tk.encode_role("assistant")
+        st = time.perf_counter()
+        self._prefill(toks[:-1])
+        ttft = time.perf_counter() - st
+        last, content = toks[-1], ""
+        usage = {"input_tokens": len(toks) - 1, "time_to_first_token": ttft, "output_tokens": 0, "tokens_per_second": 0.0}
+        st = time.perf_counter()
+        while True:
+            if self.start_pos >= self.max_context or (max_new_tokens is not None and usage["output_tokens"] >= max_new_tokens):
+                return {"stop_reason": "max_tokens", "message": {"role": "assistant", "content": content}, "usage": usage}
+            tok = self._call(last)
+            self.start_pos += 1
+            usage["output_tokens"] += 1
+            usage["tokens_per_second"] = usage["output_tokens"] / (time.perf_counter() - st)
+            last = tok
+            if tok in tk.stop_tokens:
+                return {"stop_reason": "end_turn", "message": {"role": "assistant", "content": content}, "usage": usage}
+            piece = tk.decode([tok])
+            content += piece
+            if on_token is not None:
+                on_token({"message": {"role": "assistant", "content": content}, "usage": usage, "token": piece})
 
     def chat_tokens(self, toks: list[int], max_new_tokens: int, stop_tokens=()) -> dict:
         """The loop of Llama3.chat (llama3.ts:270-296) on token ids: prefill all but the last prompt token, then decode
