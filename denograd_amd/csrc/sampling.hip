@@ -8,7 +8,7 @@
 // literally - ((x0 + x1) + x2) + ... - so a chunk is one block whose thread j adds up elements 0..j of the chunk out of
 // LDS, and the sums over chunk totals are loops of one thread.  The plain sums (softmax denominator, the mass left after
 // top-k) use the same chunks: sequential inside, then sequential over the chunk sums.  With that the token is a function
-// of (logits, parameters, random word) alone and equals the numpy restatement's bit for bit.
+// of (logits, parameters, random word) alone: any evaluation that adds in this order gets the same bits.
 //
 // Four launches for the whole-vocabulary draw (chunk c of the padded vector = block c):
 //   prep  y = (logit - penalty, NaN -> -inf) * (1/temp); chunk maxima
