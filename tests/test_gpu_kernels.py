@@ -283,7 +283,7 @@ def test_attention_decode(hip, dt, H, KV, hd, ctx):
     assert np.all(ws.numpy()[:256] == 0)
 
 
-@pytest.mark.parametrize("kind,H,KV,hd,ctx", [("f16", 32, 8, 64, 1024), ("i8", 8, 2, 128, 4096), ("f16", 4, 4, 64, 96), ("i8", 24, 8, 128, 640)])
+@pytest.mark.parametrize("kind,H,KV,hd,ctx", [("f16", 32, 8, 64, 1024), ("i8", 8, 2, 128, 4096), ("f16", 4, 4, 64, 96), ("i8", 24, 8, 128, 640), ("f16", 8, 2, 64, 8192)])
 def test_attention_and_wo_in_one_launch(hip, kind, H, KV, hd, ctx):
     """jsgrad_hip_attn_wo == jsgrad_hip_attn_decode followed by jsgrad_hip_linear(wo, residual), bit for bit, for several T,
     two layers sharing one workspace (the version tag tells their rows apart), and no bounded wait ever running out."""
