@@ -10,16 +10,24 @@
 // Tiling: 256 threads = 4 wavefronts laid out WGM x WGN; a wavefront owns TM x TN tiles of 32x32 outputs and walks K in
 // steps of 16 with v_mfma_f32_32x32x16_f16.  Both operands are K-contiguous in memory (x rows, W rows), so a lane's
 // 8-element operand fragment is one 128-bit LDS read.  LDS rows are padded by 8 halves (144-byte stride), which
-// spreads the 32 rows of a fragment read over all banks.  One LDS buffer, register prefetch of the next K tile issued
-// before the MFMAs of the current one.  Tile ids are remapped so that the blocks resident on one XCD (round-robin by
-// block id) share operand tiles in that XCD's L2.
+// spreads the 32 rows of a fragment read over all banks.  The weight fragment is the first MFMA operand, so a lane ends up
+// with four neighbouring output columns of one output row per accumulator quad: 8-byte stores in the epilogue.
+//
+// Two loop shapes.  One LDS buffer (two barriers per K tile, the next tile prefetched into registers) with two or three
+// blocks per CU, whose wavefronts cover each other's barriers and conversions.  Two LDS buffers with one 256x256 block
+// per CU (one wavefront per SIMD): one barrier per K tile, and the instruction order of a K tile is spelled out so that
+// fragment reads, conversion, LDS writes and the requests of the tile after next sit between the matrix instructions.
+// Tile ids are remapped so that the blocks resident on one XCD (round-robin by block id) share operand tiles in that
+// XCD's L2.
 #include <stdlib.h>
+#include <string.h>
 
 #include "common.h"
 
 namespace jsg {
 
 typedef float f16_t __attribute__((ext_vector_type(16)));
+typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
 
 enum { GEPI_STORE = 0, GEPI_ROPE_KV = 1, GEPI_SWIGLU = 2 };
 
@@ -56,7 +64,7 @@ __device__ __forceinline__ void i8x4_to_h2x2(uint32_t q, uint32_t &lo, uint32_t 
   hi = __builtin_bit_cast(uint32_t, b);
 }
 
-template <int KIND, int EPI, int WGM, int WGN, int TM, int TN>
+template <int KIND, int EPI, int WGM, int WGN, int TM, int TN, bool DB = false>
 __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 : 3))) void gemm_kernel(GemmArgs a) {
   static_assert(WGM * WGN == 4, "four wavefronts");
   static_assert(EPI != GEPI_SWIGLU || TN % 2 == 0, "a wavefront holds the w1 and the w3 tile of the same columns");
@@ -66,8 +74,9 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
   constexpr int B_CHUNKS = GEMM_THREADS / B_ROWS_PER_PASS;                             // 16-byte chunks per row of the K tile
   constexpr int B_LOADS = BN / B_ROWS_PER_PASS;
   static_assert(B_LOADS >= 1, "tile too narrow for this weight format");
-  extern __shared__ __align__(16) _Float16 gemm_lds[];   // [BM + BN rows][LS], then the 16-entry NF4 table
-  _Float16 *As = gemm_lds, *Bs = gemm_lds + BM * LS, *lut = gemm_lds + (BM + BN) * LS;
+  constexpr int BUF = (BM + BN) * LS;                     // halves per LDS buffer
+  extern __shared__ __align__(16) _Float16 gemm_lds[];   // one or two buffers of [BM + BN rows][LS], then the 16-entry NF4 table
+  _Float16 *As = gemm_lds, *Bs = gemm_lds + BM * LS, *lut = gemm_lds + (DB ? 2 : 1) * BUF;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WGN, wn = wave % WGN;
@@ -146,12 +155,12 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
       else { gb[i] = *(const u4_t *)(bsrc[i] + ko / 2); gs[i] = bscale_ptr[i][kt]; }
     }
   };
-  auto commit = [&]() {
+  auto commit = [&](int buf = 0) {
 #pragma unroll
-    for (int i = 0; i < A_LOADS; i++) *(u4_t *)&As[(arow_t + i * 32) * LS + achunk * 8] = ga[i];
+    for (int i = 0; i < A_LOADS; i++) *(u4_t *)&As[buf * BUF + (arow_t + i * 32) * LS + achunk * 8] = ga[i];
 #pragma unroll
     for (int i = 0; i < B_LOADS; i++) {
-      _Float16 *dst = &Bs[(brow_t + i * B_ROWS_PER_PASS) * LS];
+      _Float16 *dst = &Bs[buf * BUF + (brow_t + i * B_ROWS_PER_PASS) * LS];
       if constexpr (KIND == JSGRAD_W_F16) *(u4_t *)(dst + bchunk * 8) = gb[i];
       else if constexpr (KIND == JSGRAD_W_I8) {
         u4_t o0, o1;
@@ -184,90 +193,162 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
     }
   };
 
+  auto frags = [&](int buf, int kk, h8_t *af, h8_t *bf) {
+#pragma unroll
+    for (int i = 0; i < TM; i++) af[i] = *(const h8_t *)&As[buf * BUF + ((wm * TM + i) * 32 + l32) * LS + kk * 16 + lg * 8];
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      int rbase;
+      if constexpr (EPI == GEPI_SWIGLU) rbase = j < TN / 2 ? (wn * (TN / 2) + j) * 32 : BN / 2 + (wn * (TN / 2) + j - TN / 2) * 32;
+      else rbase = (wn * TN + j) * 32;
+      bf[j] = *(const h8_t *)&Bs[buf * BUF + (rbase + l32) * LS + kk * 16 + lg * 8];
+    }
+  };
+  auto mfmas = [&](const h8_t *af, const h8_t *bf) {
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);   // D = W tile . x tile^T
+  };
+
   const int nk = a.K / GEMM_BK;
   issue(0);
   if constexpr (KIND == JSGRAD_W_NF4) __syncthreads();   // the code table is in LDS
-  for (int kt = 0; kt < nk; kt++) {
-    commit();
-    __syncthreads();
-    if (kt + 1 < nk) issue(kt + 1);
+  if constexpr (DB) {
+    // Two LDS buffers, one barrier per K tile: while the matrix cores work on tile kt out of one buffer, the same
+    // wavefront turns the registers of tile kt+1 into the other buffer and requests tile kt+2.  The barrier waits for LDS
+    // traffic only, so the requests stay in flight across it.  The buffer written during tile kt is the one read during
+    // tile kt-1: every wavefront finished those reads before it passed the barrier that ended kt-1.
+    commit(0);
+    if (nk > 1) issue(1);
+    lds_barrier();
+    for (int kt = 0; kt < nk; kt++) {
+      const int cur = kt & 1;
+      h8_t af[2][TM], bf[2][TN];
+      frags(cur, 0, af[0], bf[0]);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int kk = 0; kk < GEMM_BK / 16; kk++) {
-      h8_t af[TM], bf[TN];
+      for (int kk = 0; kk < GEMM_BK / 16; kk++) {
+        if (kk + 1 < GEMM_BK / 16) frags(cur, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+        // past the last tile both still run (the last tile again, into the buffer nobody reads any more): one
+        // straight-line loop body
+        if (kk == 1) commit(cur ^ 1);
+        if (kk == 2) issue(min(kt + 2, nk - 1));
+        mfmas(af[kk & 1], bf[kk & 1]);
+        // The order inside this K step, spelled out for the instruction scheduler: every matrix instruction is followed by
+        // a share of the other work of the step (fragment reads of the next step, the conversion and LDS writes of the
+        // next tile, the requests of the tile after it), so that work runs while the matrix core is busy.  Left alone the
+        // scheduler puts each fragment read directly before its first use and waits out the LDS latency every time.
 #pragma unroll
-      for (int i = 0; i < TM; i++) af[i] = *(const h8_t *)&As[((wm * TM + i) * 32 + l32) * LS + kk * 16 + lg * 8];
-#pragma unroll
-      for (int j = 0; j < TN; j++) {
-        int rbase;
-        if constexpr (EPI == GEPI_SWIGLU) rbase = j < TN / 2 ? (wn * (TN / 2) + j) * 32 : BN / 2 + (wn * (TN / 2) + j - TN / 2) * 32;
-        else rbase = (wn * TN + j) * 32;
-        bf[j] = *(const h8_t *)&Bs[(rbase + l32) * LS + kk * 16 + lg * 8];
+        for (int i = 0; i < TM * TN; i++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                           // one MFMA
+          if (kk + 1 < GEMM_BK / 16 && i < TM + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+          if (kk == 1) {
+            __builtin_amdgcn_sched_group_barrier(0x002, KIND == JSGRAD_W_F16 ? 1 : (KIND == JSGRAD_W_I8 ? 8 : 12), 0);
+            __builtin_amdgcn_sched_group_barrier(0x200, KIND == JSGRAD_W_NF4 ? 2 : 1, 0);
+            if constexpr (KIND == JSGRAD_W_NF4) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);      // table look-ups
+          }
+          if (kk == 2) {
+            __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
-#pragma unroll
-      for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+      lds_barrier();
     }
-    __syncthreads();
+  } else {
+    for (int kt = 0; kt < nk; kt++) {
+      commit();
+      __syncthreads();
+      if (kt + 1 < nk) issue(kt + 1);
+#pragma unroll
+      for (int kk = 0; kk < GEMM_BK / 16; kk++) {
+        h8_t af[TM], bf[TN];
+        frags(0, kk, af, bf);
+        mfmas(af, bf);
+      }
+      __syncthreads();
+    }
   }
 
-  // ---- epilogue.  Accumulator r of a lane is output row 8*(r/4) + 4*(lane/32) + r%4, column lane%32 of the 32x32 tile.
+  // ---- epilogue.  The weight fragment is the first MFMA operand, so the 32x32 result tile is held transposed: a lane has
+  // input row (output row) m = lane % 32 and, in accumulators 4g .. 4g+3, the four neighbouring output columns
+  // 8g + 4 * (lane / 32) + 0..3.  Four fp16 results are one 8-byte store (and one 8-byte load of the residual), the 32
+  // columns of a tile are 64 contiguous bytes of the output row.
 #pragma unroll
   for (int i = 0; i < TM; i++) {
-    const int mbase = m0 + (wm * TM + i) * 32 + lg * 4;
+    const int m = m0 + (wm * TM + i) * 32 + l32;
+    if (m >= a.M) continue;
     if constexpr (EPI == GEPI_SWIGLU) {
 #pragma unroll
       for (int j = 0; j < TN / 2; j++) {
-        const int n = n0_out + (wn * (TN / 2) + j) * 32 + l32;
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const int m = mbase + 8 * (r / 4) + (r % 4);
-          if (m < a.M) {
+        for (int g = 0; g < 4; g++) {
+          const int n = n0_out + (wn * (TN / 2) + j) * 32 + 8 * g + 4 * lg;
+          h4_t o;
+#pragma unroll
+          for (int c = 0; c < 4; c++) {
             // silu(w1 x) * (w3 x), each GEMM output and the product stored as fp16 (llama.ts:108-110)
-            const float g = rn16(acc[i][j][r]), u = rn16(acc[i][j + TN / 2][r]);
-            a.y[(size_t)m * a.N + n] = (_Float16)(silu_act<_Float16>(g) * u);
+            const float gt = rn16(acc[i][j][4 * g + c]), up = rn16(acc[i][j + TN / 2][4 * g + c]);
+            o[c] = (_Float16)(silu_act<_Float16>(gt) * up);
           }
+          *(h4_t *)&a.y[(size_t)m * a.N + n] = o;
+        }
+      }
+    } else if constexpr (EPI == GEPI_STORE) {
+      h4_t res[TN][4];
+      if (a.residual) {
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int g = 0; g < 4; g++) res[j][g] = *(const h4_t *)&a.residual[(size_t)m * a.N + n0_out + (wn * TN + j) * 32 + 8 * g + 4 * lg];
+      }
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          const int n = n0_out + (wn * TN + j) * 32 + 8 * g + 4 * lg;
+          h4_t o;
+#pragma unroll
+          for (int c = 0; c < 4; c++) {
+            float v = rn16(acc[i][j][4 * g + c]);
+            if (a.residual) v = (float)res[j][g][c] + v;
+            o[c] = (_Float16)v;
+          }
+          *(h4_t *)&a.y[(size_t)m * a.N + n] = o;
         }
       }
     } else {
+      // wq | wk | wv columns; q and k get the interleaved-pair rotation (llama.ts:17-32), k and v go to the cache rows.
+      // Four neighbouring columns are two pairs of one head of one matrix (every boundary is a multiple of 4).
+      const int b = m / a.seq_len, pos = a.start_pos + m % a.seq_len;
 #pragma unroll
       for (int j = 0; j < TN; j++) {
-        const int n = n0_out + (wn * TN + j) * 32 + l32;
-        if constexpr (EPI == GEPI_STORE) {
 #pragma unroll
-          for (int r = 0; r < 16; r++) {
-            const int m = mbase + 8 * (r / 4) + (r % 4);
-            if (m < a.M) {
-              float v = rn16(acc[i][j][r]);
-              if (a.residual) v = (float)a.residual[(size_t)m * a.N + n] + v;
-              a.y[(size_t)m * a.N + n] = (_Float16)v;
-            }
-          }
-        } else {
-          // wq | wk | wv columns; q and k get the interleaved-pair rotation (llama.ts:17-32), k and v go to the cache rows
+        for (int g = 0; g < 4; g++) {
+          const int n = n0_out + (wn * TN + j) * 32 + 8 * g + 4 * lg;
           const int which = n < a.n0 ? 0 : (n < a.n0 + a.n1 ? 1 : 2);
           const int nl = which == 0 ? n : (which == 1 ? n - a.n0 : n - a.n0 - a.n1);
-          const int pair = (nl % a.head_dim) >> 1;
-          const bool odd = nl & 1;
+          h4_t o;
+          if (which < 2) {
+            const int pair = (nl % a.head_dim) >> 1;
+            const h4_t cs = *(const h4_t *)(a.rope_table + ((size_t)pos * (a.head_dim / 2) + pair) * 2);   // cos, sin of two pairs
 #pragma unroll
-          for (int r = 0; r < 16; r++) {
-            const int m = mbase + 8 * (r / 4) + (r % 4);
-            const float own = rn16(acc[i][j][r]);
-            const float other = dpp_f<0xB1>(own);              // the neighbouring column: the other half of the pair
-            if (m < a.M) {
-              const int b = m / a.seq_len, pos = a.start_pos + m % a.seq_len;
-              float v = own;
-              if (which < 2) {
-                const h2_t cs = *(const h2_t *)(a.rope_table + ((size_t)pos * (a.head_dim / 2) + pair) * 2);
-                const float c = (float)cs.x, d = (float)cs.y;
-                v = odd ? other * d + own * c : own * c - other * d;
-              }
-              if (which == 0) a.y[(size_t)m * a.n0 + nl] = (_Float16)v;
-              else {
-                _Float16 *cache = which == 1 ? a.cache_k : a.cache_v;
-                cache[((size_t)b * a.max_context + pos) * a.n1 + nl] = (_Float16)v;
-              }
+            for (int h = 0; h < 2; h++) {
+              const float ev = rn16(acc[i][j][4 * g + 2 * h]), od = rn16(acc[i][j][4 * g + 2 * h + 1]);
+              const float c = (float)cs[2 * h], d = (float)cs[2 * h + 1];
+              o[2 * h] = (_Float16)(ev * c - od * d);
+              o[2 * h + 1] = (_Float16)(ev * d + od * c);
             }
+          } else {
+#pragma unroll
+            for (int c = 0; c < 4; c++) o[c] = (_Float16)rn16(acc[i][j][4 * g + c]);
+          }
+          if (which == 0) *(h4_t *)&a.y[(size_t)m * a.n0 + nl] = o;
+          else {
+            _Float16 *cache = which == 1 ? a.cache_k : a.cache_v;
+            *(h4_t *)&cache[((size_t)b * a.max_context + pos) * a.n1 + nl] = o;
           }
         }
       }
@@ -563,35 +644,43 @@ template <int KIND, int EPI> static int dispatch_skinny(const GemmArgs &a, int p
   return two ? launch_skinny<KIND, EPI, 2, 2>(a, prof_kind) : launch_skinny<KIND, EPI, 2, 1>(a, prof_kind);
 }
 
-template <int KIND, int EPI, int WGM, int WGN, int TM, int TN> static int launch_gemm(const GemmArgs &a, int prof_kind) {
+template <int KIND, int EPI, int WGM, int WGN, int TM, int TN, bool DB = false> static int launch_gemm(const GemmArgs &a, int prof_kind) {
   constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
   const int out_per_tile = EPI == GEPI_SWIGLU ? BN / 2 : BN;
   const int tiles = ((a.M + BM - 1) / BM) * (a.N / out_per_tile);
-  constexpr size_t lds = (size_t)(BM + BN) * GEMM_LDS_STRIDE * sizeof(_Float16) + 32;
+  constexpr size_t lds = (size_t)(DB ? 2 : 1) * (BM + BN) * GEMM_LDS_STRIDE * sizeof(_Float16) + 32;
+  static_assert(lds <= 160 * 1024, "LDS of one compute unit");
   if constexpr (lds > 64 * 1024) {
     static bool raised = false;   // one process, one device, one thread: set once per instantiation
     if (!raised) {
-      JSG_HIP(hipFuncSetAttribute((const void *)gemm_kernel<KIND, EPI, WGM, WGN, TM, TN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      JSG_HIP(hipFuncSetAttribute((const void *)gemm_kernel<KIND, EPI, WGM, WGN, TM, TN, DB>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
       raised = true;
     }
   }
-  JSG_LAUNCH(prof_kind, (gemm_kernel<KIND, EPI, WGM, WGN, TM, TN>), dim3(tiles), dim3(GEMM_THREADS), lds, a);
+  JSG_LAUNCH(prof_kind, (gemm_kernel<KIND, EPI, WGM, WGN, TM, TN, DB>), dim3(tiles), dim3(GEMM_THREADS), lds, a);
   return 0;
 }
 
 template <int EPI> static int dispatch_gemm(int kind, const GemmArgs &a, int prof_kind) {
-  // tall inputs: 256x256 block tiles when the output is wide enough, else 256x128; short ones (batched decode): 32 rows
-  // x 128 columns per block
+  // tall inputs: 256x256 block tiles out of two LDS buffers when the output is wide enough (the NF4 conversion is too
+  // long to hide behind the matrix instructions of one wavefront per SIMD: it keeps the one-buffer shape with two
+  // blocks per CU), else 256x128; short ones (batched decode): 32 rows x 128 columns per block.
+  // JSG_GEMM_TILE pins a shape for tests and measurements: "db", "wide" (256x256, one buffer), "tall" (256x128), "small".
   const bool tall = a.M > 64;
   const int n_out = EPI == GEPI_SWIGLU ? 2 * a.N : a.N;
-  const bool wide = tall && getenv("JSG_GEMM_WIDE") && n_out % 256 == 0 && EPI != GEPI_ROPE_KV;
+  const char *pin = getenv("JSG_GEMM_TILE");
+  const bool can256 = tall && n_out % 256 == 0;
+  const bool piped = can256 && (pin ? !strcmp(pin, "db") : kind != JSGRAD_W_NF4);
+  const bool wide = can256 && pin && !strcmp(pin, "wide");
+  const bool small = tall && pin && !strcmp(pin, "small");
   bool taken = false;
   if (kind == JSGRAD_W_F16) { const int rc = dispatch_skinny<JSGRAD_W_F16, EPI>(a, prof_kind, &taken); if (taken) return rc; }
   if (kind == JSGRAD_W_I8) { const int rc = dispatch_skinny<JSGRAD_W_I8, EPI>(a, prof_kind, &taken); if (taken) return rc; }
 #define JSG_CASE(K)                                                                                                    \
   case K:                                                                                                              \
+    if (piped) return launch_gemm<K, EPI, 2, 2, 4, 4, true>(a, prof_kind);                                            \
     if (wide) return launch_gemm<K, EPI, 2, 2, 4, 4>(a, prof_kind);                                                   \
-    if (tall && getenv("JSG_GEMM_SMALL")) return launch_gemm<K, EPI, 2, 2, 2, 2>(a, prof_kind);                       \
+    if (small) return launch_gemm<K, EPI, 2, 2, 2, 2>(a, prof_kind);                                                  \
     return tall ? launch_gemm<K, EPI, 2, 2, 4, 2>(a, prof_kind) : launch_gemm<K, EPI, 1, 4, 1, EPI == GEPI_SWIGLU ? 2 : 1>(a, prof_kind);
   switch (kind) {
     JSG_CASE(JSGRAD_W_F16)
@@ -604,6 +693,8 @@ template <int EPI> static int dispatch_gemm(int kind, const GemmArgs &a, int pro
 
 // largest column tile any configuration uses: output widths must be multiples of it
 constexpr int GEMM_N_ALIGN = 128;
+
+static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 static int check_gemm(const char *who, int kind, int rows, int in_f) {
   JSG_REQUIRE(kind == JSGRAD_W_F16 || kind == JSGRAD_W_I8 || kind == JSGRAD_W_NF4, "%s: weight kind %d is not built for several rows (fp16, int8 and nf4 are)", who, kind);
@@ -624,6 +715,7 @@ int jsgrad_hip_gemm(int kind, const void *w, const void *scale, int out_f, int i
   JSG_REQUIRE(w && x && y, "jsgrad_hip_gemm: null pointer argument");
   JSG_REQUIRE(kind == JSGRAD_W_F16 || scale, "jsgrad_hip_gemm: quantised weights need their scales");
   JSG_REQUIRE(out_f > 0 && out_f % GEMM_N_ALIGN == 0, "jsgrad_hip_gemm: out_features %d must be a positive multiple of %d", out_f, GEMM_N_ALIGN);
+  JSG_REQUIRE(aligned16(w) && aligned16(x) && aligned16(y) && aligned16(residual), "jsgrad_hip_gemm: w, x, y and residual must be 16-byte aligned");
   GemmArgs a = {};
   a.w0 = w; a.s0 = (const _Float16 *)scale; a.n0 = out_f;
   a.M = rows; a.N = out_f; a.K = in_f;
@@ -638,7 +730,9 @@ int jsgrad_hip_gemm_qkv_rope(int kind, const void *wq, const void *sq, const voi
   if (int rc = check_gemm("jsgrad_hip_gemm_qkv_rope", kind, rows, dim)) return rc;
   JSG_REQUIRE(wq && wk && wv && x && rope_table && q_out && cache_k && cache_v, "jsgrad_hip_gemm_qkv_rope: null pointer argument");
   JSG_REQUIRE(kind == JSGRAD_W_F16 || (sq && sk && sv), "jsgrad_hip_gemm_qkv_rope: quantised weights need their scales");
-  JSG_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && n_heads > 0 && n_kv_heads > 0, "jsgrad_hip_gemm_qkv_rope: bad head geometry");
+  JSG_REQUIRE(head_dim > 0 && head_dim % 4 == 0 && n_heads > 0 && n_kv_heads > 0, "jsgrad_hip_gemm_qkv_rope: bad head geometry (head_dim a multiple of 4)");
+  JSG_REQUIRE(aligned16(wq) && aligned16(wk) && aligned16(wv) && aligned16(x) && aligned16(rope_table) && aligned16(q_out) && aligned16(cache_k) && aligned16(cache_v),
+              "jsgrad_hip_gemm_qkv_rope: weights, x, rope_table, q_out and the caches must be 16-byte aligned");
   const int nq = n_heads * head_dim, nkv = n_kv_heads * head_dim;
   JSG_REQUIRE(nq % GEMM_N_ALIGN == 0 && nkv % GEMM_N_ALIGN == 0, "jsgrad_hip_gemm_qkv_rope: n_heads*head_dim %d and n_kv_heads*head_dim %d must be multiples of %d", nq, nkv,
               GEMM_N_ALIGN);
@@ -663,6 +757,7 @@ int jsgrad_hip_gemm_ffn_gate(int kind, const void *w1, const void *s1, const voi
   JSG_REQUIRE(w1 && w3 && x && y, "jsgrad_hip_gemm_ffn_gate: null pointer argument");
   JSG_REQUIRE(kind == JSGRAD_W_F16 || (s1 && s3), "jsgrad_hip_gemm_ffn_gate: quantised weights need their scales");
   JSG_REQUIRE(hidden > 0 && hidden % GEMM_N_ALIGN == 0, "jsgrad_hip_gemm_ffn_gate: hidden_dim %d must be a positive multiple of %d", hidden, GEMM_N_ALIGN);
+  JSG_REQUIRE(aligned16(w1) && aligned16(w3) && aligned16(x) && aligned16(y), "jsgrad_hip_gemm_ffn_gate: w1, w3, x and g must be 16-byte aligned");
   GemmArgs a = {};
   a.w0 = w1; a.w1 = w3; a.s0 = (const _Float16 *)s1; a.s1 = (const _Float16 *)s3;
   a.n0 = hidden; a.n1 = hidden;

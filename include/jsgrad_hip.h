@@ -154,7 +154,8 @@ int jsgrad_hip_argmax(const void *logits, int n, int32_t *state, int32_t *tokens
  * m = b*S + s sits at position start_pos + s of sequence b.  fp16 activations; fp16, int8 or NF4 weights.  With more
  * than one row the reference expands the weight over the rows, which realises a quantised weight in fp16 first
  * (W = RN16(code * scale)); the kernels below reproduce that.  Linear layers run on the matrix cores (MFMA) with
- * float accumulation.  Output widths must be multiples of 128, in_features multiples of 64.
+ * float accumulation.  Output widths must be multiples of 128, in_features multiples of 64; weights, activations,
+ * outputs, the rope table and the caches 16-byte aligned.
  * The KV cache of a layer is [B][max_context][n_kv_heads][head_dim] (models/llama.ts:78-80).
  * --------------------------------------------------------------------------------- */
 

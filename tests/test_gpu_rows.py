@@ -122,6 +122,39 @@ def test_few_rows_streaming_kernel_equals_tiled_kernel(hip, monkeypatch):
             assert (got["1"] == got["tiled"]).mean() > 0.97
 
 
+@pytest.mark.parametrize("kind", ["float16", "int8", "nf4"])
+def test_tile_shapes_of_the_tiled_kernel_agree_bit_for_bit(hip, monkeypatch, kind):
+    """Every block shape of the tiled kernel (256x256 out of two LDS buffers, 256x256 and 256x128 out of one, 128x128)
+    walks K in the same order, so the outputs are identical; 3 and 4 K tiles, a ragged last row tile, with a residual."""
+    for rows, out_f, in_f in ((300, 512, 192), (257, 256, 256)):
+        w, s = make_weight(kind, out_f, in_f)
+        x = RNG.standard_normal((rows, in_f)).astype(np.float16)
+        res = RNG.standard_normal((rows, out_f)).astype(np.float16)
+        tw, ts = dev(w, s)
+        tx, tr = Tensor(x), Tensor(res)
+        got = {}
+        for shape in ("db", "wide", "tall", "small"):
+            monkeypatch.setenv("JSG_GEMM_TILE", shape)
+            y = Tensor.empty((rows, out_f), "float16")
+            check(hip.jsgrad_hip_gemm(KINDS[kind], tw.ptr, sp(ts), out_f, in_f, tx.ptr, rows, y.ptr, tr.ptr))
+            got[shape] = y.numpy().view(np.uint16)
+        monkeypatch.delenv("JSG_GEMM_TILE")
+        ref = (res.astype(np.float32) + orc.linear(w, s, x, out_f, in_f, True)).astype(np.float16).astype(np.float32)
+        assert_close(got["db"].view(np.float16).astype(np.float32), ref, True, f"{kind} {rows}x{out_f}x{in_f}", composed=True)
+        for shape in ("wide", "tall", "small"):
+            assert np.array_equal(got["db"], got[shape]), f"{kind} {shape} {rows}x{out_f}x{in_f}"
+
+
+@pytest.mark.parametrize("shape", ["db", "wide", "tall", "small"])
+def test_tile_shapes_fused_epilogues(hip, monkeypatch, shape):
+    """SwiGLU and rotary / cache epilogues of the tiled kernel under every block shape."""
+    monkeypatch.setenv("JSG_GEMM_TILE", shape)
+    test_gemm_ffn_gate(hip, "int8", 130, 256, 384)
+    test_gemm_ffn_gate(hip, "nf4", 70, 128, 256)
+    test_gemm_qkv_rope_writes_queries_and_cache(hip, "float16", 64, 3, 40, 256)
+    test_gemm_qkv_rope_writes_queries_and_cache(hip, "int8", 128, 2, 50, 192)
+
+
 @pytest.mark.parametrize("tiles", ["1", "2"])
 def test_few_rows_fused_epilogues_with_one_and_two_tiles_per_block(hip, monkeypatch, tiles):
     """SwiGLU and rotary / cache epilogues of the weight-streaming kernel, tiles per block pinned."""
