@@ -22,6 +22,8 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace jsg {
@@ -144,10 +146,13 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
 
   u4_t ga[A_LOADS], gb[B_LOADS];
   _Float16 gs[B_LOADS];
-  auto issue = [&](int kt) {
+  auto issue_a = [&](int kt) {
     const size_t ko = (size_t)kt * GEMM_BK;
 #pragma unroll
     for (int i = 0; i < A_LOADS; i++) ga[i] = *(const u4_t *)(asrc[i] + ko * 2);
+  };
+  auto issue_b = [&](int kt) {
+    const size_t ko = (size_t)kt * GEMM_BK;
 #pragma unroll
     for (int i = 0; i < B_LOADS; i++) {
       if constexpr (KIND == JSGRAD_W_F16) gb[i] = *(const u4_t *)(bsrc[i] + ko * 2);
@@ -155,9 +160,12 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
       else { gb[i] = *(const u4_t *)(bsrc[i] + ko / 2); gs[i] = bscale_ptr[i][kt]; }
     }
   };
-  auto commit = [&](int buf = 0) {
+  auto issue = [&](int kt) { issue_a(kt); issue_b(kt); };
+  auto commit_a = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < A_LOADS; i++) *(u4_t *)&As[buf * BUF + (arow_t + i * 32) * LS + achunk * 8] = ga[i];
+  };
+  auto commit_b = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < B_LOADS; i++) {
       _Float16 *dst = &Bs[buf * BUF + (brow_t + i * B_ROWS_PER_PASS) * LS];
@@ -192,6 +200,7 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
       }
     }
   };
+  auto commit = [&](int buf = 0) { commit_a(buf); commit_b(buf); };
 
   auto frags = [&](int buf, int kk, h8_t *af, h8_t *bf) {
 #pragma unroll
@@ -216,46 +225,63 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
   if constexpr (KIND == JSGRAD_W_NF4) __syncthreads();   // the code table is in LDS
   if constexpr (DB) {
     // Two LDS buffers, one barrier per K tile: while the matrix cores work on tile kt out of one buffer, the same
-    // wavefront turns the registers of tile kt+1 into the other buffer and requests tile kt+2.  The barrier waits for LDS
-    // traffic only, so the requests stay in flight across it.  The buffer written during tile kt is the one read during
-    // tile kt-1: every wavefront finished those reads before it passed the barrier that ended kt-1.
+    // wavefront turns the registers of tile kt+1 into the other buffer and requests tile kt+2 into the registers just
+    // freed: the x half in K step 0, the weight half in K step 2, so every request has a whole tile's time to arrive
+    // and the requests of a CU (64 KiB per tile through a 64 B/clock L1) are spread over the tile.
+    // The barrier sits between K steps 2 and 3.  By then every wavefront has written its share of tile kt+1 and has
+    // read all fragments of tile kt (those of step 3 are read during step 2), so during step 3 the fragments of the
+    // first step of tile kt+1 are read and the matrix instructions run on across the end of the tile.  The buffer
+    // written during tile kt is the one read during tile kt-1, whose last reads precede the barrier of kt-1.  The
+    // barrier waits for LDS traffic only, so the requests stay in flight across it.
     commit(0);
     if (nk > 1) issue(1);
     lds_barrier();
+    h8_t af[2][TM], bf[2][TN];
+    frags(0, 0, af[0], bf[0]);
     for (int kt = 0; kt < nk; kt++) {
       const int cur = kt & 1;
-      h8_t af[2][TM], bf[2][TN];
-      frags(cur, 0, af[0], bf[0]);
+      const int after_next = min(kt + 2, nk - 1);   // past the last tile the same steps run on the last tile again, into
+                                                    // the buffer nobody computes from any more: a straight-line loop body
       __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int kk = 0; kk < GEMM_BK / 16; kk++) {
-        if (kk + 1 < GEMM_BK / 16) frags(cur, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
-        // past the last tile both still run (the last tile again, into the buffer nobody reads any more): one
-        // straight-line loop body
-        if (kk == 1) commit(cur ^ 1);
-        if (kk == 2) issue(min(kt + 2, nk - 1));
+      auto k_step = [&](auto KK) {
+        constexpr int kk = decltype(KK)::value;
+        constexpr int LAST = GEMM_BK / 16 - 1;
+        if (kk == LAST) lds_barrier();
+        if (kk < LAST) frags(cur, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+        else frags(cur ^ 1, 0, af[0], bf[0]);
+        if (kk == 0) { commit_a(cur ^ 1); issue_a(after_next); }
+        if (kk == 2) { commit_b(cur ^ 1); issue_b(after_next); }
         mfmas(af[kk & 1], bf[kk & 1]);
         // The order inside this K step, spelled out for the instruction scheduler: every matrix instruction is followed by
-        // a share of the other work of the step (fragment reads of the next step, the conversion and LDS writes of the
-        // next tile, the requests of the tile after it), so that work runs while the matrix core is busy.  Left alone the
+        // a share of the other work of the step (fragment reads of the next step, conversion and LDS writes of the next
+        // tile, then the requests of the tile after it), so that work runs while the matrix core is busy.  Left alone the
         // scheduler puts each fragment read directly before its first use and waits out the LDS latency every time.
+        constexpr int NMF = TM * TN;
+        constexpr int LOADS = kk == 0 ? A_LOADS : B_LOADS;
+        constexpr int WRITES = kk == 0 ? A_LOADS : (KIND == JSGRAD_W_F16 ? B_LOADS : (KIND == JSGRAD_W_I8 ? 2 * B_LOADS : 4 * B_LOADS));
+        constexpr int WSTEPS = NMF - (LOADS < NMF / 2 ? LOADS : NMF / 2);     // matrix instructions that carry the writes
 #pragma unroll
-        for (int i = 0; i < TM * TN; i++) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                           // one MFMA
-          if (kk + 1 < GEMM_BK / 16 && i < TM + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
-          if (kk == 1) {
-            __builtin_amdgcn_sched_group_barrier(0x002, KIND == JSGRAD_W_F16 ? 1 : (KIND == JSGRAD_W_I8 ? 8 : 12), 0);
-            __builtin_amdgcn_sched_group_barrier(0x200, KIND == JSGRAD_W_NF4 ? 2 : 1, 0);
-            if constexpr (KIND == JSGRAD_W_NF4) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);      // table look-ups
-          }
-          if (kk == 2) {
-            __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        for (int i = 0; i < NMF; i++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                          // one MFMA
+          if (i < TM + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);          // one LDS read
+          if (kk == 0 || kk == 2) {
+            if (i < WSTEPS) {
+              if (kk == 2 && KIND != JSGRAD_W_F16) __builtin_amdgcn_sched_group_barrier(0x002, KIND == JSGRAD_W_I8 ? 10 : 14, 0);
+              if constexpr (kk == 2 && KIND == JSGRAD_W_NF4) __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);   // table look-ups
+              __builtin_amdgcn_sched_group_barrier(0x200, (WRITES + WSTEPS - 1) / WSTEPS, 0);
+            } else {
+              __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+              __builtin_amdgcn_sched_group_barrier(0x020, (LOADS + NMF - WSTEPS - 1) / (NMF - WSTEPS), 0);
+            }
           }
         }
         __builtin_amdgcn_sched_barrier(0);
-      }
-      lds_barrier();
+      };
+      static_assert(GEMM_BK / 16 == 4, "four K steps per tile");
+      k_step(std::integral_constant<int, 0>{});
+      k_step(std::integral_constant<int, 1>{});
+      k_step(std::integral_constant<int, 2>{});
+      k_step(std::integral_constant<int, 3>{});
     }
   } else {
     for (int kt = 0; kt < nk; kt++) {
@@ -662,15 +688,14 @@ template <int KIND, int EPI, int WGM, int WGN, int TM, int TN, bool DB = false> 
 }
 
 template <int EPI> static int dispatch_gemm(int kind, const GemmArgs &a, int prof_kind) {
-  // tall inputs: 256x256 block tiles out of two LDS buffers when the output is wide enough (the NF4 conversion is too
-  // long to hide behind the matrix instructions of one wavefront per SIMD: it keeps the one-buffer shape with two
-  // blocks per CU), else 256x128; short ones (batched decode): 32 rows x 128 columns per block.
+  // tall inputs: 256x256 block tiles out of two LDS buffers when the output is wide enough, else 256x128 out of one; short
+  // ones (batched decode): 32 rows x 128 columns per block.
   // JSG_GEMM_TILE pins a shape for tests and measurements: "db", "wide" (256x256, one buffer), "tall" (256x128), "small".
   const bool tall = a.M > 64;
   const int n_out = EPI == GEPI_SWIGLU ? 2 * a.N : a.N;
   const char *pin = getenv("JSG_GEMM_TILE");
   const bool can256 = tall && n_out % 256 == 0;
-  const bool piped = can256 && (pin ? !strcmp(pin, "db") : kind != JSGRAD_W_NF4);
+  const bool piped = can256 && (!pin || !strcmp(pin, "db"));
   const bool wide = can256 && pin && !strcmp(pin, "wide");
   const bool small = tall && pin && !strcmp(pin, "small");
   bool taken = false;
