@@ -299,86 +299,82 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
   }
 
   // ---- epilogue.  The weight fragment is the first MFMA operand, so the 32x32 result tile is held transposed: a lane has
-  // input row (output row) m = lane % 32 and, in accumulators 4g .. 4g+3, the four neighbouring output columns
-  // 8g + 4 * (lane / 32) + 0..3.  Four fp16 results are one 8-byte store (and one 8-byte load of the residual), the 32
-  // columns of a tile are 64 contiguous bytes of the output row.
+  // output row m = lane % 32 and, in accumulators 4g .. 4g+3, the four neighbouring output columns 8g + 4 * (lane / 32) + 0..3.
+  // Stored from there, one instruction would touch 32 output rows with 8 bytes each.  Instead every wavefront turns 32 rows
+  // x its CW columns at a time through its own piece of LDS (free after the K loop; rows padded by 8 bytes, which spreads
+  // the 8-byte writes of 16 rows over all banks) and reads them back as 16-byte pieces along the rows: a store instruction
+  // then covers whole cache lines, and so do the loads of the residual and of the rope table.
+  constexpr int TNE = EPI == GEPI_SWIGLU ? TN / 2 : TN;   // 32-column tiles of output per wavefront and row tile
+  constexpr int CW = TNE * 32, RS = CW + 4;               // columns per wavefront; halves per LDS row
+  constexpr int CPR = CW / 8;                             // 16-byte pieces per row
+  static_assert((size_t)4 * 32 * RS <= (size_t)(BM + BN) * LS, "the transposing pieces fit the K-loop buffer");
+  __syncthreads();                                        // every wavefront is done with the K-loop buffers
+  _Float16 *ep = gemm_lds + wave * 32 * RS;
+  const int ncol0 = n0_out + wn * CW;                     // first output column of this wavefront
 #pragma unroll
   for (int i = 0; i < TM; i++) {
-    const int m = m0 + (wm * TM + i) * 32 + l32;
-    if (m >= a.M) continue;
-    if constexpr (EPI == GEPI_SWIGLU) {
 #pragma unroll
-      for (int j = 0; j < TN / 2; j++) {
+    for (int j = 0; j < TNE; j++) {
 #pragma unroll
-        for (int g = 0; g < 4; g++) {
-          const int n = n0_out + (wn * (TN / 2) + j) * 32 + 8 * g + 4 * lg;
-          h4_t o;
+      for (int g = 0; g < 4; g++) {
+        h4_t o;
 #pragma unroll
-          for (int c = 0; c < 4; c++) {
+        for (int c = 0; c < 4; c++) {
+          if constexpr (EPI == GEPI_SWIGLU) {
             // silu(w1 x) * (w3 x), each GEMM output and the product stored as fp16 (llama.ts:108-110)
             const float gt = rn16(acc[i][j][4 * g + c]), up = rn16(acc[i][j + TN / 2][4 * g + c]);
             o[c] = (_Float16)(silu_act<_Float16>(gt) * up);
-          }
-          *(h4_t *)&a.y[(size_t)m * a.N + n] = o;
-        }
-      }
-    } else if constexpr (EPI == GEPI_STORE) {
-      h4_t res[TN][4];
-      if (a.residual) {
-#pragma unroll
-        for (int j = 0; j < TN; j++)
-#pragma unroll
-          for (int g = 0; g < 4; g++) res[j][g] = *(const h4_t *)&a.residual[(size_t)m * a.N + n0_out + (wn * TN + j) * 32 + 8 * g + 4 * lg];
-      }
-#pragma unroll
-      for (int j = 0; j < TN; j++) {
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-          const int n = n0_out + (wn * TN + j) * 32 + 8 * g + 4 * lg;
-          h4_t o;
-#pragma unroll
-          for (int c = 0; c < 4; c++) {
-            float v = rn16(acc[i][j][4 * g + c]);
-            if (a.residual) v = (float)res[j][g][c] + v;
-            o[c] = (_Float16)v;
-          }
-          *(h4_t *)&a.y[(size_t)m * a.N + n] = o;
-        }
-      }
-    } else {
-      // wq | wk | wv columns; q and k get the interleaved-pair rotation (llama.ts:17-32), k and v go to the cache rows.
-      // Four neighbouring columns are two pairs of one head of one matrix (every boundary is a multiple of 4).
-      const int b = m / a.seq_len, pos = a.start_pos + m % a.seq_len;
-#pragma unroll
-      for (int j = 0; j < TN; j++) {
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-          const int n = n0_out + (wn * TN + j) * 32 + 8 * g + 4 * lg;
-          const int which = n < a.n0 ? 0 : (n < a.n0 + a.n1 ? 1 : 2);
-          const int nl = which == 0 ? n : (which == 1 ? n - a.n0 : n - a.n0 - a.n1);
-          h4_t o;
-          if (which < 2) {
-            const int pair = (nl % a.head_dim) >> 1;
-            const h4_t cs = *(const h4_t *)(a.rope_table + ((size_t)pos * (a.head_dim / 2) + pair) * 2);   // cos, sin of two pairs
-#pragma unroll
-            for (int h = 0; h < 2; h++) {
-              const float ev = rn16(acc[i][j][4 * g + 2 * h]), od = rn16(acc[i][j][4 * g + 2 * h + 1]);
-              const float c = (float)cs[2 * h], d = (float)cs[2 * h + 1];
-              o[2 * h] = (_Float16)(ev * c - od * d);
-              o[2 * h + 1] = (_Float16)(ev * d + od * c);
-            }
           } else {
+            o[c] = (_Float16)acc[i][j][4 * g + c];
+          }
+        }
+        *(h4_t *)&ep[l32 * RS + j * 32 + 8 * g + 4 * lg] = o;
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wavefront's own writes, before its own reads
+    const int mrow0 = m0 + (wm * TM + i) * 32;
 #pragma unroll
-            for (int c = 0; c < 4; c++) o[c] = (_Float16)rn16(acc[i][j][4 * g + c]);
+    for (int p = 0; p < 2 * TNE; p++) {
+      const int q = p * 64 + lane, row = q / CPR, piece = q % CPR;
+      const int m = mrow0 + row, n = ncol0 + piece * 8;
+      const h8_t v = *(const h8_t *)&ep[row * RS + piece * 8];
+      if (m >= a.M) continue;
+      if constexpr (EPI == GEPI_SWIGLU) {
+        *(h8_t *)&a.y[(size_t)m * a.N + n] = v;
+      } else if constexpr (EPI == GEPI_STORE) {
+        h8_t o = v;
+        if (a.residual) {
+          const h8_t res = *(const h8_t *)&a.residual[(size_t)m * a.N + n];
+#pragma unroll
+          for (int c = 0; c < 8; c++) o[c] = (_Float16)((float)res[c] + (float)v[c]);
+        }
+        *(h8_t *)&a.y[(size_t)m * a.N + n] = o;
+      } else {
+        // wq | wk | wv columns; q and k get the interleaved-pair rotation (llama.ts:17-32), k and v go to the cache rows.
+        // Eight neighbouring columns are four pairs of one head of one matrix (every boundary is a multiple of 8).
+        const int b = m / a.seq_len, pos = a.start_pos + m % a.seq_len;
+        const int which = n < a.n0 ? 0 : (n < a.n0 + a.n1 ? 1 : 2);
+        const int nl = which == 0 ? n : (which == 1 ? n - a.n0 : n - a.n0 - a.n1);
+        h8_t o = v;
+        if (which < 2) {
+          const int pair = (nl % a.head_dim) >> 1;
+          const h8_t cs = *(const h8_t *)(a.rope_table + ((size_t)pos * (a.head_dim / 2) + pair) * 2);   // cos, sin of four pairs
+#pragma unroll
+          for (int h = 0; h < 4; h++) {
+            const float ev = (float)v[2 * h], od = (float)v[2 * h + 1];
+            const float c = (float)cs[2 * h], d = (float)cs[2 * h + 1];
+            o[2 * h] = (_Float16)(ev * c - od * d);
+            o[2 * h + 1] = (_Float16)(ev * d + od * c);
           }
-          if (which == 0) *(h4_t *)&a.y[(size_t)m * a.n0 + nl] = o;
-          else {
-            _Float16 *cache = which == 1 ? a.cache_k : a.cache_v;
-            *(h4_t *)&cache[((size_t)b * a.max_context + pos) * a.n1 + nl] = o;
-          }
+        }
+        if (which == 0) *(h8_t *)&a.y[(size_t)m * a.n0 + nl] = o;
+        else {
+          _Float16 *cache = which == 1 ? a.cache_k : a.cache_v;
+          *(h8_t *)&cache[((size_t)b * a.max_context + pos) * a.n1 + nl] = o;
         }
       }
     }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the reads, before the next row tile overwrites the piece
   }
 }
 
@@ -755,7 +751,7 @@ int jsgrad_hip_gemm_qkv_rope(int kind, const void *wq, const void *sq, const voi
   if (int rc = check_gemm("jsgrad_hip_gemm_qkv_rope", kind, rows, dim)) return rc;
   JSG_REQUIRE(wq && wk && wv && x && rope_table && q_out && cache_k && cache_v, "jsgrad_hip_gemm_qkv_rope: null pointer argument");
   JSG_REQUIRE(kind == JSGRAD_W_F16 || (sq && sk && sv), "jsgrad_hip_gemm_qkv_rope: quantised weights need their scales");
-  JSG_REQUIRE(head_dim > 0 && head_dim % 4 == 0 && n_heads > 0 && n_kv_heads > 0, "jsgrad_hip_gemm_qkv_rope: bad head geometry (head_dim a multiple of 4)");
+  JSG_REQUIRE(head_dim > 0 && head_dim % 8 == 0 && n_heads > 0 && n_kv_heads > 0, "jsgrad_hip_gemm_qkv_rope: bad head geometry (head_dim a multiple of 8)");
   JSG_REQUIRE(aligned16(wq) && aligned16(wk) && aligned16(wv) && aligned16(x) && aligned16(rope_table) && aligned16(q_out) && aligned16(cache_k) && aligned16(cache_v),
               "jsgrad_hip_gemm_qkv_rope: weights, x, rope_table, q_out and the caches must be 16-byte aligned");
   const int nq = n_heads * head_dim, nkv = n_kv_heads * head_dim;
