@@ -351,7 +351,8 @@ def run_batched(name, bsz, prompt_len, steps):
                             "traffic": None},
                "kernels": pre_kinds}
 
-    # batched decode: one position per sequence per step
+    # batched decode: one position per sequence per step (4 warm-up steps, the timed ones, 4 profiled ones)
+    steps = max(steps, 9)
     pos = prompt_len
     for _ in range(4):
         tok = m.forward_rows(tok, pos); pos += 1
