@@ -308,9 +308,25 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
   constexpr int CW = TNE * 32, RS = CW + 4;               // columns per wavefront; halves per LDS row
   constexpr int CPR = CW / 8;                             // 16-byte pieces per row
   static_assert((size_t)4 * 32 * RS <= (size_t)(BM + BN) * LS, "the transposing pieces fit the K-loop buffer");
-  __syncthreads();                                        // every wavefront is done with the K-loop buffers
   _Float16 *ep = gemm_lds + wave * 32 * RS;
   const int ncol0 = n0_out + wn * CW;                     // first output column of this wavefront
+  // the residual of the whole wavefront tile is requested at once (the registers of the K loop are free): one trip to
+  // memory instead of one per 32 rows
+  h8_t res[EPI == GEPI_STORE ? TM : 1][EPI == GEPI_STORE ? 2 * TNE : 1];
+  if constexpr (EPI == GEPI_STORE) {
+    if (a.residual) {
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int p = 0; p < 2 * TNE; p++) {
+          const int q = p * 64 + lane, row = q / CPR, piece = q % CPR;
+          int m = m0 + (wm * TM + i) * 32 + row;
+          if (m >= a.M) m = a.M - 1;
+          res[i][p] = *(const h8_t *)&a.residual[(size_t)m * a.N + ncol0 + piece * 8];
+        }
+    }
+  }
+  __syncthreads();                                        // every wavefront is done with the K-loop buffers
 #pragma unroll
   for (int i = 0; i < TM; i++) {
 #pragma unroll
@@ -344,9 +360,8 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
       } else if constexpr (EPI == GEPI_STORE) {
         h8_t o = v;
         if (a.residual) {
-          const h8_t res = *(const h8_t *)&a.residual[(size_t)m * a.N + n];
 #pragma unroll
-          for (int c = 0; c < 8; c++) o[c] = (_Float16)((float)res[c] + (float)v[c]);
+          for (int c = 0; c < 8; c++) o[c] = (_Float16)((float)res[i][p][c] + (float)v[c]);
         }
         *(h8_t *)&a.y[(size_t)m * a.N + n] = o;
       } else {
