@@ -125,8 +125,8 @@ def test_few_rows_streaming_kernel_equals_tiled_kernel(hip, monkeypatch):
 @pytest.mark.parametrize("kind", ["float16", "int8", "nf4"])
 def test_tile_shapes_of_the_tiled_kernel_agree_bit_for_bit(hip, monkeypatch, kind):
     """Every block shape of the tiled kernel (256x256 out of two LDS buffers, 256x256 and 256x128 out of one, 128x128)
-    walks K in the same order, so the outputs are identical; 3 and 4 K tiles, a ragged last row tile, with a residual."""
-    for rows, out_f, in_f in ((300, 512, 192), (257, 256, 256)):
+    walks K in the same order, so the outputs are identical; 1, 3 and 4 K tiles, a ragged last row tile, with a residual."""
+    for rows, out_f, in_f in ((300, 512, 192), (257, 256, 256), (130, 256, 64)):
         w, s = make_weight(kind, out_f, in_f)
         x = RNG.standard_normal((rows, in_f)).astype(np.float16)
         res = RNG.standard_normal((rows, out_f)).astype(np.float16)
