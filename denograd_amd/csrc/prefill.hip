@@ -30,7 +30,7 @@ struct PrefillAttnArgs {
   float scale_log2;                  // float(1/sqrt(HD)) * log2(e)
 };
 
-template <int HD> __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(PrefillAttnArgs a) {
+template <int HD> __global__ __launch_bounds__(PF_THREADS, 2) void attn_prefill_kernel(PrefillAttnArgs a) {
   constexpr int KS = HD + 8;          // K tile row stride in halves
   constexpr int VS = PF_KEYS + 8;     // V^T tile row stride in halves
   constexpr int KC = HD / 8;          // 16-byte chunks per cache row
