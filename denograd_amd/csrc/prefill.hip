@@ -130,35 +130,44 @@ template <int HD> __global__ __launch_bounds__(PF_THREADS, 2) void attn_prefill_
         s[tk] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[c], s[tk], 0, 0, 0);
       }
     }
-    // accumulator r of s[tk] is key k0 + tk*32 + 8*(r/4) + 4*lg + r%4 for query row l32
+    // accumulator r of s[tk] is key k0 + tk*32 + 8*(r/4) + 4*lg + r%4 for query row l32.  Only a tile that reaches past
+    // the first query row of the wavefront has masked keys (uniform test); the scale is positive, so the maximum is
+    // taken over the raw scores and the scale folded into the exponent: exp2(s * scale - max * scale).
+    if (k0 + PF_KEYS - 1 > a.start_pos + qw0) {
+#pragma unroll
+      for (int tk = 0; tk < 2; tk++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int key = k0 + tk * 32 + 8 * (r / 4) + 4 * lg + (r % 4);
+          if (key > qpos) s[tk][r] = -INFINITY;
+        }
+    }
     float mx = m_run;
 #pragma unroll
     for (int tk = 0; tk < 2; tk++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int key = k0 + tk * 32 + 8 * (r / 4) + 4 * lg + (r % 4);
-        const float v = key <= qpos ? s[tk][r] * a.scale_log2 : -INFINITY;
-        s[tk][r] = v;
-        mx = fmaxf(mx, v);
-      }
+      for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[tk][r]);
     mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float alpha = __builtin_amdgcn_exp2f(m_run - mx);   // first visible tile: exp2(-inf) = 0
+    const float alpha = __builtin_amdgcn_exp2f((m_run - mx) * a.scale_log2);   // first visible tile: exp2(-inf) = 0
     m_run = mx;
+    const float mxs = mx * a.scale_log2;
     float psum = 0.0f;
     h8_t pf[2][2];
 #pragma unroll
     for (int tk = 0; tk < 2; tk++)
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        const float p = __builtin_amdgcn_exp2f(s[tk][r] - mx);
+        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[tk][r], a.scale_log2, -mxs));
         psum += p;
         pf[tk][r / 8][r % 8] = (_Float16)p;
       }
     l_run = l_run * alpha + psum;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {   // the running maximum of some row moved (uniform branch)
 #pragma unroll
-    for (int td = 0; td < HD / 32; td++)
+      for (int td = 0; td < HD / 32; td++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) o_acc[td][r] *= alpha;
+        for (int r = 0; r < 16; r++) o_acc[td][r] *= alpha;
+    }
 
     // O^T += V^T . P^T : k-slot s' of lane half lg in step (tk, hs) is key tk*32 + hs*16 + 8*(s'/4) + 4*lg + s'%4
 #pragma unroll
