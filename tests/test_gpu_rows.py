@@ -95,6 +95,10 @@ def test_gemm_rejects_bad_shapes(hip):
         check(hip.jsgrad_hip_gemm(ffi.W_F32, t.ptr, None, 128, 64, t.ptr, 4, t.ptr, None))
     with pytest.raises(ffi.HipError, match="scales"):
         check(hip.jsgrad_hip_gemm(ffi.W_I8, t.ptr, None, 128, 64, t.ptr, 4, t.ptr, None))
+    with pytest.raises(ffi.HipError, match="16-byte aligned"):
+        check(hip.jsgrad_hip_gemm(ffi.W_F16, t.ptr, None, 128, 64, t.ptr + 2, 4, t.ptr, None))
+    with pytest.raises(ffi.HipError, match="16-byte aligned"):
+        check(hip.jsgrad_hip_gemm(ffi.W_F16, t.ptr, None, 128, 64, t.ptr, 4, t.ptr, t.ptr + 8))
 
 
 def test_few_rows_streaming_kernel_equals_tiled_kernel(hip, monkeypatch):
