@@ -151,10 +151,11 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
 #pragma unroll
     for (int i = 0; i < A_LOADS; i++) ga[i] = *(const u4_t *)(asrc[i] + ko * 2);
   };
-  auto issue_b = [&](int kt) {
+  auto issue_b = [&](int kt, int lo = 0, int hi = 1 << 30) {
     const size_t ko = (size_t)kt * GEMM_BK;
 #pragma unroll
     for (int i = 0; i < B_LOADS; i++) {
+      if (i < lo || i >= hi) continue;
       if constexpr (KIND == JSGRAD_W_F16) gb[i] = *(const u4_t *)(bsrc[i] + ko * 2);
       else if constexpr (KIND == JSGRAD_W_I8) gb[i] = *(const u4_t *)(bsrc[i] + ko);
       else { gb[i] = *(const u4_t *)(bsrc[i] + ko / 2); gs[i] = bscale_ptr[i][kt]; }
@@ -165,9 +166,10 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
 #pragma unroll
     for (int i = 0; i < A_LOADS; i++) *(u4_t *)&As[buf * BUF + (arow_t + i * 32) * LS + achunk * 8] = ga[i];
   };
-  auto commit_b = [&](int buf) {
+  auto commit_b = [&](int buf, int lo = 0, int hi = 1 << 30) {
 #pragma unroll
     for (int i = 0; i < B_LOADS; i++) {
+      if (i < lo || i >= hi) continue;
       _Float16 *dst = &Bs[buf * BUF + (brow_t + i * B_ROWS_PER_PASS) * LS];
       if constexpr (KIND == JSGRAD_W_F16) *(u4_t *)(dst + bchunk * 8) = gb[i];
       else if constexpr (KIND == JSGRAD_W_I8) {
@@ -226,8 +228,9 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
   if constexpr (DB) {
     // Two LDS buffers, one barrier per K tile: while the matrix cores work on tile kt out of one buffer, the same
     // wavefront turns the registers of tile kt+1 into the other buffer and requests tile kt+2 into the registers just
-    // freed: the x half in K step 0, the weight half in K step 2, so every request has a whole tile's time to arrive
-    // and the requests of a CU (64 KiB per tile through a 64 B/clock L1) are spread over the tile.
+    // freed: the x half in K step 0, the weight half in K steps 1 and 2 (half of its loads each, which also spreads the
+    // conversion of quantised weights), so every request has a whole tile's time to arrive and the requests of a CU
+    // (64 KiB per tile through a 64 B/clock L1) are spread over the tile.
     // The barrier sits between K steps 2 and 3.  By then every wavefront has written its share of tile kt+1 and has
     // read all fragments of tile kt (those of step 3 are read during step 2), so during step 3 the fragments of the
     // first step of tile kt+1 are read and the matrix instructions run on across the end of the tile.  The buffer
@@ -250,24 +253,27 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
         if (kk < LAST) frags(cur, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
         else frags(cur ^ 1, 0, af[0], bf[0]);
         if (kk == 0) { commit_a(cur ^ 1); issue_a(after_next); }
-        if (kk == 2) { commit_b(cur ^ 1); issue_b(after_next); }
+        constexpr int HB = B_LOADS > 1 ? B_LOADS / 2 : 1;   // weight loads of K step 1; the rest in step 2
+        if (kk == 1) { commit_b(cur ^ 1, 0, HB); issue_b(after_next, 0, HB); }
+        if (kk == 2) { commit_b(cur ^ 1, HB, B_LOADS); issue_b(after_next, HB, B_LOADS); }
         mfmas(af[kk & 1], bf[kk & 1]);
         // The order inside this K step, spelled out for the instruction scheduler: every matrix instruction is followed by
         // a share of the other work of the step (fragment reads of the next step, conversion and LDS writes of the next
         // tile, then the requests of the tile after it), so that work runs while the matrix core is busy.  Left alone the
         // scheduler puts each fragment read directly before its first use and waits out the LDS latency every time.
         constexpr int NMF = TM * TN;
-        constexpr int LOADS = kk == 0 ? A_LOADS : B_LOADS;
-        constexpr int WRITES = kk == 0 ? A_LOADS : (KIND == JSGRAD_W_F16 ? B_LOADS : (KIND == JSGRAD_W_I8 ? 2 * B_LOADS : 4 * B_LOADS));
+        constexpr int BL = kk == 1 ? HB : B_LOADS - HB;
+        constexpr int LOADS = kk == 0 ? A_LOADS : BL;
+        constexpr int WRITES = kk == 0 ? A_LOADS : (KIND == JSGRAD_W_F16 ? BL : (KIND == JSGRAD_W_I8 ? 2 * BL : 4 * BL));
         constexpr int WSTEPS = NMF - (LOADS < NMF / 2 ? LOADS : NMF / 2);     // matrix instructions that carry the writes
 #pragma unroll
         for (int i = 0; i < NMF; i++) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                          // one MFMA
           if (i < TM + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);          // one LDS read
-          if (kk == 0 || kk == 2) {
+          if (kk < LAST && LOADS > 0) {
             if (i < WSTEPS) {
-              if (kk == 2 && KIND != JSGRAD_W_F16) __builtin_amdgcn_sched_group_barrier(0x002, KIND == JSGRAD_W_I8 ? 10 : 14, 0);
-              if constexpr (kk == 2 && KIND == JSGRAD_W_NF4) __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);   // table look-ups
+              if (kk > 0 && KIND != JSGRAD_W_F16) __builtin_amdgcn_sched_group_barrier(0x002, KIND == JSGRAD_W_I8 ? 6 : 10, 0);
+              if constexpr (kk > 0 && KIND == JSGRAD_W_NF4) __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);   // table look-ups
               __builtin_amdgcn_sched_group_barrier(0x200, (WRITES + WSTEPS - 1) / WSTEPS, 0);
             } else {
               __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
