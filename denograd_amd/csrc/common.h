@@ -219,17 +219,20 @@ __device__ __forceinline__ float xexp2f(float d) {
   if (d != d) u = NAN;
   return u;
 }
-// xexp2 for half tensors: fp16-rounded coefficients, float Horner chain, bounds [23, -22]
+// xexp2 for half tensors: fp16-rounded coefficients, float Horner chain, bounds [23, -22].
+// The same values as the float version's sequence with fewer instructions: whatever d lies outside [-22, 23) or is not a
+// number gets its result from the three tests at the end, so the non-finite mask and the range test of the rounding are
+// not needed in front (the conversion to int saturates, nothing traps, q is clamped before it is used); inside the bounds
+// u * 2^q is a normal number, so one exact scaling by 2^q equals the two exact multiplications by 2^(q>>1) and 2^(q-(q>>1)).
 __device__ __forceinline__ float xexp2h(float d) {
   const float c[7] = {0.1535920892e-3f, 0.1339262701e-2f, 0.9618384764e-2f, 0.5550347269e-1f, 0.2402264476e+0f, 0.6931471825e+0f, 1.0f};
-  float x = mask_nonfinite(d);
-  int q = rintk(x);
-  float s = __fsub_rn(x, (float)q);
+  int q = (int)__fadd_rn(d, d < 0.0f ? -0.5f : 0.5f);
+  float s = __fsub_rn(d, (float)q);
   float u = rn16(c[0]);
 #pragma unroll
   for (int i = 1; i < 7; i++) u = __fadd_rn(__fmul_rn(u, s), rn16(c[i]));
   q = q > 60 ? 60 : (q < -60 ? -60 : q);
-  u = __fmul_rn(__fmul_rn(u, pow2i(q >> 1)), pow2i(q - (q >> 1)));
+  u = __builtin_amdgcn_ldexpf(u, q);
   if (d >= 23.0f) u = INFINITY;
   if (d < -22.0f) u = 0.0f;
   if (d != d) u = NAN;

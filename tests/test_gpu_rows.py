@@ -185,6 +185,29 @@ def test_gemm_ffn_gate(hip, kind, rows, dim, hidden):
     assert_close(tg.numpy().astype(np.float32), ref, True, f"ffn_gate {kind} {rows}", composed=True)
 
 
+def test_swiglu_epilogue_silu_bit_exact_for_every_fp16_input(hip):
+    """One-hot input rows pick single weights, so the gate GEMM output is each fp16 value itself (no summation) and the
+    epilogue's silu(g) * 1 can be compared with the oracle's on every finite fp16 bit pattern (weight rows that hold an infinity
+    or a NaN are left out: 0 * inf in the other rows' sums makes the whole row NaN)."""
+    hidden, dim = 1024, 64
+    w1 = np.arange(65536, dtype=np.uint16).view(np.float16).reshape(hidden, dim)
+    w3 = np.ones((hidden, dim), np.float16)
+    x = np.eye(dim, dtype=np.float16)
+    t1, t3, tx, tg = Tensor(w1), Tensor(w3), Tensor(x), Tensor.empty((dim, hidden), "float16")
+    check(hip.jsgrad_hip_gemm_ffn_gate(ffi.W_F16, t1.ptr, None, t3.ptr, None, tx.ptr, dim, tg.ptr, dim, hidden))
+    got = tg.numpy().T.reshape(-1)                                   # got[n * dim + r] = silu(w1[n][r])
+    vals = w1.reshape(-1).astype(np.float32)
+    with np.errstate(all="ignore"):
+        ref = orc.silu(vals, True).astype(np.float16)
+    finite_in = np.isfinite(vals)
+    nan_rows = ~np.isfinite(w1.astype(np.float32)).reshape(hidden, dim)
+    clean = np.repeat(~nan_rows.any(axis=1), dim)
+    sel = finite_in & clean
+    sel[0x8000] = False      # -0.0 leaves the GEMM as +0.0 (a sum that starts from +0.0), so silu sees another input
+    assert sel.sum() > 60000
+    assert np.array_equal(got[sel].view(np.uint16), ref[sel].view(np.uint16))
+
+
 @pytest.mark.parametrize("B,S,dim", [(2, 37, 256), (16, 1, 2048), (3, 9, 2048)])   # prefill rows; batched decode and few rows on the streaming kernel
 @pytest.mark.parametrize("kind,hd", [("float16", 64), ("int8", 128), ("nf4", 64)])
 def test_gemm_qkv_rope_writes_queries_and_cache(hip, kind, hd, B, S, dim):
