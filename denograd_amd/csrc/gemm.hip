@@ -712,9 +712,13 @@ template <int EPI> static int dispatch_gemm(int kind, const GemmArgs &a, int pro
   const int n_out = EPI == GEPI_SWIGLU ? 2 * a.N : a.N;
   const char *pin = getenv("JSG_GEMM_TILE");
   const bool can256 = tall && n_out % 256 == 0;
-  const bool piped = can256 && (!pin || !strcmp(pin, "db"));
+  // unpinned: the largest block shape that still gives (nearly) every CU a block; a prompt of a few hundred rows is better off with
+  // 128x128 blocks on all CUs than with 256x256 blocks on a quarter of them
+  const int cus = state().cu_count;
+  auto blocks_of = [&](int bm, int bn) { return ((a.M + bm - 1) / bm) * (n_out / bn); };
+  const bool piped = can256 && (pin ? !strcmp(pin, "db") : 4 * blocks_of(256, 256) >= 3 * cus);
   const bool wide = can256 && pin && !strcmp(pin, "wide");
-  const bool small = tall && pin && !strcmp(pin, "small");
+  const bool small = tall && (pin ? !strcmp(pin, "small") : (!piped && blocks_of(256, 128) < cus));
   bool taken = false;
   if (kind == JSGRAD_W_F16) { const int rc = dispatch_skinny<JSGRAD_W_F16, EPI>(a, prof_kind, &taken); if (taken) return rc; }
   if (kind == JSGRAD_W_I8) { const int rc = dispatch_skinny<JSGRAD_W_I8, EPI>(a, prof_kind, &taken); if (taken) return rc; }
