@@ -254,9 +254,20 @@ template <> __device__ __forceinline__ float silu_act<float>(float a) {
   float u = xexp2f(__fmul_rn(a, -1.4426950408889634f));
   return __fmul_rn(a, __fdiv_rn(1.0f, __fadd_rn(1.0f, u)));
 }
+// 1 / d for d = 1 + exp2(...) >= 1 (or +inf, or NaN): no scaling for tiny or huge operands is needed, so the division is the
+// hardware reciprocal refined the way the full IEEE sequence does it (two residual steps), without that sequence's range
+// handling.  Same bits as __fdiv_rn(1, d) for every input the fp16 silu can produce (checked exhaustively in the tests).
+__device__ __forceinline__ float recip_ge1(float d) {
+  float r = __builtin_amdgcn_rcpf(d);
+  float e = __builtin_fmaf(-d, r, 1.0f);
+  r = __builtin_fmaf(e, r, r);
+  e = __builtin_fmaf(-d, r, 1.0f);
+  r = __builtin_fmaf(e, r, r);
+  return d == INFINITY ? 0.0f : r;
+}
 template <> __device__ __forceinline__ float silu_act<_Float16>(float a) {
   float u = xexp2h(rn16(__fmul_rn(a, rn16(-1.4426950408889634f))));
-  return __fmul_rn(a, __fdiv_rn(1.0f, __fadd_rn(1.0f, u)));
+  return __fmul_rn(a, recip_ge1(__fadd_rn(1.0f, u)));
 }
 
 }  // namespace jsg
