@@ -20,6 +20,8 @@ typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
 // lane-local (plus one exchange between the two lane halves), and the fp16 probabilities are already laid out as the
 // B operand of O^T = V^T . P^T.  The k-slot order of an MFMA operand is free as long as both operands agree; V^T
 // fragments are read from a transposed LDS tile in the order the score accumulators come out.
+// Two blocks per CU: at head_dim 128 the kernel wants a few registers more than half of a SIMD's file, and a second block
+// that computes while this one waits at its barriers is worth more than those registers.
 constexpr int PF_THREADS = 256, PF_QROWS = 128, PF_KEYS = 64;
 
 struct PrefillAttnArgs {
