@@ -96,7 +96,7 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
     const int per = nblocks / 8;
     if (bid < per * 8) bid = (bid & 7) * per + (bid >> 3);
   }
-  constexpr int GROUP = 8;
+  constexpr int GROUP = KIND == JSGRAD_W_F16 ? 8 : 4;   // quantised weight tiles are half or a quarter of the bytes of an x tile: fewer x tiles, more weight tiles per XCD
   const int in_group = GROUP * tiles_n;
   const int first_m = (bid / in_group) * GROUP;
   const int gsz = min(tiles_m - first_m, GROUP);
