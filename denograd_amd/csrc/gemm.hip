@@ -77,15 +77,19 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
   constexpr int B_LOADS = BN / B_ROWS_PER_PASS;
   static_assert(B_LOADS >= 1, "tile too narrow for this weight format");
   constexpr int BUF = (BM + BN) * LS;                     // halves per LDS buffer
-  extern __shared__ __align__(16) _Float16 gemm_lds[];   // one or two buffers of [BM + BN rows][LS], then the 16-entry NF4 table
+  extern __shared__ __align__(16) _Float16 gemm_lds[];   // one or two buffers of [BM + BN rows][LS], then 32 spare bytes and the 256-entry NF4 table
   _Float16 *As = gemm_lds, *Bs = gemm_lds + BM * LS, *lut = gemm_lds + (DB ? 2 : 1) * BUF;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WGN, wn = wave % WGN;
   const int l32 = lane & 31, lg = lane >> 5;
 
+  // NF4: one table entry per BYTE, the two code values of its nibbles as a packed pair (element 2j is the high nibble,
+  // llama3.ts:92-94), so a byte costs one LDS read and one packed multiplication by the block scale
+  uint32_t *pairs = (uint32_t *)(lut + 16);
   if constexpr (KIND == JSGRAD_W_NF4) {
-    if (tid < 16) lut[tid] = (_Float16)NF4_CODE[tid];
+    const h2_t c = {(_Float16)NF4_CODE[tid >> 4], (_Float16)NF4_CODE[tid & 15]};
+    pairs[tid] = __builtin_bit_cast(uint32_t, c);
   }
 
   // ---- tile id: XCD-contiguous, then grouped so that neighbouring ids share an x tile column-block
@@ -192,9 +196,7 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
 #pragma unroll
           for (int b = 0; b < 4; b++) {
             const uint32_t byte = (wds[d] >> (8 * b)) & 0xffu;
-            const h2_t c = {lut[byte >> 4], lut[byte & 15]};
-            h2_t r = c * sv;
-            outw[b] = __builtin_bit_cast(uint32_t, r);
+            outw[b] = pk_mul_h2(pairs[byte], sv);
           }
           o.x = outw[0]; o.y = outw[1]; o.z = outw[2]; o.w = outw[3];
           *(u4_t *)(dst + bchunk * 32 + d * 8) = o;
@@ -691,7 +693,7 @@ template <int KIND, int EPI, int WGM, int WGN, int TM, int TN, bool DB = false> 
   constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
   const int out_per_tile = EPI == GEPI_SWIGLU ? BN / 2 : BN;
   const int tiles = ((a.M + BM - 1) / BM) * (a.N / out_per_tile);
-  constexpr size_t lds = (size_t)(DB ? 2 : 1) * (BM + BN) * GEMM_LDS_STRIDE * sizeof(_Float16) + 32;
+  constexpr size_t lds = (size_t)(DB ? 2 : 1) * (BM + BN) * GEMM_LDS_STRIDE * sizeof(_Float16) + 32 + (KIND == JSGRAD_W_NF4 ? 1024 : 0);
   static_assert(lds <= 160 * 1024, "LDS of one compute unit");
   if constexpr (lds > 64 * 1024) {
     static bool raised = false;   // one process, one device, one thread: set once per instantiation
