@@ -1,8 +1,10 @@
 /*
  * jsgrad_oracle.c -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
  *
- * A plain-C, single-threaded CPU restatement of the arithmetic that jsgrad's CLANG
- * device performs for Llama-3 inference.  It exists only as the checker for the HIP
+ * A plain-C CPU restatement of the arithmetic that jsgrad's CLANG device performs for
+ * Llama-3 inference.  One thread unless or_set_threads() says otherwise (the reference's
+ * CLANG device is single-threaded; threads only split independent outputs among them,
+ * every output is computed by the same sequence of operations either way).  It exists only as the checker for the HIP
  * path (tests, the smoke check and the cpu_baseline leg of the benchmark); the
  * product library never links, loads or calls it.
  *
@@ -43,6 +45,12 @@
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+static inline int omp_thread(void) { return omp_get_thread_num(); }
+#else
+static inline int omp_thread(void) { return 0; }
+#endif
 
 /* ------------------------------------------------------------------ fp16 <-> fp32 */
 
@@ -375,10 +383,42 @@ typedef struct {
  *             only yields the exact fp16 code values.)
  *   int8/nf4, several input rows (materialised=1): the weight is expanded over the rows,
  *             which realises the dequantised matrix in fp16 first: W = RN16(float(code)*scale). */
+static int g_threads = 1;
+/* Threads for the loops over independent outputs (rows of a Linear, heads of the attention).  1 = the reference's way. */
+void or_set_threads(int n) { g_threads = n < 1 ? 1 : n; }
+
+/* one weight row as the floats the products use: W[o][k] as stored, code*scale, or RN16(code*scale) */
+static void weight_row(const or_linear_t *L, int o, int materialised, const float *code, float *wrow) {
+  const int in_f = L->in_f;
+  switch (L->kind) {
+    case OR_W_F32: memcpy(wrow, (const float *)L->w + (size_t)o * in_f, sizeof(float) * (size_t)in_f); break;
+    case OR_W_F16: { const uint16_t *w = (const uint16_t *)L->w + (size_t)o * in_f; for (int k = 0; k < in_f; k++) wrow[k] = h2f(w[k]); break; }
+    case OR_W_I8: {
+      const int8_t *w = (const int8_t *)L->w + (size_t)o * in_f;
+      const float s = h2f(L->scale[o]);
+      if (materialised) for (int k = 0; k < in_f; k++) wrow[k] = rn16((float)w[k] * s);
+      else for (int k = 0; k < in_f; k++) wrow[k] = (float)w[k] * s;
+      break;
+    }
+    default: {
+      const uint8_t *w = (const uint8_t *)L->w + ((size_t)o * in_f) / 2;
+      const uint16_t *sc = L->scale + ((size_t)o * in_f) / 64;
+      for (int k = 0; k < in_f; k += 2) {
+        float s = h2f(sc[k / 64]);
+        uint8_t b = w[k / 2];
+        float w0 = code[b >> 4] * s, w1 = code[b & 15] * s;
+        if (materialised) { w0 = rn16(w0); w1 = rn16(w1); }
+        wrow[k] = w0; wrow[k + 1] = w1;
+      }
+    }
+  }
+}
+
 void or_linear_ex(const or_linear_t *L, const float *x, float *y, int act16, int materialised) {
   const int in_f = L->in_f;
   float code[16];
   or_nf4_code(code);
+#pragma omp parallel for schedule(static) num_threads(g_threads) if (g_threads > 1)
   for (int o = 0; o < L->out_f; o++) {
     float acc = 0.0f;
     switch (L->kind) {
@@ -408,8 +448,50 @@ void or_linear_ex(const or_linear_t *L, const float *x, float *y, int act16, int
   }
 }
 void or_linear(const or_linear_t *L, const float *x, float *y, int act16) { or_linear_ex(L, x, y, act16, 0); }
-/* ctypes-friendly wrapper around or_linear_ex for n_rows input rows */
+
+/* The same Linear for S input rows x[S][in_f] -> y[S][out_f].  Every y[s][o] is the sum or_linear_ex forms (one float
+ * accumulator, sequential in k, a rounded product added at every step); only the organisation differs: a weight row is
+ * turned into floats once, and OR_TILE input rows advance through k side by side (their accumulators are independent, so
+ * the compiler may keep them in one vector register: IEEE multiply and add per lane, no contraction). */
+#define OR_TILE 32
+void or_linear_rows(const or_linear_t *L, const float *x, int S, float *y, int act16, int materialised) {
+  if (S == 1) { or_linear_ex(L, x, y, act16, materialised); return; }
+  const int in_f = L->in_f, out_f = L->out_f;
+  const int ntile = (S + OR_TILE - 1) / OR_TILE;
+  /* xt[tile][k][OR_TILE]: the input transposed inside tiles of rows (rows past S are zero and never stored) */
+  float *xt = (float *)calloc((size_t)ntile * in_f * OR_TILE, sizeof(float));
+  for (int s = 0; s < S; s++)
+    for (int k = 0; k < in_f; k++) xt[((size_t)(s / OR_TILE) * in_f + k) * OR_TILE + s % OR_TILE] = x[(size_t)s * in_f + k];
+  float code[16];
+  or_nf4_code(code);
+#pragma omp parallel num_threads(g_threads) if (g_threads > 1)
+  {
+    float *wrow = (float *)malloc(sizeof(float) * (size_t)in_f);
+#pragma omp for schedule(static)
+    for (int o = 0; o < out_f; o++) {
+      weight_row(L, o, materialised, code, wrow);
+      for (int t = 0; t < ntile; t++) {
+        const float *xp = xt + (size_t)t * in_f * OR_TILE;
+        float acc[OR_TILE];
+        for (int i = 0; i < OR_TILE; i++) acc[i] = 0.0f;
+        for (int k = 0; k < in_f; k++) {
+          const float wk = wrow[k];
+          for (int i = 0; i < OR_TILE; i++) acc[i] = acc[i] + xp[(size_t)k * OR_TILE + i] * wk;
+        }
+        for (int i = 0; i < OR_TILE && t * OR_TILE + i < S; i++) y[(size_t)(t * OR_TILE + i) * out_f + o] = rn_act(acc[i], act16);
+      }
+    }
+    free(wrow);
+  }
+  free(xt);
+}
+/* ctypes-friendly wrapper for n_rows input rows: more than one row sees the weight expanded over the rows (materialised) */
 void or_linear_call(int kind, int out_f, int in_f, const void *w, const void *scale, const float *x, int n_rows, float *y, int act16) {
+  or_linear_t L = {kind, out_f, in_f, w, (const uint16_t *)scale};
+  or_linear_rows(&L, x, n_rows, y, act16, n_rows > 1);
+}
+/* the row-by-row evaluation of the same call (what or_linear_rows must reproduce bit for bit; used by the tests) */
+void or_linear_call_rowwise(int kind, int out_f, int in_f, const void *w, const void *scale, const float *x, int n_rows, float *y, int act16) {
   or_linear_t L = {kind, out_f, in_f, w, (const uint16_t *)scale};
   for (int r = 0; r < n_rows; r++) or_linear_ex(&L, x + (size_t)r * in_f, y + (size_t)r * out_f, act16, n_rows > 1);
 }
@@ -532,33 +614,35 @@ void or_embed(const or_model_t *m, int tok, float *h) { embed_row(m, tok, h); }
  * GQA: query head h reads kv head h / n_rep (repeat_kv, llama.ts:34-39). */
 static void attention(or_model_t *m, int layer, const float *xn, int S, int start_pos, float *out) {
   const or_layer_t *l = &m->layers[layer];
-  const int d = m->dim, H = m->n_heads, KV = m->n_kv_heads, hd = m->head_dim, n_rep = H / KV, act16 = m->act16;
+  const int H = m->n_heads, KV = m->n_kv_heads, hd = m->head_dim, n_rep = H / KV, act16 = m->act16;
   const int T = start_pos + S;
   const int mat = S > 1 || m->batched;
   const float scale = (float)(1.0 / sqrt((double)hd));
-  float *q = (float *)malloc(sizeof(float) * (size_t)H * hd);
-  float *k = (float *)malloc(sizeof(float) * (size_t)KV * hd);
   float *attn = (float *)malloc(sizeof(float) * (size_t)S * H * hd);
   float *qs = (float *)malloc(sizeof(float) * (size_t)S * H * hd);
-  float *sc = (float *)malloc(sizeof(float) * (size_t)T);
+  float *sc_all = (float *)malloc(sizeof(float) * (size_t)T * (size_t)g_threads);   /* one score row per thread */
   float *fc = (float *)malloc(sizeof(float) * (size_t)hd);
   float *ck = m->cache_k + (size_t)layer * m->max_context * KV * hd;
   float *cv = m->cache_v + (size_t)layer * m->max_context * KV * hd;
   /* all new rows enter the cache before any query reads it (assign is realised first, :87) */
+  float *ks = (float *)malloc(sizeof(float) * (size_t)S * KV * hd);
+  or_linear_rows(&l->wq, xn, S, qs, act16, mat);
+  or_linear_rows(&l->wk, xn, S, ks, act16, mat);
+  or_linear_rows(&l->wv, xn, S, cv + (size_t)start_pos * KV * hd, act16, mat);
   for (int s = 0; s < S; s++) {
     int pos = start_pos + s;
     for (int i = 0; i < hd; i++) fc[i] = rn_act(m->freqs[(size_t)pos * hd + i], act16); /* llama.ts:205 cast */
-    or_linear_ex(&l->wq, xn + (size_t)s * d, q, act16, mat);
-    or_linear_ex(&l->wk, xn + (size_t)s * d, k, act16, mat);
-    or_linear_ex(&l->wv, xn + (size_t)s * d, cv + (size_t)pos * KV * hd, act16, mat);
-    rope_rows(q, H, hd, fc, act16);
-    rope_rows(k, KV, hd, fc, act16);
-    memcpy(qs + (size_t)s * H * hd, q, sizeof(float) * (size_t)H * hd);
-    memcpy(ck + (size_t)pos * KV * hd, k, sizeof(float) * (size_t)KV * hd);
+    rope_rows(qs + (size_t)s * H * hd, H, hd, fc, act16);
+    rope_rows(ks + (size_t)s * KV * hd, KV, hd, fc, act16);
+    memcpy(ck + (size_t)pos * KV * hd, ks + (size_t)s * KV * hd, sizeof(float) * (size_t)KV * hd);
   }
-  for (int s = 0; s < S; s++) {
-    int vis = start_pos + s + 1; /* causal mask triu(start_pos+1), llama.ts:208: keys t <= start_pos+s */
-    for (int h = 0; h < H; h++) {
+  free(ks);
+#pragma omp parallel for schedule(dynamic) num_threads(g_threads) if (g_threads > 1)
+  for (int sh = 0; sh < S * H; sh++) {
+    const int s = sh / H, h = sh % H;
+    float *sc = sc_all + (size_t)omp_thread() * T;
+    {
+      int vis = start_pos + s + 1; /* causal mask triu(start_pos+1), llama.ts:208: keys t <= start_pos+s */
       const int g = h / n_rep;
       const float *qh = qs + ((size_t)s * H + h) * hd;
       for (int t = 0; t < T; t++) {
@@ -583,19 +667,19 @@ static void attention(or_model_t *m, int layer, const float *xn, int S, int star
       }
     }
   }
-  for (int s = 0; s < S; s++) or_linear_ex(&l->wo, attn + (size_t)s * H * hd, out + (size_t)s * d, act16, mat);
-  free(q); free(k); free(attn); free(qs); free(sc); free(fc);
+  or_linear_rows(&l->wo, attn, S, out, act16, mat);
+  free(attn); free(qs); free(sc_all); free(fc);
 }
 
 /* FeedForward.call models/llama.ts:108-110: w2( silu(w1 x) * (w3 x) ).
  * Kernels (R5): w1 -> buffer; w3 with the epilogue silu(a)*RN_act(dot) -> buffer; w2. */
-static void feed_forward(const or_model_t *m, const or_layer_t *l, const float *xn, float *out, int mat) {
+static void feed_forward(const or_model_t *m, const or_layer_t *l, const float *xn, int S, float *out, int mat) {
   const int F = m->hidden, act16 = m->act16;
-  float *a = (float *)malloc(sizeof(float) * (size_t)F), *u = (float *)malloc(sizeof(float) * (size_t)F);
-  or_linear_ex(&l->w1, xn, a, act16, mat);
-  or_linear_ex(&l->w3, xn, u, act16, mat);
-  for (int i = 0; i < F; i++) a[i] = rn_act(silu_act(a[i], act16) * u[i], act16);
-  or_linear_ex(&l->w2, a, out, act16, mat);
+  float *a = (float *)malloc(sizeof(float) * (size_t)S * F), *u = (float *)malloc(sizeof(float) * (size_t)S * F);
+  or_linear_rows(&l->w1, xn, S, a, act16, mat);
+  or_linear_rows(&l->w3, xn, S, u, act16, mat);
+  for (long i = 0; i < (long)S * F; i++) a[i] = rn_act(silu_act(a[i], act16) * u[i], act16);
+  or_linear_rows(&l->w2, a, S, out, act16, mat);
   free(a); free(u);
 }
 
@@ -615,10 +699,8 @@ int or_model_forward(or_model_t *m, const int *tokens, int S, int start_pos, flo
     for (int s = 0; s < S; s++) or_rmsnorm(h + (size_t)s * d, l->attention_norm, d, m->norm_eps, act16, xn + (size_t)s * d);
     attention(m, L, xn, S, start_pos, t);
     for (long i = 0; i < (long)S * d; i++) h[i] = rn_act(h[i] + t[i], act16);
-    for (int s = 0; s < S; s++) {
-      or_rmsnorm(h + (size_t)s * d, l->ffn_norm, d, m->norm_eps, act16, xn + (size_t)s * d);
-      feed_forward(m, l, xn + (size_t)s * d, t + (size_t)s * d, S > 1 || m->batched);
-    }
+    for (int s = 0; s < S; s++) or_rmsnorm(h + (size_t)s * d, l->ffn_norm, d, m->norm_eps, act16, xn + (size_t)s * d);
+    feed_forward(m, l, xn, S, t, S > 1 || m->batched);
     for (long i = 0; i < (long)S * d; i++) h[i] = rn_act(h[i] + t[i], act16);
   }
   float *lg = logits ? logits : (float *)malloc(sizeof(float) * (size_t)m->vocab);

@@ -51,6 +51,8 @@ def lib() -> C.CDLL:
             "or_nf4_code": ([vp], None),
             "or_nf4_quantize": ([vp, i64, vp, vp], None), "or_nf4_dequant": ([vp, vp, i64, vp], None),
             "or_linear_call": ([i32, i32, i32, vp, vp, vp, i32, vp, i32], None),
+            "or_linear_call_rowwise": ([i32, i32, i32, vp, vp, vp, i32, vp, i32], None),
+            "or_set_threads": ([i32], None),
             "or_rmsnorm": ([vp, vp, i32, f32, i32, vp], None),
             "or_rope": ([vp, i32, i32, vp, i32], None),
             "or_argmax": ([vp, i32], i32),
@@ -165,13 +167,21 @@ def _kind_of(w: np.ndarray, scale) -> int:
     raise TypeError(f"unsupported weight dtype {w.dtype}")
 
 
-def linear(w, scale, x, out_f: int, in_f: int, act16: bool) -> np.ndarray:
-    """y = x . W^T for n rows of x (float32 values already representable in the activation dtype)."""
+def set_threads(n: int) -> None:
+    """Threads for loops over independent outputs (1 = single-threaded like the reference's CLANG device, the default).
+    Results do not depend on it."""
+    lib().or_set_threads(int(n))
+
+
+def linear(w, scale, x, out_f: int, in_f: int, act16: bool, rowwise: bool = False) -> np.ndarray:
+    """y = x . W^T for n rows of x (float32 values already representable in the activation dtype).
+    rowwise: evaluate row by row with the one-row routine (same results; the tests compare the two)."""
     w = np.ascontiguousarray(w)
     s = None if scale is None else np.ascontiguousarray(scale, np.float16)
     x = _f32(x).reshape(-1, in_f)
     y = np.empty((x.shape[0], out_f), np.float32)
-    lib().or_linear_call(_kind_of(w, s), out_f, in_f, _p(w), _p(s), _p(x), x.shape[0], _p(y), int(act16))
+    fn = lib().or_linear_call_rowwise if rowwise else lib().or_linear_call
+    fn(_kind_of(w, s), out_f, in_f, _p(w), _p(s), _p(x), x.shape[0], _p(y), int(act16))
     return y
 
 

@@ -1,0 +1,264 @@
+"""Parity at the TRUE widths of the benchmark configurations (dim, heads, head_dim, FFN width, vocabulary 128 256, weight
+format), with two layers so that the CPU oracle finishes in seconds, and with the KV cache filled up to each
+configuration's context so that attention runs at its real length:
+
+  Llama-3.2-1B fp16 at 640 positions | 3B-shaped int8 at 1152 | 8B NF4 at 4160 | 8B int8 at 2112 (also in batches).
+
+The weights are made and quantised on the device (the device quantisers are bit-exact against the oracle's, see
+test_gpu_kernels.py) and copied to the host for the oracle, so both sides hold the same codes and scales; the cache rows
+are seeded random fp16 values given to both sides.  Bars: logits within rtol/atol 1e-2 of the oracle's, the oracle's
+greedy token unless its own top-2 logits lie within 2 fp16 ulp; new cache rows within 1e-2.
+Kernel-level cases at K = 4096 / 14336 and 2048-position prefill attention follow at the end."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle as orc
+from denograd_amd import ffi, synthetic
+from denograd_amd.ffi import check
+from denograd_amd.llama3 import Llama3
+from denograd_amd.state import get_state_dict
+from denograd_amd.tensor import Tensor
+from tests.helpers import assert_close
+from tests.test_gpu_prefill import check_token
+from tests.test_gpu_rows import attention_ref
+
+pytestmark = pytest.mark.gpu
+
+# name -> (synthetic config, visible positions the decode steps start from)
+FULL = {
+    "1B-f16": ("1B", 640),
+    "3B-int8": ("3B-int8", 1152),
+    "8B-nf4": ("8B-nf4", 4160),
+    "8B-int8": ("8B-int8", 2112),
+}
+THREADS = min(16, os.cpu_count() or 1)
+
+
+@pytest.fixture(scope="module", autouse=True)
+def oracle_threads():
+    orc.set_threads(THREADS)     # splits independent outputs among threads; results do not depend on it
+    yield
+    orc.set_threads(1)
+
+
+_built = {}
+
+
+def build(name):
+    """The 2-layer model at the configuration's widths on the device, and the oracle on a host copy of the same tensors."""
+    if name not in _built:
+        _built.clear()           # one model at a time
+        base, ctx = FULL[name]
+        cfg = synthetic.config(base, n_layers=2, max_context=ctx + 600)
+        gpu = Llama3.from_config(cfg).random_init(seed=5, tied=cfg["tied"])
+        gpu.model._prepare()
+        sd = {k: v.numpy() for k, v in get_state_dict(gpu.model).items()}
+        _built[name] = (cfg, gpu, orc.OracleModel(cfg, sd), sd)
+    return _built[name]
+
+
+def fill_cache(gpu, cpu, cfg, n_rows, seed, bsz=1, b=0):
+    """The same seeded fp16 rows into positions [0, n_rows) of sequence b's cache on the device and (unless cpu is None)
+    into the oracle's; per layer the K rows are drawn first, then the V rows."""
+    KV, hd = cfg["n_kv_heads"], cfg["dim"] // cfg["n_heads"]
+    lib = ffi.load()
+    rng = np.random.default_rng(seed)
+    for l, layer in enumerate(gpu.model.layers):
+        c = layer.attention.cache_kv
+        assert c.shape == (2, bsz, cfg["max_context"], KV, hd)
+        for plane in (0, 1):
+            rows = rng.standard_normal((n_rows, KV, hd), dtype=np.float32).astype(np.float16)
+            off = ((plane * bsz + b) * cfg["max_context"]) * KV * hd * 2
+            check(lib.jsgrad_hip_copyin(c.ptr + off, rows.ctypes.data, rows.nbytes))
+            if cpu is not None:
+                (cpu.cache_k if plane == 0 else cpu.cache_v)[l, :n_rows] = rows.astype(np.float32)
+    check(lib.jsgrad_hip_sync())
+
+
+def fill_oracle_cache(cpu, cfg, n_rows, seed):
+    """The rows fill_cache(seed) gave the device, drawn again in the same order, into the (reset) oracle cache."""
+    cpu.reset()
+    KV, hd = cfg["n_kv_heads"], cfg["dim"] // cfg["n_heads"]
+    rng = np.random.default_rng(seed)
+    for l in range(cfg["n_layers"]):
+        for dst in (cpu.cache_k, cpu.cache_v):
+            dst[l, :n_rows] = rng.standard_normal((n_rows, KV, hd), dtype=np.float32).astype(np.float16).astype(np.float32)
+
+
+def ratio(lg_g, lg_c):
+    return float(np.max(np.abs(lg_g - lg_c) / (1e-2 + 1e-2 * np.abs(lg_c))))
+
+
+@pytest.mark.parametrize("name", list(FULL))
+def test_decode_steps_at_the_configurations_context(name):
+    """Six teacher-forced one-token steps from the configuration's context on (eager, captured, replayed graph)."""
+    cfg, gpu, cpu, _ = build(name)
+    ctx = FULL[name][1]
+    cpu.set_batched(False)
+    for layer in gpu.model.layers:
+        layer.attention._ensure_cache("float16", gpu.device, 1)
+    gpu.model.forward_jit.reset()
+    fill_cache(gpu, cpu, cfg, ctx, seed=17)
+    toks = [int(t) for t in synthetic.random_prompt(cfg, 6, seed=3)]
+    gpu.start_pos = ctx
+    worst, near = 0.0, 0
+    for i, t in enumerate(toks):
+        pos = ctx + i
+        tok_c, lg_c = cpu.forward([t], pos)
+        tok_g = gpu._call(t); gpu.start_pos += 1
+        lg_g = gpu.model.logits.numpy().astype(np.float32)
+        r = ratio(lg_g, lg_c)
+        worst = max(worst, r)
+        assert r <= 1.0, f"{name}: logits differ at position {pos}: {r:.3f} of the 1e-2 budget"
+        check_token(tok_g, tok_c, lg_c, f"{name} pos {pos}")
+        near += tok_g != tok_c
+    assert near <= 1
+    assert gpu.model.attn_wo_error() == 0
+    # the rows this run appended to the cache (layer 1 sees layer 0's output)
+    hd, KV = cfg["dim"] // cfg["n_heads"], cfg["n_kv_heads"]
+    c = gpu.model.layers[1].attention.cache_kv.numpy().astype(np.float32)
+    assert np.allclose(c[0, 0, ctx:ctx + 6], cpu.cache_k[1, ctx:ctx + 6], rtol=1e-2, atol=1e-2)
+    assert np.allclose(c[1, 0, ctx:ctx + 6], cpu.cache_v[1, ctx:ctx + 6], rtol=1e-2, atol=1e-2)
+    assert np.array_equal(c[0, 0, ctx - 2:ctx], cpu.cache_k[1, ctx - 2:ctx])       # older rows untouched
+    print(f"{name}: worst logit ratio {worst:.3f} of the 1e-2 budget at {ctx}+ positions, KV {KV}x{hd}")
+
+
+def test_8b_int8_one_pass_over_512_positions_of_two_sequences():
+    """BASELINE config 5's prefill shape in small: tokens [2, 512] in ONE pass on top of 1024 cached positions per sequence
+    (tiled MFMA GEMMs at K = 4096 / 14336, causal attention over 1536 keys), against the oracle's several-row forward."""
+    name = "8B-int8"
+    cfg, gpu, cpu, _ = build(name)
+    B, S, start = 2, 512, 1024
+    cpu.set_batched(True)
+    for layer in gpu.model.layers:
+        layer.attention._ensure_cache("float16", gpu.device, B)
+    prompts = np.stack([synthetic.random_prompt(cfg, S, seed=50 + b) for b in range(B)]).astype(np.int32)
+    for b in range(B):
+        fill_cache(gpu, None, cfg, start, seed=70 + b, bsz=B, b=b)
+    tok = gpu.model.forward_rows(prompts, start).numpy()
+    lg = gpu.model.rows_logits().numpy().astype(np.float32)
+    caches = [layer.attention.cache_kv.numpy().astype(np.float32) for layer in gpu.model.layers]
+    for b in range(B):
+        fill_oracle_cache(cpu, cfg, start, seed=70 + b)
+        tok_c, lg_c = cpu.forward(prompts[b], start)
+        r = ratio(lg[b], lg_c)
+        assert r <= 1.0, f"sequence {b}: prefill logits {r:.3f} of the 1e-2 budget"
+        check_token(int(tok[b]), tok_c, lg_c, f"sequence {b}")
+        for l in range(cfg["n_layers"]):
+            assert np.allclose(caches[l][0, b, start:start + S], cpu.cache_k[l, start:start + S], rtol=1e-2, atol=1e-2), (b, l)
+            assert np.allclose(caches[l][1, b, start:start + S], cpu.cache_v[l, start:start + S], rtol=1e-2, atol=1e-2), (b, l)
+    cpu.set_batched(False)
+
+
+def test_8b_int8_batched_decode_step_of_16_sequences():
+    """BASELINE config 5's decode shape: one position for each of 16 sequences at 2112 visible positions (the few-row
+    weight-streaming GEMM, batched decode attention), against the oracle run per sequence with `batched` set."""
+    name = "8B-int8"
+    cfg, gpu, cpu, _ = build(name)
+    B, ctx = 16, FULL[name][1]
+    cpu.set_batched(True)
+    for layer in gpu.model.layers:
+        layer.attention._ensure_cache("float16", gpu.device, B)
+    for b in range(B):
+        fill_cache(gpu, None, cfg, ctx, seed=200 + b, bsz=B, b=b)
+    feed = synthetic.random_prompt(cfg, B, seed=9).astype(np.int32)
+    # two steps fed the same tokens; compared at the second, whose attention also reads the row the first step wrote
+    gpu.model.forward_rows(feed.reshape(B, 1), ctx)
+    tok = gpu.model.forward_rows(feed.reshape(B, 1), ctx + 1).numpy()
+    lg = gpu.model.rows_logits().numpy().astype(np.float32)
+    worst = 0.0
+    for b in range(B):
+        fill_oracle_cache(cpu, cfg, ctx, seed=200 + b)
+        cpu.forward([int(feed[b])], ctx)
+        tok_c, lg_c = cpu.forward([int(feed[b])], ctx + 1)
+        r = ratio(lg[b], lg_c)
+        worst = max(worst, r)
+        assert r <= 1.0, f"sequence {b}: batched decode logits {r:.3f} of the 1e-2 budget"
+        check_token(int(tok[b]), tok_c, lg_c, f"sequence {b}")
+    cpu.set_batched(False)
+    print(f"batched decode of 16: worst logit ratio {worst:.3f}")
+
+
+# ---------------------------------------------------------------- kernel level, full reduce lengths
+KINDS = {"float16": ffi.W_F16, "int8": ffi.W_I8, "nf4": ffi.W_NF4}
+_RNG = np.random.default_rng(41)
+
+
+def big_weight(kind, out_f, in_f):
+    w = _RNG.standard_normal((out_f, in_f), dtype=np.float32) * np.float32(0.02)
+    if kind == "float16":
+        return w.astype(np.float16), None
+    if kind == "int8":
+        return orc.int8_quantize(w)
+    return orc.nf4_quantize(w)
+
+
+def weight_rows(kind, w, s, out_f, in_f, idx):
+    """The rows `idx` of a weight as a smaller weight of the same format (output columns are independent)."""
+    if kind == "float16":
+        return np.ascontiguousarray(w[idx]), None
+    if kind == "int8":
+        return np.ascontiguousarray(w[idx]), np.ascontiguousarray(s[idx])
+    return np.ascontiguousarray(w.reshape(out_f, in_f // 2)[idx]).reshape(-1), np.ascontiguousarray(s.reshape(out_f, in_f // 64)[idx]).reshape(-1, 1)
+
+
+@pytest.mark.parametrize("kind", ["float16", "int8", "nf4"])
+@pytest.mark.parametrize("rows,out_f,in_f", [(256, 4096, 14336), (256, 14336, 4096), (16, 4096, 14336), (16, 128256, 4096)])
+def test_gemm_at_8b_reduce_lengths(hip, kind, rows, out_f, in_f):
+    """jsgrad_hip_gemm (tiled for 256 rows, weight-streaming for 16) with K = 4096 and 14336 against the oracle's several-row
+    Linear on a sample of 160 output columns (each column is its own sum) and every input row."""
+    if out_f == 128256 and kind == "nf4":
+        pytest.skip("the lm_head is never NF4 (llama3.ts:101)")
+    w, s = big_weight(kind, out_f, in_f)
+    x = _RNG.standard_normal((rows, in_f), dtype=np.float32).astype(np.float16)
+    res = _RNG.standard_normal((rows, out_f), dtype=np.float32).astype(np.float16)
+    tw, ts = Tensor(w), (Tensor(s) if s is not None else None)
+    tx, tr, ty = Tensor(x), Tensor(res), Tensor.empty((rows, out_f), "float16")
+    check(hip.jsgrad_hip_gemm(KINDS[kind], tw.ptr, ts.ptr if ts is not None else None, out_f, in_f, tx.ptr, rows, ty.ptr, tr.ptr))
+    idx = np.sort(_RNG.choice(out_f, 160, replace=False))
+    idx[0], idx[-1] = 0, out_f - 1
+    wi, si = weight_rows(kind, w, s, out_f, in_f, idx)
+    ref = orc.linear(wi, si, x, len(idx), in_f, True)
+    ref = (res[:, idx].astype(np.float32) + ref).astype(np.float16).astype(np.float32)
+    assert_close(ty.numpy()[:, idx].astype(np.float32), ref, True, f"gemm {kind} {rows}x{out_f}x{in_f}", composed=True)
+
+
+@pytest.mark.parametrize("kind", ["float16", "int8", "nf4"])
+@pytest.mark.parametrize("rows", [16, 256])
+def test_gemm_ffn_gate_at_8b_widths(hip, kind, rows):
+    """w1 and w3 of the 8B shape side by side (an output 2 x 14336 = 28672 wide over K = 4096) with the SwiGLU epilogue."""
+    dim, hidden = 4096, 14336
+    w1, s1 = big_weight(kind, hidden, dim)
+    w3, s3 = big_weight(kind, hidden, dim)
+    x = _RNG.standard_normal((rows, dim), dtype=np.float32).astype(np.float16)
+    t1, t3 = Tensor(w1), Tensor(w3)
+    ts1, ts3 = (Tensor(s1), Tensor(s3)) if s1 is not None else (None, None)
+    tx, tg = Tensor(x), Tensor.empty((rows, hidden), "float16")
+    p = lambda t: t.ptr if t is not None else None
+    check(hip.jsgrad_hip_gemm_ffn_gate(KINDS[kind], t1.ptr, p(ts1), t3.ptr, p(ts3), tx.ptr, rows, tg.ptr, dim, hidden))
+    idx = np.sort(_RNG.choice(hidden, 128, replace=False))
+    idx[0], idx[-1] = 0, hidden - 1
+    a = orc.linear(*weight_rows(kind, w1, s1, hidden, dim, idx), x, len(idx), dim, True)
+    u = orc.linear(*weight_rows(kind, w3, s3, hidden, dim, idx), x, len(idx), dim, True)
+    ref = (orc.silu(a.reshape(-1), True).reshape(a.shape) * u).astype(np.float16).astype(np.float32)
+    assert_close(tg.numpy()[:, idx].astype(np.float32), ref, True, f"ffn_gate {kind} {rows} rows", composed=True)
+
+
+@pytest.mark.parametrize("hd,H,KV", [(128, 32, 8), (64, 32, 8)])
+def test_attn_prefill_2048_positions_on_a_row_sample(hip, hd, H, KV):
+    """Causal attention over S = 2048 new positions (the benchmark's prompt length) at the 8B and 1B head layouts; a float64
+    reference on 24 query rows spread over the sequence (first, last, tile edges)."""
+    B, S, start = 1, 2048, 0
+    q = _RNG.standard_normal((S, H * hd), dtype=np.float32).astype(np.float16)
+    ck = _RNG.standard_normal((1, S, KV, hd), dtype=np.float32).astype(np.float16)
+    cv = _RNG.standard_normal((1, S, KV, hd), dtype=np.float32).astype(np.float16)
+    tq, tk, tv, to = Tensor(q), Tensor(ck), Tensor(cv), Tensor.empty((S, H * hd), "float16")
+    check(hip.jsgrad_hip_attn_prefill(tq.ptr, tk.ptr, tv.ptr, to.ptr, B, S, start, H, KV, hd, S))
+    got = to.numpy().astype(np.float64)
+    rows = sorted({0, 1, 63, 64, 127, 128, 129, 1023, 1024, 2046, 2047, *(int(r) for r in _RNG.integers(0, S, 13))})
+    for r in rows:
+        ref = attention_ref(q[r:r + 1], ck[:, :r + 1], cv[:, :r + 1], 1, 1, r, H, KV, hd)
+        assert np.allclose(got[r], ref[0], rtol=1e-2, atol=1e-2), r
+        assert np.max(np.abs(got[r] - ref[0])) < 4e-3, r

@@ -257,3 +257,53 @@ def test_argmax_lowest_index_on_ties():
         for perm in range(20):
             v = RNG.integers(0, 3, n).astype(np.float32)
             assert orc.argmax(v) == int(np.flatnonzero(v == v.max())[0])
+
+
+# ---------------------------------------------------------------- the several-row organisation and threads change nothing
+@pytest.mark.parametrize("kind", ["f32", "f16", "i8", "nf4"])
+def test_linear_rows_path_is_bit_identical_to_row_by_row(kind):
+    """or_linear_rows (tiles of input rows side by side, weight row converted once, outputs split over threads) must give
+    exactly the sums of the one-row routine evaluated row by row."""
+    rng = np.random.default_rng(11)
+    out_f, in_f = 70, 192
+    w = (rng.standard_normal((out_f, in_f)) * 0.05).astype(np.float32)
+    for n_rows in (2, 31, 32, 33, 67):
+        x = rng.standard_normal((n_rows, in_f)).astype(np.float16).astype(np.float32)
+        if kind == "f32":
+            args = (w, None)
+        elif kind == "f16":
+            args = (w.astype(np.float16), None)
+        elif kind == "i8":
+            args = orc.int8_quantize(w)
+        else:
+            args = orc.nf4_quantize(w)
+        act16 = kind != "f32"
+        ref = orc.linear(*args, x, out_f, in_f, act16, rowwise=True)
+        for threads in (1, 3):
+            orc.set_threads(threads)
+            try:
+                got = orc.linear(*args, x, out_f, in_f, act16)
+            finally:
+                orc.set_threads(1)
+            assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), (kind, n_rows, threads)
+
+
+def test_model_forward_does_not_depend_on_threads():
+    from denograd_amd import synthetic
+    from tests.helpers import quantize_state
+    cfg = dict(synthetic.config("tiny16"), quantize="int8", tied=True)
+    sd = quantize_state(cfg, synthetic.random_state_dict(cfg, seed=3))
+    toks = synthetic.random_prompt(cfg, 9, seed=3)
+    outs = []
+    for threads in (1, 4):
+        orc.set_threads(threads)
+        try:
+            m = orc.OracleModel(cfg, sd)
+            t1, lg1 = m.forward(toks[:6], 0)           # several rows
+            t2, lg2 = m.forward([int(toks[6])], 6)     # one row on top of the cache
+            outs.append((t1, lg1.copy(), t2, lg2.copy()))
+        finally:
+            orc.set_threads(1)
+    assert outs[0][0] == outs[1][0] and outs[0][2] == outs[1][2]
+    assert np.array_equal(outs[0][1].view(np.uint32), outs[1][1].view(np.uint32))
+    assert np.array_equal(outs[0][3].view(np.uint32), outs[1][3].view(np.uint32))
