@@ -54,6 +54,22 @@ template <typename AT, int HD> static int launch_attn(const AttnArgs &a, int n_r
   return 0;
 }
 
+// ---- the variant that allocates nothing: its workspace is a file-scope device array
+// Each GPU the library runs on holds its own copy of the array (at its own address) until the process ends.  In host code
+// the array's name is only a stand-in: the device address comes from hipGetSymbolAddress, once per device, and that
+// pointer is what kernels and fills are given.
+constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)8 << 20;
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+constexpr int NOALLOC_MAX_DEVICES = 64;
+static void *g_scratch_ptr[NOALLOC_MAX_DEVICES];   // per device, set on the first call there
+
+// the chunk counters must start at zero whatever an earlier call left behind (a fill kernel, not a memset node: callers may
+// be capturing a graph)
+__global__ void zero_words_kernel(int *p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
 }  // namespace jsg
 
 using namespace jsg;
@@ -91,6 +107,33 @@ int jsgrad_hip_attn_decode_batch(const void *q, const void *cache_k, const void 
   a.partial_bstride = (size_t)n_heads * 256 * (head_dim + 2);
   const int n_rep = n_heads / n_kv_heads;
   return head_dim == 64 ? launch_attn<_Float16, 64>(a, n_rep, batch) : launch_attn<_Float16, 128>(a, n_rep, batch);
+}
+
+size_t jsgrad_hip_attn_decode_static_max_bytes(void) { return NOALLOC_SCRATCH_BYTES; }
+
+int jsgrad_hip_attn_decode_static(const void *q, const void *cache_k, const void *cache_v, const int32_t *st, void *out, int n_heads, int n_kv_heads,
+                                  int head_dim, int max_context, int act) {
+  JSG_READY();
+  JSG_REQUIRE(q && cache_k && cache_v && st && out, "jsgrad_hip_attn_decode_static: null pointer argument");
+  JSG_REQUIRE(n_heads > 0 && n_kv_heads > 0 && max_context > 0, "jsgrad_hip_attn_decode_static: n_heads %d / n_kv_heads %d / max_context %d", n_heads, n_kv_heads, max_context);
+  JSG_REQUIRE(max_context <= 256 * ATT_CHUNK_MAX, "jsgrad_hip_attn_decode_static: max_context %d exceeds %d", max_context, 256 * ATT_CHUNK_MAX);
+  // counters [0, 256), then one partial result per (head, chunk): only the chunks this max_context can produce are needed
+  const size_t need = 256 + (size_t)n_heads * nsplit_for(max_context, 1) * ((size_t)head_dim + 2) * sizeof(float);
+  JSG_REQUIRE(need <= NOALLOC_SCRATCH_BYTES,
+              "jsgrad_hip_attn_decode_static: %d heads of %d at max_context %d need %zu bytes of workspace, the built-in one holds %zu; use jsgrad_hip_attn_decode "
+              "with a workspace of its own", n_heads, head_dim, max_context, need, (size_t)NOALLOC_SCRATCH_BYTES);
+  const int dev = state().device;
+  JSG_REQUIRE(dev >= 0 && dev < NOALLOC_MAX_DEVICES, "jsgrad_hip_attn_decode_static: device %d", dev);
+  if (g_scratch_ptr[dev] == nullptr) {   // once per device, with that device current (jsgrad_hip_init made it so)
+    void *p = nullptr;
+    JSG_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    JSG_REQUIRE(p != nullptr, "jsgrad_hip_attn_decode_static: no device address for the built-in workspace");
+    g_scratch_ptr[dev] = p;
+  }
+  void *ws = g_scratch_ptr[dev];
+  hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, state().stream, (int *)ws, 64);
+  JSG_LAUNCHED();
+  return jsgrad_hip_attn_decode(q, cache_k, cache_v, st, out, ws, n_heads, n_kv_heads, head_dim, max_context, act);
 }
 
 int jsgrad_hip_attn_decode(const void *q, const void *cache_k, const void *cache_v, const int32_t *st, void *out, void *workspace, int n_heads,

@@ -137,6 +137,17 @@ size_t jsgrad_hip_attn_workspace_bytes(int n_heads, int n_kv_heads, int head_dim
 int jsgrad_hip_attn_decode(const void *q, const void *cache_k, const void *cache_v, const int32_t *state, void *out, void *workspace,
                            int n_heads, int n_kv_heads, int head_dim, int max_context, int act);
 
+/* jsgrad_hip_attn_decode without the workspace argument, for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The partial
+ * results and chunk counters live in an array built into the library: jsgrad_hip_attn_decode_static_max_bytes() bytes
+ * (8 MiB) on every GPU the library runs on, held until the process ends.  The call allocates and frees nothing; shapes whose
+ * workspace (256 + n_heads * chunks(max_context) * (head_dim + 2) * 4 bytes, chunks <= 256) does not fit are refused with an
+ * error.  All calls on one GPU share the array: they are ordered by the library's stream; calls that overlap on one GPU
+ * (other streams, other threads) race.  Same results as jsgrad_hip_attn_decode, bit for bit. */
+size_t jsgrad_hip_attn_decode_static_max_bytes(void);
+int jsgrad_hip_attn_decode_static(const void *q, const void *cache_k, const void *cache_v, const int32_t *state, void *out,
+                                  int n_heads, int n_kv_heads, int head_dim, int max_context, int act);
+
 /* ffn_norm + w1, w3 + SwiGLU (FeedForward.call, models/llama.ts:108-110): g[hidden] = silu(w1 x) * (w3 x). */
 int jsgrad_hip_ffn_gate(int kind, const void *w1, const void *s1, const void *w3, const void *s3, const void *x,
                         const void *norm_weight, float eps, void *g, int dim, int hidden, int act);
