@@ -120,13 +120,16 @@ def read_only_launches(lib, cfg, T, attn_wo, reps=12):
     return {"families": fams, "step_ms": sum(fams.values()), "sizes_us": {str(b): round(1e3 * t, 2) for b, t in sorted(cache.items())}}
 
 
-def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=True, blocker_steps=40, per_op_steps=64, fused_step=False):
+def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=True, blocker_steps=40, per_op_steps=64, fused_step=False,
+                 prefill="serial", with_sampled=True):
+    """prefill: "serial" feeds the prompt token by token as the reference does (llama3.ts:307-311); "rows" feeds it in one
+    several-position pass (matrix-core GEMMs), which is what a long prompt takes in practice."""
     from denograd_amd import ffi, synthetic
     from denograd_amd.ffi import check
     from denograd_amd.llama3 import Llama3
 
     lib = ffi.load()
-    ctx = prompt_len + warmup + steps + 3 * (profile_steps + blocker_steps) + 2 * per_op_steps + 32
+    ctx = prompt_len + warmup + steps + 3 * (profile_steps + blocker_steps) + (2 * per_op_steps if with_sampled or fused_step else 0) + 32
     cfg = synthetic.config(name, max_context=ctx)
     t0 = time.perf_counter()
     llm = Llama3.from_config(cfg, fused_step=fused_step).random_init(seed=0, tied=cfg["tied"])
@@ -136,10 +139,12 @@ def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=Tru
     log(f"[{name}] weights on device in {time.perf_counter() - t0:.1f}s")
     prompt = [int(t) for t in synthetic.random_prompt(cfg, prompt_len, seed=0)]
     t0 = time.perf_counter()
+    llm.batched_prefill = prefill == "rows"
     llm._prefill(prompt[:-1])
     llm._call(prompt[-1])
     llm.start_pos += 1
-    log(f"[{name}] token-serial prefill of {prompt_len} tokens in {time.perf_counter() - t0:.2f}s")
+    llm.model._rows = None       # the several-row scratch of a one-pass prefill is not needed any more
+    log(f"[{name}] {'one-pass' if prefill == 'rows' else 'token-serial'} prefill of {prompt_len} tokens in {time.perf_counter() - t0:.2f}s")
 
     m = llm.model
     m.generate(warmup)
@@ -184,7 +189,7 @@ def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=Tru
     fused = m._fused is not None
     kinds = profiled(profile_steps)
     sampled = None
-    if not fused:
+    if not fused and with_sampled:
         # the same steps ending in the reference's default sampler (temperature 0.95, whole-vocabulary draw, llama3.ts:192)
         # instead of the greedy argmax: four small launches more per token
         m._set_sampling(0.95, 0, 0.0, 0.0, 0.0)
@@ -242,13 +247,38 @@ def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=Tru
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                 "bytes_per_launch": int(bytes_now), "avg_us_per_launch": round(step_ms * 1e3, 2)}
     else:
-        dom = "linear"   # w2 and the lm_head (and wo, when it is a launch of its own): the weight-streaming family with the most launches
+        # the lm_head on its own (the same event pairs, eager launches on cold-ish data), so that the `linear` family can be
+        # reported per matrix: one lm_head launch of ~0.5 GB and L launches of w2 (and wo where it is a launch of its own)
+        check(lib.jsgrad_hip_profile(1))
+        for _ in range(6):
+            m.output.call(m._ctx.h, out=m._ctx.logits, norm=m.norm)
+        n_, tot_ = C.c_int(), C.c_double()
+        check(lib.jsgrad_hip_profile_read(ffi.PROF_KINDS["linear"], C.byref(n_), C.byref(tot_)))
+        check(lib.jsgrad_hip_profile(0))
+        head_ms = tot_.value / max(1, n_.value)
+        V, d, L = cfg["vocab_size"], cfg["dim"], cfg["n_layers"]
+        head_b = (V * d + V * 2) if cfg["quantize"] == "int8" else V * d * 2
+        rest_n = fam["linear"]["launches_per_step"] - 1
+        rest_ms = max(1e-9, fam["linear"]["ms_per_step"] - head_ms)
+        rest_b = kb["linear"] - head_b
+        fam["linear"]["per_matrix"] = {
+            "lm_head": {"launches_per_step": 1, "bytes_per_launch": int(head_b), "avg_us_per_launch": round(1e3 * head_ms, 2), "GBps": round(head_b / (head_ms * 1e-3) / 1e9, 1)},
+            ("w2" if "attn_wo" in fam else "wo+w2"): {"launches_per_step": rest_n, "bytes_per_launch": int(rest_b / rest_n), "avg_us_per_launch": round(1e3 * rest_ms / rest_n, 2),
+                                                      "GBps": round(rest_b / (rest_ms * 1e-3) / 1e9, 1)}}
+        # the dominant kernel: the weight-streaming family the step spends the most time in
+        dom = max((k for k in kb if k in fam), key=lambda k: fam[k]["ms_per_step"])
+        kern = {"linear": "gemv_kernel<EPI_STORE> (w2, lm_head)", "ffn_gate": "gemv_kernel<EPI_SWIGLU> (ffn_norm + w1, w3 + SwiGLU)",
+                "qkv_rope": "gemv_kernel<EPI_ROPE_KV> (attention_norm + wq, wk, wv + rotary + cache write)",
+                "attn_wo": "attn_wo_kernel (decode attention + wo + residual)", "attn_decode": "attn_decode_kernel"}[dom]
         achieved = fam[dom]["GBps"]
-        roof = {"bound": "hbm", "kernel": f"gemv_kernel ({dom})", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        roof = {"bound": "hbm", "kernel": kern, "family": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get((name, dom, "attn_wo" in fam)),
                 "bytes_per_launch": int(kb[dom] / fam[dom]["launches_per_step"]), "avg_us_per_launch": round(fam[dom]["avg_us_per_launch"], 2),
+                "ms_per_step": round(fam[dom]["ms_per_step"], 4),
                 # the same launches as read-only kernels of the same sizes: the rate a launch of this size can reach at all
-                "read_only_GBps": round(kb[dom] / (read_only["families"][dom] * 1e-3) / 1e9, 1)}
+                "read_only_GBps": round(kb[dom] / (read_only["families"][dom] * 1e-3) / 1e9, 1),
+                "families": {k: {"ms_per_step": round(fam[k]["ms_per_step"], 4), "GBps": round(fam[k]["GBps"], 1), "frac": round(fam[k]["GBps"] / HBM_PEAK_GBS, 4)}
+                             for k in kb if k in fam}}
     rnd = lambda d: {k: {kk: (round(vv, 3) if isinstance(vv, float) else vv) for kk, vv in v.items()} for k, v in d.items()}
     res = {
         "name": name, "tok_s": tok_s, "ms_per_step": 1e3 * wall / steps, "event_ms_per_step": ms.value / steps,
@@ -268,7 +298,7 @@ def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=Tru
     return llm, cfg, res
 
 
-def cpu_baseline(llm, cfg, budget_s=15.0):
+def cpu_baseline(llm, cfg, budget_s=15.0, n_prompt=4):
     """Time the oracle on the host (1 thread) on the same weights and check its tokens against the GPU's."""
     import oracle as orc
     from denograd_amd import synthetic
@@ -279,7 +309,8 @@ def cpu_baseline(llm, cfg, budget_s=15.0):
     log(f"[cpu] weights copied to host in {time.perf_counter() - t0:.1f}s")
     ocfg = dict(cfg, max_context=64)
     cpu = orc.OracleModel(ocfg, sd)
-    prompt = [int(t) for t in synthetic.random_prompt(cfg, 4, seed=7)]
+    orc.set_threads(1)          # the reference's CLANG device runs one thread
+    prompt = [int(t) for t in synthetic.random_prompt(cfg, n_prompt, seed=7)]
     t0 = time.perf_counter()
     cpu.forward([prompt[0]], 0, want_logits=False)
     per = time.perf_counter() - t0
@@ -455,6 +486,8 @@ def main():
     ap.add_argument("--workload", default="1B", help="primary synthetic config (denograd_amd/synthetic.py)")
     ap.add_argument("--secondary", default="8B-int8", help="second workload measured in the same run ('' to skip)")
     ap.add_argument("--secondary-steps", type=int, default=128)
+    ap.add_argument("--others", default="3B-int8:1024:64,8B-nf4:4096:64", help="further bs=1 decode legs as name:prompt:steps (the remaining BASELINE configurations; "
+                    "their prompts are fed in one several-position pass); '' to skip")
     ap.add_argument("--batched", default="8B-int8", help="workload of the batched prefill + batched decode leg ('' to skip)")
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--batch-prompt", type=int, default=2048)
@@ -488,10 +521,20 @@ def main():
     llm, cfg, res = run_workload(args.workload, args.prompt, args.steps, args.warmup, use_graph=not args.no_graph, fused_step=step_mode)
     cpu = None if args.no_cpu else cpu_baseline(llm, cfg)
     del llm
-    secondary = None
+    secondary, cpu2 = None, None
     if args.secondary:
         llm2, cfg2, secondary = run_workload(args.secondary, args.prompt, args.secondary_steps, args.warmup, use_graph=not args.no_graph, fused_step=step_mode)
+        cpu2 = None if args.no_cpu else cpu_baseline(llm2, cfg2, budget_s=12.0, n_prompt=2)
         del llm2
+    others = {}
+    for spec in filter(None, args.others.split(",")):
+        oname, oprompt, osteps = spec.split(":")
+        llm3, cfg3, r3 = run_workload(oname, int(oprompt), int(osteps), args.warmup, profile_steps=4, use_graph=not args.no_graph, fused_step=False,
+                                      prefill="rows", with_sampled=False)
+        del llm3
+        others[oname] = {"value": round(r3["tok_s"], 2), "unit": "tok/s", "steps": int(osteps), "ms_per_step": round(r3["ms_per_step"], 4),
+                         "dtype": f"{cfg3['quantize']} weights, f16 activations", "config": r3["config"], "roofline": r3["roofline"],
+                         "step_roofline": r3["step_roofline"], "kernels": r3["kernels"]}
 
     out = {
         "metric": "decode tok/s bs=1 + % HBM roofline, Llama-3.2-1B fp16 & 8B int8",
@@ -506,7 +549,9 @@ def main():
         out["secondary"] = {"value": round(secondary["tok_s"], 2), "unit": "tok/s", "steps": args.secondary_steps, "ms_per_step": round(secondary["ms_per_step"], 4),
                             "dtype": "i8 weights, f16 activations", "config": secondary["config"], "roofline": secondary["roofline"],
                             "step_roofline": secondary["step_roofline"], "kernels": secondary["kernels"], "per_op_path": secondary.get("per_op_path"),
-                            "sampled": secondary.get("sampled")}
+                            "sampled": secondary.get("sampled"), "cpu_baseline": cpu2}
+    if others:
+        out["others"] = others
     if args.batched:
         out["batched"] = run_batched(args.batched, args.batch, args.batch_prompt, args.batch_steps)
     out["formats"] = run_formats()

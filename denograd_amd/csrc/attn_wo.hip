@@ -64,20 +64,50 @@ static int aw_nsplit(int max_context) {
   return by_lds > wanted ? by_lds : wanted;
 }
 
-template <int KIND, int HD> static int launch_attn_wo(const AttnArgs &at, const GemvArgs &a, int n_rep, int layer, int out_f) {
+// Blocks of attn_wo_kernel<KIND, HD, n_rep> the device can hold at once (occupancy x CUs).  The blocks that run attention
+// items are the first `items` of the grid; the rest, and the attention blocks themselves once their item is done, wait in
+// the wo part for the attention row.  If more items existed than blocks fit the device, the waiting blocks could keep
+// item blocks from ever starting, so such a launch is refused.
+template <int KIND, int HD> static int aw_capacity(int n_rep, size_t lds, int *out) {
+  int per_cu = 0;
+#define JSG_REP(N)                                                                                                                      \
+  case N:                                                                                                                               \
+    JSG_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void *)attn_wo_kernel<KIND, HD, N>, AW_THREADS, lds));          \
+    break;
+  switch (n_rep) {
+    JSG_REP(1) JSG_REP(2) JSG_REP(3) JSG_REP(4)
+    default: return fail("jsgrad_hip_attn_wo: n_heads/n_kv_heads = %d is not one of 1,2,3,4", n_rep);
+  }
+#undef JSG_REP
+  *out = per_cu * state().cu_count;
+  return 0;
+}
+
+template <int KIND, int HD> static int launch_attn_wo(const AttnArgs &at, const GemvArgs &a, int n_rep, int layer, int out_f, int *query_capacity) {
   const int ngroups = (out_f + 1) / 2, need = (ngroups + 3) / 4;
   const int cap = state().cu_count * 4;
   int blocks = need < cap ? need : cap;
   const int items = at.n_kv_heads * at.nsplit;
   if (blocks < items) blocks = items;
   const size_t lds = (size_t)Gemv<KIND, _Float16, EPI_STORE, 2, 4, false>::x_elems(a.in_f) * sizeof(_Float16);
+  // capacity per (kernel instance, staging size): asked for once, the answer does not change
+  static int cached_capacity[5] = {0, 0, 0, 0, 0};
+  static size_t cached_lds[5] = {0, 0, 0, 0, 0};
+  if (n_rep < 1 || n_rep > 4) return fail("jsgrad_hip_attn_wo: n_heads/n_kv_heads = %d is not one of 1,2,3,4", n_rep);
+  if (cached_capacity[n_rep] == 0 || cached_lds[n_rep] != lds) {
+    if (int e = aw_capacity<KIND, HD>(n_rep, lds, &cached_capacity[n_rep])) return e;
+    cached_lds[n_rep] = lds;
+  }
+  if (query_capacity) { *query_capacity = cached_capacity[n_rep]; return 0; }
+  JSG_REQUIRE(items <= cached_capacity[n_rep],
+              "jsgrad_hip_attn_wo: %d attention items (%d kv heads x %d chunks of the context) but the device holds %d blocks of this kernel at once; "
+              "use jsgrad_hip_attn_decode + jsgrad_hip_linear for this shape", items, at.n_kv_heads, at.nsplit, cached_capacity[n_rep]);
 #define JSG_REP(N)                                                                                                   \
   case N:                                                                                                            \
     JSG_LAUNCH(PROF_ATTN_WO, (attn_wo_kernel<KIND, HD, N>), dim3(blocks), dim3(AW_THREADS), lds, at, a, layer);       \
     break;
   switch (n_rep) {
     JSG_REP(1) JSG_REP(2) JSG_REP(3) JSG_REP(4)
-    default: return fail("jsgrad_hip_attn_wo: n_heads/n_kv_heads = %d is not one of 1,2,3,4", n_rep);
   }
 #undef JSG_REP
   return 0;
@@ -95,12 +125,15 @@ size_t jsgrad_hip_attn_wo_workspace_bytes(int n_heads, int n_kv_heads, int head_
   return 512 + (size_t)n_heads * 256 * (head_dim + 2) * sizeof(float) + (size_t)n_heads * head_dim * sizeof(uint32_t);
 }
 
-int jsgrad_hip_attn_wo(const void *q, const void *cache_k, const void *cache_v, const int32_t *st, void *workspace, int n_heads, int n_kv_heads,
-                       int head_dim, int max_context, int kind, const void *wo, const void *so, int dim, const void *residual, void *y, int layer) {
+int jsgrad_hip_attn_wo_items(int n_kv_heads, int max_context) { return n_kv_heads * aw_nsplit(max_context); }
+
+static int attn_wo_impl(const void *q, const void *cache_k, const void *cache_v, const int32_t *st, void *workspace, int n_heads, int n_kv_heads,
+                        int head_dim, int max_context, int kind, const void *wo, const void *so, int dim, const void *residual, void *y, int layer,
+                        int *query_capacity) {
   JSG_READY();
-  JSG_REQUIRE(q && cache_k && cache_v && st && workspace && wo && y, "jsgrad_hip_attn_wo: null pointer argument");
+  if (!query_capacity) JSG_REQUIRE(q && cache_k && cache_v && st && workspace && wo && y, "jsgrad_hip_attn_wo: null pointer argument");
   JSG_REQUIRE(kind == JSGRAD_W_F16 || kind == JSGRAD_W_I8, "jsgrad_hip_attn_wo: weight kind %d (fp16 and int8 are built)", kind);
-  JSG_REQUIRE(kind == JSGRAD_W_F16 || so, "jsgrad_hip_attn_wo: quantised weight needs a scale");
+  JSG_REQUIRE(kind == JSGRAD_W_F16 || so || query_capacity, "jsgrad_hip_attn_wo: quantised weight needs a scale");
   JSG_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_kv_heads <= 64 && n_heads % n_kv_heads == 0, "jsgrad_hip_attn_wo: n_heads %d / n_kv_heads %d", n_heads, n_kv_heads);
   JSG_REQUIRE(head_dim == 64 || head_dim == 128, "jsgrad_hip_attn_wo: head_dim %d (64 and 128 are built)", head_dim);
   JSG_REQUIRE(max_context > 0 && max_context <= 64 * ATT_CHUNK_MAX, "jsgrad_hip_attn_wo: max_context %d exceeds %d", max_context, 64 * ATT_CHUNK_MAX);
@@ -123,13 +156,28 @@ int jsgrad_hip_attn_wo(const void *q, const void *cache_k, const void *cache_v, 
   a.err = (int *)(ws + 256);
   const int n_rep = n_heads / n_kv_heads;
 #define JSG_KIND(K) \
-  case K: return head_dim == 64 ? launch_attn_wo<K, 64>(at, a, n_rep, layer, dim) : launch_attn_wo<K, 128>(at, a, n_rep, layer, dim);
+  case K: return head_dim == 64 ? launch_attn_wo<K, 64>(at, a, n_rep, layer, dim, query_capacity) : launch_attn_wo<K, 128>(at, a, n_rep, layer, dim, query_capacity);
   switch (kind) {
     JSG_KIND(JSGRAD_W_F16)
     JSG_KIND(JSGRAD_W_I8)
   }
 #undef JSG_KIND
   return fail("jsgrad_hip_attn_wo: weight kind %d", kind);
+}
+
+int jsgrad_hip_attn_wo(const void *q, const void *cache_k, const void *cache_v, const int32_t *st, void *workspace, int n_heads, int n_kv_heads,
+                       int head_dim, int max_context, int kind, const void *wo, const void *so, int dim, const void *residual, void *y, int layer) {
+  return attn_wo_impl(q, cache_k, cache_v, st, workspace, n_heads, n_kv_heads, head_dim, max_context, kind, wo, so, dim, residual, y, layer, nullptr);
+}
+
+int jsgrad_hip_attn_wo_fits(int n_heads, int n_kv_heads, int head_dim, int max_context, int kind, int dim, int *host_out_items, int *host_out_capacity) {
+  JSG_REQUIRE(host_out_items && host_out_capacity, "jsgrad_hip_attn_wo_fits: null pointer");
+  int cap = 0;
+  if (int e = attn_wo_impl(nullptr, nullptr, nullptr, nullptr, nullptr, n_heads, n_kv_heads, head_dim, max_context, kind, nullptr, nullptr, dim, nullptr, nullptr, 0, &cap))
+    return e;
+  *host_out_items = jsgrad_hip_attn_wo_items(n_kv_heads, max_context);
+  *host_out_capacity = cap;
+  return 0;
 }
 
 int jsgrad_hip_attn_wo_status(const void *workspace, int *host_out_error) {

@@ -171,7 +171,10 @@ __device__ __forceinline__ float row8_sum(float v) {
 // A row that blocks of one launch hand to each other: one 32-bit word per element, the fp16 value below, a version tag
 // above.  A reader asks for the words and takes them once every tag is the one it expects: no flag, and the writer does
 // not have to wait for its stores to be acknowledged before anything.
-__device__ __forceinline__ uint32_t tw_tag(int version) { return (uint32_t)version % 65535u + 1u; }   // never 0: fresh memory matches nothing
+// The tag is the version modulo 65535, plus one (never 0: fresh or cleared memory matches nothing).  Two versions that differ
+// by a multiple of 65535 share a tag, so a tag tells launches apart only among versions close to each other: rows are
+// rewritten in full by every launch, and whoever makes the version jump (the host moving the decode position) clears the row.
+__device__ __forceinline__ uint32_t tw_tag(int version) { return (uint32_t)version % 65535u + 1u; }
 __device__ __forceinline__ void tw_store(uint32_t *p, uint32_t tag, float v) {
   const _Float16 h = (_Float16)v;
   st_coherent((int *)p, (int)((tag << 16) | (uint32_t)__builtin_bit_cast(uint16_t, h)));

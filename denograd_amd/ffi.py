@@ -63,6 +63,8 @@ SIGNATURES: dict[str, tuple[list, object]] = {
     "jsgrad_hip_attn_wo_workspace_bytes": ([_i32, _i32, _i32], _sz),
     "jsgrad_hip_attn_wo": ([_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp, _i32], _i32),
     "jsgrad_hip_attn_wo_status": ([_vp, C.POINTER(_i32)], _i32),
+    "jsgrad_hip_attn_wo_items": ([_i32, _i32], _i32),
+    "jsgrad_hip_attn_wo_fits": ([_i32, _i32, _i32, _i32, _i32, _i32, C.POINTER(_i32), C.POINTER(_i32)], _i32),
     "jsgrad_hip_ffn_gate": ([_i32, _vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _i32, _i32, _i32], _i32),
     "jsgrad_hip_argmax": ([_vp, _i32, _vp, _vp, _i32, _i32, _i32], _i32),
     "jsgrad_hip_embed_rows": ([_i32, _vp, _vp, _vp, _i32, _vp, _i32, _i32], _i32),

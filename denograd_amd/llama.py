@@ -130,6 +130,18 @@ class TransformerBlock:
         return self.feed_forward.call_rows(rows.xn, n, rows, residual=h, out=x)
 
 
+def attn_wo_fits(n_heads: int, n_kv_heads: int, head_dim: int, max_context: int, kind: int, dim: int, capacity: int | None = None) -> bool:
+    """Whether attention and wo of this shape may share a launch: every block that runs an attention item (kv heads x chunks
+    of the context) must be on the device at once, because the blocks that are done wait there for the attention row.
+    `capacity`: blocks of that kernel the device holds at once (asked of the library when not given)."""
+    lib = ffi.load()
+    if capacity is None:
+        items, cap = C.c_int(0), C.c_int(0)
+        check(lib.jsgrad_hip_attn_wo_fits(n_heads, n_kv_heads, head_dim, max_context, kind, dim, C.byref(items), C.byref(cap)))
+        return items.value <= cap.value
+    return lib.jsgrad_hip_attn_wo_items(n_kv_heads, max_context) <= capacity
+
+
 class _Scratch:
     """Per-model activation rows and the attention workspace, allocated once (nothing is allocated per token)."""
 
@@ -149,7 +161,17 @@ class _Scratch:
     def enable_attn_wo(self, n_heads: int, n_kv_heads: int, head_dim: int, device: str) -> None:
         nbytes = ffi.load().jsgrad_hip_attn_wo_workspace_bytes(n_heads, n_kv_heads, head_dim)
         self.attn_wo_ws = Tensor.zeros((nbytes,), "uint8", device)
+        self._tagged_row_bytes = n_heads * head_dim * 4
         self.fuse_attn_wo = True
+
+    def clear_attn_row(self) -> None:
+        """Wipe the attention row that the blocks of a fused attention + wo launch hand to each other.  Its words carry a
+        16-bit tag made from (position, layer) modulo 65535, unique among CONSECUTIVE launches (each rewrites the whole row);
+        after a jump of the position an old row could carry the tag a new launch expects (128 * dpos = dlayer mod 65535), so
+        whoever moves the position clears the row: tag 0 matches no launch."""
+        if self.attn_wo_ws is not None:
+            ws = self.attn_wo_ws
+            check(ffi.load().jsgrad_hip_memset(ws.ptr + ws.nbytes - self._tagged_row_bytes, 0, self._tagged_row_bytes))
 
 
 class _RowScratch:
@@ -296,6 +318,13 @@ class Transformer:
         check(ffi.load().jsgrad_hip_attn_wo_status(self._ctx.attn_wo_ws.ptr, C.byref(e)))
         return e.value
 
+    def check_errors(self) -> None:
+        """Raise if a bounded wait inside a fused attention + wo launch ran out since the model was made (another process
+        holding compute units, or a device fault): the tokens after that point are not to be trusted.  Called wherever
+        the host waits for the device anyway (the per-token read of Llama3._call, the end of Llama3.generate)."""
+        if self.attn_wo_error():
+            raise ffi.HipError("a fused attention + wo launch gave up waiting for its attention row; results after that launch are invalid")
+
     # ---- plumbing
     @property
     def dtype(self) -> str:
@@ -314,15 +343,17 @@ class Transformer:
                 layer.attention.layer_id = i
             wo = self.layers[0].attention.wo
             if (self.fuse_attn_wo and self.dtype == "float16" and wo.kind in (ffi.W_F16, ffi.W_I8) and 2 <= len(self.layers) <= 128 and hd in (64, 128)
-                    and self.n_heads // self.n_kv_heads in (1, 2, 3, 4) and self.max_context <= 64 * 256 and self.n_heads * hd * 2 <= 64 * 1024):
+                    and self.n_heads // self.n_kv_heads in (1, 2, 3, 4) and self.max_context <= 64 * 256 and self.n_heads * hd * 2 <= 64 * 1024
+                    and self.n_kv_heads <= 64 and attn_wo_fits(self.n_heads, self.n_kv_heads, hd, self.max_context, wo.kind, self.dim)):
                 self._ctx.enable_attn_wo(self.n_heads, self.n_kv_heads, hd, self.device)
             if self.fused_step:
                 self._fused = _FusedStep(self, self._ctx, self._fused_mode())      # raises NotImplementedError for models it was not built for
         return self._ctx
 
-    def _step(self) -> Tensor:
-        """One decode step for the token / position in `state`; leaves the greedy token in state[0] and
-        advances state[1].  Pure kernel launches: safe to capture."""
+    def _step(self, draw: bool = True) -> Tensor:
+        """One decode step for the token / position in `state`; leaves the picked token in state[0] and
+        advances state[1].  Pure kernel launches: safe to capture.  draw=False: the token of this position is not wanted
+        (an inner position of a several-token call), so nothing is drawn from the random stream; the argmax fills in."""
         ctx = self._prepare()
         if self._pos >= self.max_context:
             raise ValueError(f"KV cache of {self.max_context} positions is full")
@@ -334,14 +365,14 @@ class Transformer:
         for layer in self.layers:
             h = layer.call(h, self.state, self.freqs_cis, ctx)
         self.output.call(h, out=ctx.logits, norm=self.norm)
-        self._pick_token(ctx.logits)
+        self._pick_token(ctx.logits, draw)
         return Tensor(buffer=self.state.lazydata.view(1, "int32", 0), shape=(), dtype="int32", device=self.device)
 
-    def _pick_token(self, logits: Tensor) -> None:
+    def _pick_token(self, logits: Tensor, draw: bool = True) -> None:
         """`sample(logits.flatten(), ...)` (llama.ts:212): the token goes to state[0], the position advances."""
         lib = ffi.load()
         temp, k, p, af, ap = self._sampling
-        if temp < 1e-6:
+        if temp < 1e-6 or not draw:
             check(lib.jsgrad_hip_argmax(logits.ptr, self.vocab_size, self.state.ptr, self.tokens_out.ptr, self.max_context, 1, act_code(self.dtype)))
             return
         if self._sample_ws is None:
@@ -378,6 +409,8 @@ class Transformer:
         if not (0 <= token < self.vocab_size):
             raise ValueError(f"token {token} outside the vocabulary of {self.vocab_size}")
         self.state.lazydata.copyin(np.array([token, start_pos], np.int32))
+        if start_pos != self._pos and self._ctx is not None:
+            self._ctx.clear_attn_row()      # the position jumps: see _Scratch.clear_attn_row
         self._pos = start_pos
 
     @property
@@ -389,22 +422,26 @@ class Transformer:
     def forward(self, tokens, start_pos: int, temperature: float = 0.0, top_k: int = 0, top_p: float = 0.8, alpha_f: float = 0.0, alpha_p: float = 0.0) -> Tensor:
         """llama.ts:201-213 for one sequence.  Several tokens are fed position by position (the reference's own
         prefill is token-serial, models/llama3.ts:307-311); the returned tensor is the token picked after the last one
-        (every position draws, as in the reference: each one advances the random counter and the alpha counter)."""
+        and it is the only draw of the call: the reference samples once, from the logits of the last position
+        (llama.ts:210-212), so one call advances the random counter and the alpha counter by one whatever seqlen is.
+        Llama3._prefill calls with one token each, so there every position draws, as in the reference)."""
         self._set_sampling(temperature, top_k, top_p, alpha_f, alpha_p)
         toks = np.asarray(tokens.numpy() if isinstance(tokens, Tensor) else tokens, np.int32)
         if toks.ndim != 2 or toks.shape[0] != 1:
             raise ValueError(f"tokens must have shape [1, seqlen], got {toks.shape}; several sequences go through forward_rows")
         ret = None
+        n = toks.shape[1]
         for i, t in enumerate(toks[0]):
             self.set_state(int(t), start_pos + i)
-            ret = self._step()
+            ret = self._step(draw=(i == n - 1))
         return ret
 
-    def forward_rows(self, tokens, start_pos: int) -> Tensor:
+    def forward_rows(self, tokens, start_pos: int, temperature: float = 0.0, top_k: int = 0, top_p: float = 0.8, alpha_f: float = 0.0, alpha_p: float = 0.0) -> Tensor:
         """llama.ts:201-213 for tokens of shape [bsz, seqlen] in ONE pass: every Linear is a matrix-core GEMM over all
-        bsz*seqlen rows, attention is causal over cache rows [0, start_pos + s].  Returns the greedy next token of every
-        sequence, an int32 tensor [bsz] (the reference flattens the logits of all sequences into one argmax,
-        llama.ts:212, which is only meaningful for bsz == 1).  fp16 activations; fp16 / int8 / NF4 weights.
+        bsz*seqlen rows, attention is causal over cache rows [0, start_pos + s].  Returns the next token of every
+        sequence, an int32 tensor [bsz]: for one sequence picked like `forward` does (one draw from the last position's
+        logits at temperature > 0), for several the greedy one (the reference flattens the logits of all sequences into
+        one sample, llama.ts:212, which is only meaningful for bsz == 1).  fp16 activations; fp16 / int8 / NF4 weights.
         `tokens` may be a device int32 tensor [bsz, seqlen] (e.g. the tensor a previous call returned, reshaped)."""
         lib = ffi.load()
         ctx = self._prepare()
@@ -425,6 +462,8 @@ class Transformer:
             tok_dev = None
         if bsz < 1 or seqlen < 1:
             raise ValueError(f"empty token tensor {bsz}x{seqlen}")
+        if temperature >= 1e-6 and bsz != 1:
+            raise NotImplementedError("sampling is defined for one sequence; several sequences are decoded greedily")
         if not (0 <= start_pos and start_pos + seqlen <= self.max_context):
             raise ValueError(f"positions [{start_pos}, {start_pos + seqlen}) outside the KV cache of {self.max_context} positions")
         hd = self.dim // self.n_heads
@@ -447,6 +486,7 @@ class Transformer:
                                         self.dim, self.vocab_size))
         # the attention of a one-position call reads the position from the device state word, like the one-row kernels
         self.state.lazydata.ensure_allocated().copyin(np.array([0, start_pos + seqlen - 1], np.int32))
+        ctx.clear_attn_row()     # the position moves by more than one: see _Scratch.clear_attn_row
         h = rows.h
         for layer in self.layers:
             h = layer.call_rows(h, bsz, seqlen, start_pos, self.state, self.freqs_cis, rows)
@@ -469,7 +509,8 @@ class Transformer:
                                           ctx.logits.ptr, None))
             else:
                 out.call(Tensor(buffer=last.lazydata.view(self.dim, "float16", 0), shape=(self.dim,), dtype="float16", device=self.device), out=ctx.logits, norm=self.norm)
-            check(lib.jsgrad_hip_argmax(ctx.logits.ptr, self.vocab_size, self.state.ptr, self.tokens_out.ptr, self.max_context, 1, act_code(self.dtype)))
+            self._set_sampling(temperature, top_k, top_p, alpha_f, alpha_p)
+            self._pick_token(ctx.logits)
             check(lib.jsgrad_hip_copy(rows.next_tokens.ptr, self.state.ptr, 4))
             self._pos = start_pos + seqlen
         else:

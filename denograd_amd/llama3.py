@@ -115,7 +115,7 @@ class Llama3:
     """llama3.ts:170-338 without the download / tokenizer plumbing: construct from shape parameters (`size` or an
     explicit `args` dict), load a state dict, then `_prefill` / `_call` / `generate` token ids."""
 
-    def __init__(self, size: str | None = None, quantize: str | None = None, device: str = "HIP", max_context: int = 8192, temperature: float = 0.0,
+    def __init__(self, size: str | None = None, quantize: str | None = None, device: str = "HIP", max_context: int = 8192, temperature: float = 0.95,
                  top_k: int = 0, top_p: float = 0.0, alpha_f: float = 0.0, alpha_p: float = 0.0, args: dict | None = None, fused_step: bool = False):
         # quantize: None (tensors as loaded), "float16" (every tensor cast to float16, llama3.ts:234), "int8", "nf4"
         self.cast_float16 = quantize == "float16"
@@ -137,10 +137,12 @@ class Llama3:
 
     # ---- loading
     @staticmethod
-    def from_config(cfg: dict, device: str = "HIP", fused_step: bool = False) -> "Llama3":
+    def from_config(cfg: dict, device: str = "HIP", fused_step: bool = False, temperature: float = 0.0) -> "Llama3":
+        """A model of a synthetic configuration (denograd_amd/synthetic.py).  Greedy unless told otherwise: the parity and
+        benchmark runs compare argmax tokens; the constructor itself defaults to the reference's temperature 0.95 (llama3.ts:192)."""
         args = {k: cfg[k] for k in ("dim", "hidden_dim", "n_heads", "n_kv_heads", "n_layers", "norm_eps", "rope_theta", "vocab_size")}
         q = cfg["quantize"] if cfg["quantize"] in ("int8", "nf4") else None
-        return Llama3(quantize=q, device=device, max_context=cfg["max_context"], args=args, fused_step=fused_step)
+        return Llama3(quantize=q, device=device, max_context=cfg["max_context"], temperature=temperature, args=args, fused_step=fused_step)
 
     def load_weights(self, weights: dict, quantized: bool = False) -> "Llama3":
         """llama3.ts:233-255: `weights` holds unquantised Meta-style tensors (host arrays or device Tensors) unless
@@ -226,7 +228,9 @@ class Llama3:
     def _call(self, tok: int) -> int:
         """llama3.ts:334-337: one model call and the per-token device->host read."""
         res = self.model.call(np.array([[tok]], np.int32), self.start_pos, self.temperature, self.top_k, self.top_p, self.alpha_f, self.alpha_p)
-        return int(res.item())
+        tok = int(res.item())
+        self.model.check_errors()
+        return tok
 
     def _prefill(self, toks: list[int]) -> None:
         """llama3.ts:297-312: skip the shared prefix of the previous prompt when starting over, then feed tokens one at a time."""
@@ -238,7 +242,7 @@ class Llama3:
             self.last_seen_toks = toks
             toks = toks[i:]
         if self.batched_prefill and len(toks) > 1:
-            self.model.forward_rows(np.array([toks], np.int32), self.start_pos)
+            self.model.forward_rows(np.array([toks], np.int32), self.start_pos, self.temperature, self.top_k, self.top_p, self.alpha_f, self.alpha_p)
             self.start_pos += len(toks)
             return
         for tok in toks:
@@ -333,6 +337,7 @@ class Llama3:
             self.model.generate(n_new - 1)
             self.start_pos += n_new - 1
         hist = self.model.tokens_out.numpy()
+        self.model.check_errors()
         out = hist[first_pos:first_pos + n_new].astype(np.int32)
         assert out[0] == first
         return out

@@ -268,6 +268,12 @@ size_t jsgrad_hip_attn_wo_workspace_bytes(int n_heads, int n_kv_heads, int head_
 int jsgrad_hip_attn_wo(const void *q, const void *cache_k, const void *cache_v, const int32_t *state, void *workspace, int n_heads, int n_kv_heads,
                        int head_dim, int max_context, int kind, const void *wo, const void *wo_scale, int dim, const void *residual, void *y, int layer);
 int jsgrad_hip_attn_wo_status(const void *workspace, int *host_out_error);
+/* Launch geometry of jsgrad_hip_attn_wo.  _items: blocks that run an attention item (kv heads x chunks of max_context; plain
+ * arithmetic, needs no device).  _fits: that number and the number of blocks of the kernel the device holds at once; a launch
+ * with more items than that is refused by jsgrad_hip_attn_wo (blocks that are done wait on the device for the attention row,
+ * so every item block must be resident), and the caller runs jsgrad_hip_attn_decode + jsgrad_hip_linear instead. */
+int jsgrad_hip_attn_wo_items(int n_kv_heads, int max_context);
+int jsgrad_hip_attn_wo_fits(int n_heads, int n_kv_heads, int head_dim, int max_context, int kind, int dim, int *host_out_items, int *host_out_capacity);
 
 /* ---------------------------------------------------------------------------------
  * Load-time kernels

@@ -62,3 +62,21 @@ def test_product_does_not_import_the_oracle():
                 src = open(os.path.join(dirpath, f)).read()
                 assert not re.search(r"^\s*(import|from)\s+oracle\b", src, flags=re.M), f"{f} imports the oracle"
                 assert "liboracle" not in src
+
+
+def test_attention_wo_launch_capacity_rule():
+    """Attention and wo share a launch only when every block that runs an attention item fits the device at once (blocks that
+    are done wait there for the attention row).  The item count is plain arithmetic in the library; the decision is made
+    against a given capacity here (on a GPU the library asks the occupancy calculator)."""
+    from denograd_amd.llama import attn_wo_fits
+    lib = ffi.load()
+    # chunks of the context: one per 32 positions, at most 64, at least one per 256 positions
+    assert lib.jsgrad_hip_attn_wo_items(8, 841) == 8 * 27
+    assert lib.jsgrad_hip_attn_wo_items(8, 2304) == 8 * 64
+    assert lib.jsgrad_hip_attn_wo_items(2, 64) == 2 * 2
+    assert lib.jsgrad_hip_attn_wo_items(8, 16384) == 8 * 64
+    cap = 4 * 256      # four blocks of 256 threads per compute unit
+    assert attn_wo_fits(32, 8, 128, 8192, ffi.W_I8, 4096, capacity=cap)            # the 8B shape: 512 items
+    assert not attn_wo_fits(32, 32, 64, 2048, ffi.W_F16, 2048, capacity=cap)       # 32 kv heads x 64 chunks = 2048 items
+    assert attn_wo_fits(32, 32, 64, 1024, ffi.W_F16, 2048, capacity=cap)           # 32 x 32 = 1024 items just fit
+    assert not attn_wo_fits(64, 64, 64, 2048, ffi.W_F16, 4096, capacity=cap)

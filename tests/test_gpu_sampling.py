@@ -128,3 +128,25 @@ def test_model_samples_what_the_restatement_draws_from_its_logits():
     assert len(set(a)) > 4                                         # not stuck on one token
     run(7, 0.8, 12, 0.9, 0.4, 0.2)                                 # top-k / top-p / alpha through the model
     assert run(7, temperature=0.0, check_draws=False) == run(9, temperature=0.0, check_draws=False)      # greedy ignores the seed
+
+
+def test_one_draw_per_forward_call_whatever_the_sequence_length(hip):
+    """Transformer.forward on [1, S] samples once, from the last position's logits (llama.ts:210-212): the random counter
+    advances by one per call, token-serial or in one several-row pass, and the token is the restatement's draw."""
+    cfg = dict(synthetic.config("tiny16"))
+    sd = synthetic.random_state_dict(cfg, seed=2, std=0.05)
+    prompt = synthetic.random_prompt(cfg, 7, seed=5).reshape(1, -1)
+    for one_pass in (False, True):
+        llama.manual_seed(11)
+        llm = Llama3.from_config(cfg).load_weights(sd)
+        m = llm.model
+        counter = lambda: int(llama.rng_state(m.device).numpy().view(np.uint32)[2])
+        assert counter() == 0
+        tok = m.forward_rows(prompt, 0, 0.9, 0, 0.0).numpy()[0] if one_pass else m.forward(prompt, 0, 0.9, 0, 0.0).item()
+        assert counter() == 1
+        lg = m.logits.numpy().astype(np.float32)
+        assert int(tok) == S.sample(lg, 0.9, 0, 0.0, 0.0, 0.0, S.rand_f32(11, 0), np.zeros(cfg["vocab_size"], np.int32))
+        m.forward(np.array([[int(tok)]], np.int32), 7, 0.9, 0, 0.0)
+        assert counter() == 2
+    with pytest.raises(NotImplementedError, match="one sequence"):
+        m.forward_rows(np.zeros((2, 3), np.int32), 0, 0.9)
