@@ -5,8 +5,9 @@
 
 namespace jsg {
 
+// fp16 activations: four blocks per CU (128 registers per lane), which the grid is sized for
 template <int KIND, typename AT, int EPI, int ROWS, int UNROLL>
-__global__ __launch_bounds__(256) void gemv_kernel(GemvArgs a) {
+__global__ __launch_bounds__(256, sizeof(AT) == 2 ? 4 : 1) void gemv_kernel(GemvArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   __shared__ float red[8];
   __shared__ float lut[KIND == JSGRAD_W_NF4 ? NF4_LUT_WORDS : 16];
@@ -14,7 +15,7 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemvArgs a) {
   // read the position now, not in the epilogue: the load then overlaps the weight stream instead of ending the kernel
   const int pos = EPI == EPI_ROPE_KV ? a.st[1] : 0;
   GemvBuf buf;
-  G::run(a, (AT *)smem, red, lut, buf, false, pos);
+  G::template run<true>(a, (AT *)smem, red, lut, buf, false, pos);
 }
 
 // ---- host-side dispatch ------------------------------------------------------------------------

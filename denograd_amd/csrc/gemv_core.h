@@ -300,6 +300,98 @@ template <typename AT, bool COHERENT> __device__ __forceinline__ void stage_x(co
   __syncthreads();
 }
 
+// The same staging in two halves, for an input row that is ready when the kernel starts: issue() requests x (and the norm
+// weight) into registers BEFORE the first weight items are requested, finish() turns them into the LDS row afterwards.
+// Loads return in the order they were issued, so a row requested behind 16 KiB of weights per wavefront arrives only when
+// that whole window has landed (tens of megabytes over the chip) and nothing can be multiplied until then; requested first,
+// it is there after one round trip and the arithmetic runs along with the weight stream.  The barriers wait for LDS traffic
+// only, so the weight requests stay in flight.
+constexpr int XSTAGE_CHUNKS = 8;   // 16-byte chunks of x a thread holds (plain rows; a normed row has at most 4, host-checked)
+struct XStage {
+  u4_t xr[XSTAGE_CHUNKS];   // a normed row: chunks in xr[0..3], the norm weight's in xr[4..7]
+};
+template <typename AT> __device__ __forceinline__ void stage_x_issue(const GemvArgs &a, XStage &st) {
+  constexpr int EPC = 16 / sizeof(AT);
+  const int tid = threadIdx.x, nt = blockDim.x, nchunks = a.in_f / EPC;
+  const u4_t *xg = (const u4_t *)a.x;
+  if (a.norm_w != nullptr) {
+    const u4_t *wg = (const u4_t *)a.norm_w;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int c = tid + i * nt;
+      const int cc = c < nchunks ? c : nchunks - 1;   // past the end: a valid chunk again, not used
+      st.xr[i] = ldg(xg + cc);
+      st.xr[4 + i] = ldg(wg + cc);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < XSTAGE_CHUNKS; i++) {
+      const int c = tid + i * nt;
+      st.xr[i] = ldg(xg + (c < nchunks ? c : nchunks - 1));
+    }
+  }
+}
+template <typename AT> __device__ __forceinline__ void stage_x_finish(const GemvArgs &a, const XStage &st, AT *xs, float *red, int padded) {
+  constexpr int EPC = 16 / sizeof(AT);
+  const int n = a.in_f, tid = threadIdx.x, nt = blockDim.x, nchunks = n / EPC;
+  u4_t *xl = (u4_t *)xs;
+  for (int c = nchunks + tid; c < padded / EPC; c += nt) xl[c] = u4_t{0, 0, 0, 0};
+  if (a.norm_w == nullptr) {
+#pragma unroll
+    for (int i = 0; i < XSTAGE_CHUNKS; i++) {
+      const int c = tid + i * nt;
+      if (c < nchunks) xl[c] = st.xr[i];
+    }
+    for (int c = tid + XSTAGE_CHUNKS * nt; c < nchunks; c += nt) xl[c] = ldg((const u4_t *)a.x + c);   // rows longer than the registers hold
+    lds_barrier();
+    return;
+  }
+  float ss = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    if (tid + i * nt < nchunks) {
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        if constexpr (sizeof(AT) == 2) {
+          h2_t h = as_h2(st.xr[i][e]);
+          ss = fmaf((float)h[0], (float)h[0], ss);
+          ss = fmaf((float)h[1], (float)h[1], ss);
+        } else {
+          float f = __uint_as_float(st.xr[i][e]);
+          ss = fmaf(f, f, ss);
+        }
+      }
+    }
+  }
+  ss = wave_sum(ss);
+  const int wave = tid >> 6, nw = nt >> 6;
+  if ((tid & 63) == 0) red[wave] = ss;
+  lds_barrier();
+  float tot = 0.0f;
+  for (int i = 0; i < nw; i++) tot += red[i];
+  const float r = __fsqrt_rn(__fdiv_rn(1.0f, __fadd_rn(__fmul_rn(tot, a.inv_d), a.eps)));
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int c = tid + i * nt;
+    if (c < nchunks) {
+      u4_t o;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        if constexpr (sizeof(AT) == 2) {
+          h2_t h = as_h2(st.xr[i][e]), w = as_h2(st.xr[4 + i][e]), y;
+          y[0] = (_Float16)((float)(_Float16)((float)h[0] * r) * (float)w[0]);
+          y[1] = (_Float16)((float)(_Float16)((float)h[1] * r) * (float)w[1]);
+          o[e] = __builtin_bit_cast(uint32_t, y);
+        } else {
+          o[e] = __float_as_uint((__uint_as_float(st.xr[i][e]) * r) * __uint_as_float(st.xr[4 + i][e]));
+        }
+      }
+      xl[c] = o;
+    }
+  }
+  lds_barrier();
+}
+
 // One item's registers: the weight vectors plus, on the item that finishes a row group, the operands its epilogue will
 // need (row scales, residual, rotary pair), fetched with the weights so that no load latency is left at the end.
 // Every configuration in use moves 8 x 16 bytes per lane and item (UNROLL x NM x ROWS = 8) and has ROWS = 2, so one
@@ -525,11 +617,8 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
     }
   }
 
-  // xs: LDS for in_f activations; red: LDS float[blockDim/64]; lut: LDS float[16] (NF4 code book, written here), and for
-  // NF4 weights with fp16 activations NF4_LUT_WORDS words (the table of code pairs behind it)
-  __device__ static __forceinline__ void run(const GemvArgs &a, AT *xs, float *red, float *lut, Buf &bufA, bool preloaded, int pos) {
-    const int wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
-    const int ng = ngroups(a), nb = nbatch(a), gstride = gridDim.x * nw;
+  // the NF4 tables in LDS (published by the barrier at the end of stage_x)
+  __device__ static __forceinline__ void fill_lut(float *lut) {
     if constexpr (KIND == JSGRAD_W_NF4) {
       if (threadIdx.x < 16) lut[threadIdx.x] = NF4_CODE[threadIdx.x];
       if constexpr (sizeof(AT) == 2) {   // the table of code pairs, one entry per byte value (lut has NF4_LUT_WORDS words then)
@@ -539,6 +628,18 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
         }
       }
     }
+  }
+
+  // xs: LDS for in_f activations; red: LDS float[blockDim/64]; lut: LDS float[16] (NF4 code book, written here), and for
+  // NF4 weights with fp16 activations NF4_LUT_WORDS words (the table of code pairs behind it)
+  // EARLY_X: the input row exists when the kernel starts (it is not produced inside this launch): request it first.
+  template <bool EARLY_X = false>
+  __device__ static __forceinline__ void run(const GemvArgs &a, AT *xs, float *red, float *lut, Buf &bufA, bool preloaded, int pos) {
+    const int wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int ng = ngroups(a), nb = nbatch(a), gstride = gridDim.x * nw;
+    XStage xst;
+    if constexpr (EARLY_X) stage_x_issue<AT>(a, xst);
+    fill_lut(lut);
     int grp = blockIdx.x * nw + wave, b = 0;
     if (!preloaded && grp < ng) load_item(a, bufA, grp, 0, pos);
     auto advance = [&](int &g, int &bb) {
@@ -549,9 +650,15 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
     Buf bufB;
     int gB = grp, bB = b;
     advance(gB, bB);
-    if (gB < ng) load_item(a, bufB, gB, bB, pos);
-
-    stage_x<AT, COHERENT>(a, xs, red, nb * UNROLL * STEP);  // block-wide, ends with a barrier (which also publishes lut)
+    // block-wide, ends with a barrier (which also publishes lut)
+    if constexpr (EARLY_X) {
+      // x is back after one round trip; its registers are free again before the second item's are needed
+      stage_x_finish<AT>(a, xst, xs, red, nb * UNROLL * STEP);
+      if (gB < ng) load_item(a, bufB, gB, bB, pos);
+    } else {
+      if (gB < ng) load_item(a, bufB, gB, bB, pos);
+      stage_x<AT, COHERENT>(a, xs, red, nb * UNROLL * STEP);
+    }
 
     float acc[NM][ROWS];
     while (grp < ng) {
