@@ -28,16 +28,10 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_decode_kernel(AttnArgs a) {
   A::item(a, sm, g, split, T, chunk, n_active);
 }
 
-// splits: enough that a chunk fits the LDS score buffer, and no more than the merge can index there.  One sequence wants
-// short chunks (the launch is a chain of latencies); many sequences fill the chip by themselves, and every extra split
-// only adds its fixed cost (query load, partial store, counter, merge), so the splits stop at about 8 blocks per CU.
+// chunks the grid and the workspace provide: what the chunk policy can ask for at any T up to max_context
 static int nsplit_for(int max_context, int heads_x_batch) {
-  int by_lds = (max_context + ATT_CHUNK_MAX - 1) / ATT_CHUNK_MAX;
-  int wanted = (max_context + 31) / 32;
-  if (wanted > 64) wanted = 64;
-  const int fill = (2048 + heads_x_batch - 1) / heads_x_batch;
-  if (wanted > fill) wanted = fill;
-  return by_lds > wanted ? by_lds : wanted;
+  (void)heads_x_batch;
+  return att_max_chunks(max_context);
 }
 
 template <typename AT, int HD> static int launch_attn(const AttnArgs &a, int n_rep, int batch = 1) {

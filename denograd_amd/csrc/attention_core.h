@@ -16,14 +16,23 @@
 namespace jsg {
 
 constexpr int ATT_CHUNK_MAX = 256;  // positions per item held in LDS; also the most chunks the merge can index
-constexpr int ATT_CHUNK_MIN = 32;   // a block covers this many rows with the requests it sends before anything else (one
-                                    // iteration at head_dim 64, two at 128), so shorter chunks finish no sooner and only
-                                    // add partial results for the merge to fetch
 
-// rows per chunk when T visible positions are cut into at most nsplit chunks
+// Rows per chunk for T visible positions.  A launch is a chain of round trips (rows, partial results, merge), and the merge
+// fetches one partial result per chunk, so chunks are few and long rather than many and short: 64 rows up to 512 positions,
+// 128 up to 2048, 256 beyond (at most 8 / 16 / T/256 chunks per kv head).
+// `nsplit` chunks is what the workspace and the grid provide: the chunk grows if T would need more.
 __host__ __device__ __forceinline__ int att_chunk_rows(int T, int nsplit) {
-  const int c = (T + nsplit - 1) / nsplit;
-  return c < ATT_CHUNK_MIN ? ATT_CHUNK_MIN : c;
+  int c = T <= 512 ? 64 : (T <= 2048 ? 128 : 256);
+  const int need = (T + nsplit - 1) / nsplit;
+  return c < need ? need : c;
+}
+// chunks a launch must provide for every T up to max_context (the count is not monotonic in T across the policy's steps)
+__host__ __device__ __forceinline__ int att_max_chunks(int max_context) {
+  auto n = [](int T) { const int c = T <= 512 ? 64 : (T <= 2048 ? 128 : 256); return (T + c - 1) / c; };
+  int m = n(max_context < 512 ? max_context : 512);
+  if (max_context > 512) { const int v = n(max_context < 2048 ? max_context : 2048); m = v > m ? v : m; }
+  if (max_context > 2048) { const int v = n(max_context); m = v > m ? v : m; }
+  return m;
 }
 
 struct AttnArgs {
@@ -68,7 +77,11 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
 
   // T visible positions cut into chunks of `chunk` rows (n_active of them); this call handles chunk `split` of kv head g.
   // Must be called by every thread of the block (it contains barriers).
-  __device__ static void item(const AttnArgs &a, Smem &sm, int g, int split, int T, int chunk, int n_active) {
+  // after_requests: called once the requests for the query rows and the first K and V rows (ten iterations of the block) are
+  // out; a caller with other loads to issue puts them there, behind the rows the item's chain of round trips waits for.
+  struct NoHook { __device__ __forceinline__ void operator()() const {} };
+  __device__ static void item(const AttnArgs &a, Smem &sm, int g, int split, int T, int chunk, int n_active) { item(a, sm, g, split, T, chunk, n_active, NoHook()); }
+  template <typename Hook> __device__ static __forceinline__ void item(const AttnArgs &a, Smem &sm, int g, int split, int T, int chunk, int n_active, Hook after_requests) {
     const int t0 = split * chunk, t1 = min(T, t0 + chunk), CH = t1 - t0;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = NW * 64;
     const int sub = lane % G, grp = lane / G;
@@ -170,6 +183,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
         vbat[i] = *(const u4_t *)(vbase + (size_t)(t < t1 ? t : t1 - 1) * row_stride);
       }
     }
+    after_requests();   // loads return in order: whatever the caller requests now does not hold up the rows above
     lds_barrier();
     if (NREP <= NW) {
       // Wavefront j does the whole softmax of head j by itself - maximum, exp, sum - with no barrier in between: lane i holds
@@ -342,41 +356,46 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
     }
     __syncthreads();
     if (!sm.is_last) return;
-    // merge: one wavefront per query head turns the per-chunk (m, l) into weights exp(m_s - M) and 1/L ...
+    // merge.  Every thread owns two neighbouring output elements and requests their partial sums of the first MB chunks
+    // right away; while those travel, one wavefront per query head fetches the per-chunk (m, l), turns them into weights
+    // exp(m_s - M) and 1/L in LDS; then the sums are folded in chunk order.  One round trip for up to MB chunks.
     const float *base = a.partial + (size_t)g * a.nsplit * NREP * (HD + 2);
+    constexpr int MB = 16;                       // chunks per batch of requests
+    constexpr int NPAIR = NREP * HD / 2;         // element pairs of this kv head's query heads
+    auto ld_pair = [&](const float *po, int s_) -> uint64_t {   // two floats of chunk s_ (8-byte aligned: HD + 2 is even)
+      return __hip_atomic_load(as_global<uint64_t>(po + (size_t)(s_ < n_active ? s_ : n_active - 1) * NREP * (HD + 2)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    };
+    const int p0 = tid < NPAIR ? tid : 0;        // threads beyond the pairs request pair 0 again (their result is not stored)
+    const int j0 = (2 * p0) / HD, d0 = (2 * p0) % HD;
+    const float *po0 = base + (size_t)j0 * (HD + 2) + d0;
+    uint64_t part[MB];
+#pragma unroll
+    for (int u = 0; u < MB; u++) part[u] = ld_pair(po0, u);
     constexpr int MSL = ATT_CHUNK_MAX / 64;   // chunks per lane
     for (int j = wave; j < NREP; j += NW) {
-      float ms[MSL], ls[MSL];                  // (m, l) of this lane's chunks, all requested in one go
+      uint64_t mls[MSL];                       // (m, l) of this lane's chunks, all requested in one go
 #pragma unroll
-      for (int i = 0; i < MSL; i++) {
-        const int s_ = lane + i * 64;
-        if (i * 64 < n_active) {               // same for the whole wavefront
-          const float *ps = base + ((size_t)(s_ < n_active ? s_ : n_active - 1) * NREP + j) * (HD + 2);
-          ms[i] = ld_coherent(ps + HD);
-          ls[i] = ld_coherent(ps + HD + 1);
-        }
-      }
+      for (int i = 0; i < MSL; i++)
+        if (i * 64 < n_active) mls[i] = ld_pair(base + (size_t)j * (HD + 2) + HD, lane + i * 64);   // same test for the whole wavefront
       float M = -INFINITY;
 #pragma unroll
       for (int i = 0; i < MSL; i++)
-        if (lane + i * 64 < n_active) M = fmaxf(M, ms[i]);
+        if (lane + i * 64 < n_active) M = fmaxf(M, __uint_as_float((uint32_t)mls[i]));
       M = wave_max(M);
       float L = 0.0f;
 #pragma unroll
       for (int i = 0; i < MSL; i++) {
         const int s_ = lane + i * 64;
         if (s_ < n_active) {
-          const float w = exp_f32(ms[i] - M);
+          const float w = exp_f32(__uint_as_float((uint32_t)mls[i]) - M);
           sm.sc[j][s_] = w;  // n_active <= nsplit <= ATT_CHUNK_MAX
-          L = fmaf(ls[i], w, L);
+          L = fmaf(__uint_as_float((uint32_t)(mls[i] >> 32)), w, L);
         }
       }
       L = wave_sum(L);
       if (lane == 0) sm.l_sh[j] = 1.0f / L;  // softmax normalisation is e * (1/sum) (tensor.ts:2211-2214)
     }
-    __syncthreads();
-    // ... then every thread sums its output elements over the chunks in chunk order.  Two elements at a time: the first 32
-    // chunks of both are requested together (one round trip where there would be two; few chunks is the usual case)
+    lds_barrier();
     auto finish = [&](int i, float O) {
       const int j = i / HD, d = i % HD;
       AT *dst = (AT *)a.out + (size_t)(g * NREP + j) * HD + d;
@@ -385,45 +404,25 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       else if constexpr (COHERENT) st_coherent(dst, (AT)r);
       else *dst = (AT)r;
     };
-    auto ld_part = [&](const float *po, int s) { return ld_coherent(po + (size_t)(s < n_active ? s : n_active - 1) * NREP * (HD + 2)); };
-    constexpr bool PAIRS = NREP * HD > NW * 64;              // more elements than threads: a thread has at least two
-    for (int i0 = tid; i0 < NREP * HD; i0 += (PAIRS ? 2 : 1) * nthreads) {
-      const int i1 = i0 + nthreads;
-      const bool two = PAIRS && i1 < NREP * HD;
-      const int ja = i0 / HD, jb = (two ? i1 : i0) / HD;
-      const float *pa = base + (size_t)ja * (HD + 2) + i0 % HD, *pb = base + (size_t)jb * (HD + 2) + (two ? i1 : i0) % HD;
-      float parta[32], partb[32];
-#pragma unroll
-      for (int u = 0; u < 32; u++) parta[u] = ld_part(pa, u);
-      if constexpr (PAIRS) {
-#pragma unroll
-        for (int u = 0; u < 32; u++) partb[u] = ld_part(pb, u);
-      }
+    for (int p = tid; p < NPAIR; p += nthreads) {
+      const int j = (2 * p) / HD, d = (2 * p) % HD;
+      const float *po = base + (size_t)j * (HD + 2) + d;
       float Oa = 0.0f, Ob = 0.0f;
+      for (int s0 = 0; s0 < n_active; s0 += MB) {
+        if (s0 > 0 || p != tid) {                 // the first batch of the first pair is already here
 #pragma unroll
-      for (int u = 0; u < 32; u++)
-        if (u < n_active) Oa = fmaf(parta[u], sm.sc[ja][u], Oa);
-      if constexpr (PAIRS) {
-#pragma unroll
-        for (int u = 0; u < 32; u++)
-          if (u < n_active) Ob = fmaf(partb[u], sm.sc[jb][u], Ob);
-      }
-      for (int s0 = 32; s0 < n_active; s0 += 32) {           // more than 32 chunks: the rest in batches, element by element
-#pragma unroll
-        for (int u = 0; u < 32; u++) parta[u] = ld_part(pa, s0 + u);
-#pragma unroll
-        for (int u = 0; u < 32; u++)
-          if (s0 + u < n_active) Oa = fmaf(parta[u], sm.sc[ja][s0 + u], Oa);
-        if constexpr (PAIRS) {
-#pragma unroll
-          for (int u = 0; u < 32; u++) partb[u] = ld_part(pb, s0 + u);
-#pragma unroll
-          for (int u = 0; u < 32; u++)
-            if (s0 + u < n_active) Ob = fmaf(partb[u], sm.sc[jb][s0 + u], Ob);
+          for (int u = 0; u < MB; u++) part[u] = ld_pair(po, s0 + u);
         }
+#pragma unroll
+        for (int u = 0; u < MB; u++)
+          if (s0 + u < n_active) {
+            const float w = sm.sc[j][s0 + u];
+            Oa = fmaf(__uint_as_float((uint32_t)part[u]), w, Oa);
+            Ob = fmaf(__uint_as_float((uint32_t)(part[u] >> 32)), w, Ob);
+          }
       }
-      finish(i0, Oa);
-      if (two) finish(i1, Ob);
+      finish(2 * p, Oa);
+      finish(2 * p + 1, Ob);
     }
     if (tid == 0) __hip_atomic_store(&a.counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }

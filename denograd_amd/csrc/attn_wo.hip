@@ -17,7 +17,10 @@
 
 namespace jsg {
 
-constexpr int AW_THREADS = 256;
+// One block of 16 wavefronts per CU: an attention item is worked on by 16 wavefronts (its chain of dependent steps is what the
+// launch waits for), and the attention row is fetched by 256 blocks instead of 1024.
+constexpr int AW_THREADS = 1024;
+constexpr int AW_WAVES = AW_THREADS / 64;
 
 template <int KIND, int HD, int NREP>
 __global__ __launch_bounds__(AW_THREADS) void attn_wo_kernel(AttnArgs at, GemvArgs a, int layer) {
@@ -26,7 +29,7 @@ __global__ __launch_bounds__(AW_THREADS) void attn_wo_kernel(AttnArgs at, GemvAr
   typedef Gemv<KIND, AT, EPI_STORE, 2, 4, false> G;
   extern __shared__ __align__(16) unsigned char smem[];   // the staged input row of wo
   __shared__ typename A::Smem sm;
-  __shared__ float red[8];
+  __shared__ float red[AW_WAVES];
   __shared__ float lut[16];
 
   const int pos = at.st[1];   // asked for first, waited for after the weight requests below are out
@@ -84,8 +87,8 @@ template <int KIND, int HD> static int aw_capacity(int n_rep, size_t lds, int *o
 }
 
 template <int KIND, int HD> static int launch_attn_wo(const AttnArgs &at, const GemvArgs &a, int n_rep, int layer, int out_f, int *query_capacity) {
-  const int ngroups = (out_f + 1) / 2, need = (ngroups + 3) / 4;
-  const int cap = state().cu_count * 4;
+  const int ngroups = (out_f + 1) / 2, need = (ngroups + AW_WAVES - 1) / AW_WAVES;
+  const int cap = state().cu_count * (16 / AW_WAVES);
   int blocks = need < cap ? need : cap;
   const int items = at.n_kv_heads * at.nsplit;
   if (blocks < items) blocks = items;

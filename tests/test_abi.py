@@ -70,13 +70,14 @@ def test_attention_wo_launch_capacity_rule():
     against a given capacity here (on a GPU the library asks the occupancy calculator)."""
     from denograd_amd.llama import attn_wo_fits
     lib = ffi.load()
-    # chunks of the context: one per 32 positions, at most 64, at least one per 256 positions
-    assert lib.jsgrad_hip_attn_wo_items(8, 841) == 8 * 27
-    assert lib.jsgrad_hip_attn_wo_items(8, 2304) == 8 * 64
-    assert lib.jsgrad_hip_attn_wo_items(2, 64) == 2 * 2
-    assert lib.jsgrad_hip_attn_wo_items(8, 16384) == 8 * 64
+    # chunks of the context: 64 rows up to 512 positions, 128 up to 2048, 256 beyond; the most any T <= max_context asks for
+    assert lib.jsgrad_hip_attn_wo_items(8, 841) == 8 * 8        # T = 512 -> 8 chunks of 64 (841 itself: 7 of 128)
+    assert lib.jsgrad_hip_attn_wo_items(8, 2304) == 8 * 16      # T = 2048 -> 16 chunks of 128
+    assert lib.jsgrad_hip_attn_wo_items(2, 64) == 2 * 1
+    assert lib.jsgrad_hip_attn_wo_items(8, 16384) == 8 * 64     # 64 chunks of 256
     cap = 4 * 256      # four blocks of 256 threads per compute unit
-    assert attn_wo_fits(32, 8, 128, 8192, ffi.W_I8, 4096, capacity=cap)            # the 8B shape: 512 items
-    assert not attn_wo_fits(32, 32, 64, 2048, ffi.W_F16, 2048, capacity=cap)       # 32 kv heads x 64 chunks = 2048 items
-    assert attn_wo_fits(32, 32, 64, 1024, ffi.W_F16, 2048, capacity=cap)           # 32 x 32 = 1024 items just fit
-    assert not attn_wo_fits(64, 64, 64, 2048, ffi.W_F16, 4096, capacity=cap)
+    assert attn_wo_fits(32, 8, 128, 8192, ffi.W_I8, 4096, capacity=cap)            # the 8B shape: 256 items
+    assert attn_wo_fits(32, 32, 64, 2048, ffi.W_F16, 2048, capacity=cap)           # 32 kv heads x 16 chunks = 512 items
+    assert not attn_wo_fits(32, 32, 64, 16384, ffi.W_F16, 2048, capacity=cap)      # 32 x 64 = 2048 items
+    assert attn_wo_fits(32, 32, 64, 8192, ffi.W_F16, 2048, capacity=cap)           # 32 x 32 = 1024 items just fit
+    assert not attn_wo_fits(64, 64, 64, 8192, ffi.W_F16, 4096, capacity=cap)
