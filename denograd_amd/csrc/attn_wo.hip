@@ -32,40 +32,42 @@ __global__ __launch_bounds__(AW_THREADS) void attn_wo_kernel(AttnArgs at, GemvAr
   __shared__ float red[AW_WAVES];
   __shared__ float lut[16];
 
-  const int pos = at.st[1];   // asked for first, waited for after the weight requests below are out
-
-  // this wavefront's first wo item, requested before anything else
-  GemvBuf buf;
-  const int wave = threadIdx.x >> 6, grp = blockIdx.x * (AW_THREADS / 64) + wave;
-  const bool preloaded = grp < G::ngroups(a);
-  if (preloaded) G::load_item(a, buf, grp, 0, 0);
-  __builtin_amdgcn_sched_barrier(0);
-
-  // the version of this launch: no other launch that writes the same tagged row has it (another layer, or another
-  // position of the same layer; a model has at least two layers here)
-  const uint32_t tag = tw_tag(pos * 128 + layer);
-  at.out_tag = tag;
+  // The position first, and nothing else until it is here: a small request issued into an idle memory system is back in a
+  // fraction of a microsecond, behind the bursts of weight requests of all blocks it takes several times as long, and every
+  // later step of the attention items hangs on it.
+  const int pos = at.st[1];
+  const uint32_t tag = tw_tag(pos * 128 + layer);   // the version of this launch: no other launch that writes the same tagged
+  at.out_tag = tag;                                 // row has it (another layer, or another position of the same layer)
   a.x_tag = tag;
 
+  GemvBuf buf;
+  const int wave = threadIdx.x >> 6, grp = blockIdx.x * AW_WAVES + wave;
+  const bool preloaded = grp < G::ngroups(a);
+  bool has_item = false;
   if (pos >= 0 && pos < at.max_context) {
     const int T = pos + 1;
     const int chunk = att_chunk_rows(T, at.nsplit);   // <= ATT_CHUNK_MAX, checked on the host against max_context
     const int n_active = (T + chunk - 1) / chunk;
     const int id = blockIdx.x;
-    if (id < at.n_kv_heads * n_active) A::item(at, sm, id % at.n_kv_heads, id / at.n_kv_heads, T, chunk, n_active);
+    has_item = id < at.n_kv_heads * n_active;
+    if (has_item) {
+      // the attention item requests its rows, then this wavefront's first wo item goes out behind them (inside item(), through
+      // the hook), so that the rows are not queued behind the weights
+      A::item(at, sm, id % at.n_kv_heads, id / at.n_kv_heads, T, chunk, n_active, [&]() { if (preloaded) G::load_item(a, buf, grp, 0, 0); });
+    }
   } else if (blockIdx.x == 0 && threadIdx.x == 0) {
     st_coherent(a.err, 1);   // no attention row will come for such a position
+  }
+  if (!has_item) {
+    // blocks without an attention item give the items' requests a head start before they flood the memory system
+    __builtin_amdgcn_s_sleep(64);
+    if (preloaded) G::load_item(a, buf, grp, 0, 0);
   }
   __syncthreads();   // the LDS of the attention item is done with
   G::run(a, (AT *)smem, red, lut, buf, preloaded, 0);
 }
 
-static int aw_nsplit(int max_context) {
-  int by_lds = (max_context + ATT_CHUNK_MAX - 1) / ATT_CHUNK_MAX;
-  int wanted = (max_context + 31) / 32;
-  if (wanted > 64) wanted = 64;
-  return by_lds > wanted ? by_lds : wanted;
-}
+static int aw_nsplit(int max_context) { return att_max_chunks(max_context); }
 
 // Blocks of attn_wo_kernel<KIND, HD, n_rep> the device can hold at once (occupancy x CUs).  The blocks that run attention
 // items are the first `items` of the grid; the rest, and the attention blocks themselves once their item is done, wait in
