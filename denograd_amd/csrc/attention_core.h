@@ -73,15 +73,14 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
     float o_part[NW < 4 ? NW : 4][NREP][HD];   // wavefronts fold into four slots, then the slots are summed
     float m_sh[NREP], l_sh[NREP];
     int is_last;
+    __attribute__((aligned(16))) AT qs[NREP][HD];   // the query rows of the kv head
   };
 
   // T visible positions cut into chunks of `chunk` rows (n_active of them); this call handles chunk `split` of kv head g.
   // Must be called by every thread of the block (it contains barriers).
-  // after_requests: called once the requests for the query rows and the first K and V rows (ten iterations of the block) are
-  // out; a caller with other loads to issue puts them there, behind the rows the item's chain of round trips waits for.
-  struct NoHook { __device__ __forceinline__ void operator()() const {} };
-  __device__ static void item(const AttnArgs &a, Smem &sm, int g, int split, int T, int chunk, int n_active) { item(a, sm, g, split, T, chunk, n_active, NoHook()); }
-  template <typename Hook> __device__ static __forceinline__ void item(const AttnArgs &a, Smem &sm, int g, int split, int T, int chunk, int n_active, Hook after_requests) {
+  // Loads return in the order they were issued, and the block's barriers in front of the partial results wait for every
+  // outstanding one: a caller with other loads to issue (weights of a following stage) issues them after this call.
+  __device__ static void item(const AttnArgs &a, Smem &sm, int g, int split, int T, int chunk, int n_active) {
     const int t0 = split * chunk, t1 = min(T, t0 + chunk), CH = t1 - t0;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = NW * 64;
     const int sub = lane % G, grp = lane / G;
@@ -89,18 +88,19 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
     const AT *kbase = (const AT *)a.cache_k + (size_t)g * HD + (size_t)sub * EPL;
     const AT *vbase = (const AT *)a.cache_v + (size_t)g * HD + (size_t)sub * EPL;
 
-    // this lane's slice of the n_rep query rows
-    float qf[NREP][EPL];
+    // the n_rep query rows of this kv head: requested once per block (16-byte pieces), ahead of the K and V rows, and handed
+    // to every lane through LDS
+    constexpr int QCH = NREP * HD / EPL;      // 16-byte pieces of the query rows
+    u4_t qpiece = u4_t{0, 0, 0, 0};
+    if (tid < QCH) {
+      const AT *qp = (const AT *)a.q + (size_t)g * NREP * HD + (size_t)tid * EPL;
+      if constexpr (COHERENT) {
 #pragma unroll
-    for (int j = 0; j < NREP; j++) {
-      const AT *qp = (const AT *)a.q + (size_t)(g * NREP + j) * HD + sub * EPL;
-#pragma unroll
-      for (int e = 0; e < EPL; e++) {
-        if constexpr (COHERENT) qf[j][e] = (float)ld_coherent(qp + e);
-        else qf[j][e] = (float)qp[e];
+        for (int e = 0; e < 4; e++) qpiece[e] = __hip_atomic_load(as_global<uint32_t>(qp) + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      } else {
+        qpiece = *(const u4_t *)qp;
       }
     }
-
     // The K and V rows of this thread's first NPRE iterations are requested together, before anything is computed: a chunk is
     // usually that short, and the launch is a chain of round trips, so V must not wait for the softmax.
     constexpr int NPRE = 2;
@@ -113,25 +113,6 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       vpre[i] = *(const u4_t *)(vbase + off);
     }
 
-    // ---- phase 1: scores of the chunk
-    auto score_row = [&](u4_t raw, int t) {
-      float kf[EPL];
-      if constexpr (sizeof(AT) == 2) {
-#pragma unroll
-        for (int e = 0; e < 4; e++) { h2_t h = as_h2(raw[e]); kf[2 * e] = (float)h[0]; kf[2 * e + 1] = (float)h[1]; }
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; e++) kf[e] = __uint_as_float(raw[e]);
-      }
-#pragma unroll
-      for (int j = 0; j < NREP; j++) {
-        float p = 0.0f;
-#pragma unroll
-        for (int e = 0; e < EPL; e++) p = fmaf(qf[j][e], kf[e], p);
-        p = group_sum<G>(p);
-        if (sub == 0) sm.sc[j][t - t0] = p * a.scale;
-      }
-    };
     // a chunk with more rows than the up-front requests cover: its first batch of K rows is asked for before the first
     // scores are computed
     const int tb_v = t0 + (wave + NPRE * NW) * RPI + grp;
@@ -145,6 +126,28 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
         kbat[i] = *(const u4_t *)(kbase + (size_t)(t < t1 ? t : t1 - 1) * row_stride);
       }
     }
+    // the query rows are here first (requested first): publish them, take this lane's slice
+    if (tid < QCH) ((u4_t *)sm.qs)[tid] = qpiece;
+    lds_barrier();
+    u4_t qv[NREP];
+#pragma unroll
+    for (int j = 0; j < NREP; j++) qv[j] = ((const u4_t *)sm.qs)[j * G + sub];
+    // ---- phase 1: scores of the chunk.  fp16: packed dot products with float accumulation (the products are exact in float)
+    auto score_row = [&](u4_t raw, int t) {
+#pragma unroll
+      for (int j = 0; j < NREP; j++) {
+        float p = 0.0f;
+        if constexpr (sizeof(AT) == 2) {
+#pragma unroll
+          for (int e = 0; e < 4; e++) p = __builtin_amdgcn_fdot2(as_h2(qv[j][e]), as_h2(raw[e]), p, false);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; e++) p = fmaf(__uint_as_float(qv[j][e]), __uint_as_float(raw[e]), p);
+        }
+        p = group_sum<G>(p);
+        if (sub == 0) sm.sc[j][t - t0] = p * a.scale;
+      }
+    };
 #pragma unroll
     for (int i = 0; i < NPRE; i++) {
       const int t = t0 + (wave + i * NW) * RPI + grp;
@@ -183,7 +186,6 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
         vbat[i] = *(const u4_t *)(vbase + (size_t)(t < t1 ? t : t1 - 1) * row_stride);
       }
     }
-    after_requests();   // loads return in order: whatever the caller requests now does not hold up the rows above
     lds_barrier();
     if (NREP <= NW) {
       // Wavefront j does the whole softmax of head j by itself - maximum, exp, sum - with no barrier in between: lane i holds
@@ -333,7 +335,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
             *slot = round == 0 ? of[j][e] : *slot + of[j][e];
           }
       }
-      __syncthreads();
+      lds_barrier();
     }
     float *mine = a.partial + ((size_t)g * a.nsplit + split) * NREP * (HD + 2);
     for (int i = tid; i < NREP * HD; i += nthreads) {
