@@ -70,7 +70,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
   struct Smem {
     float sc[NREP][ATT_CHUNK_MAX];
     float red[NREP][NW];
-    float o_part[NW < 4 ? NW : 4][NREP][HD];   // wavefronts fold into four slots, then the slots are summed
+    __attribute__((aligned(16))) float o_part[NW][NREP][HD];   // every wavefront's partial output; summed in wavefront order
     float m_sh[NREP], l_sh[NREP];
     int is_last;
     __attribute__((aligned(16))) AT qs[NREP][HD];   // the query rows of the kv head
@@ -323,20 +323,17 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
         v = add_xor32(v);
         of[j][e] = v;
       }
-    // wavefronts fold into (at most) four LDS slots, four at a time
-    constexpr int SLOTS = NW < 4 ? NW : 4;
-    for (int round = 0; round < NW / SLOTS; round++) {
-      if (grp == 0 && wave / SLOTS == round) {
+    // every wavefront leaves its partial output in a slot of its own (16-byte stores), one barrier, then each element is the
+    // sum over the slots in wavefront order: independent reads, one LDS round trip (folding slot into slot would be a chain
+    // of read-add-write round trips, one per element)
+    if (grp == 0) {
 #pragma unroll
-        for (int j = 0; j < NREP; j++)
+      for (int j = 0; j < NREP; j++)
 #pragma unroll
-          for (int e = 0; e < EPL; e++) {
-            float *slot = &sm.o_part[wave % SLOTS][j][sub * EPL + e];
-            *slot = round == 0 ? of[j][e] : *slot + of[j][e];
-          }
-      }
-      lds_barrier();
+        for (int e = 0; e < EPL; e += 4) *(f4_t *)&sm.o_part[wave][j][sub * EPL + e] = f4_t{of[j][e], of[j][e + 1], of[j][e + 2], of[j][e + 3]};
     }
+    lds_barrier();
+    constexpr int SLOTS = NW;
     float *mine = a.partial + ((size_t)g * a.nsplit + split) * NREP * (HD + 2);
     for (int i = tid; i < NREP * HD; i += nthreads) {
       const int j = i / HD, d = i % HD;

@@ -316,6 +316,7 @@ int jsgrad_hip_decode_step(const jsgrad_hip_step_t *d) {
   const int feat = d->hidden > d->dim ? d->hidden : d->dim;
   size_t lds = (size_t)(feat > d->n_heads * d->head_dim ? feat : d->n_heads * d->head_dim) * sizeof(_Float16);
   const size_t attn_lds = 40 * 1024;   // >= sizeof(Attn<half, 128, 4, 16>::Smem)
+  static_assert(sizeof(Attn<_Float16, 128, 4, 16, true>::Smem) <= 40 * 1024, "attention LDS of the step kernel");
   if (lds < attn_lds) lds = attn_lds;
   JSG_REQUIRE(lds <= 60 * 1024, "jsgrad_hip_decode_step: %zu bytes of LDS needed", lds);
 
