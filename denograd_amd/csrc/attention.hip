@@ -4,7 +4,7 @@
 
 namespace jsg {
 
-constexpr int ATT_THREADS = 256;
+constexpr int ATT_THREADS = 1024;   // 16 wavefronts work on an item (attention_core.h requests every row of a chunk up front)
 
 template <typename AT, int HD, int NREP>
 __global__ __launch_bounds__(ATT_THREADS) void attn_decode_kernel(AttnArgs a) {

@@ -62,14 +62,29 @@ template <int G> __device__ __forceinline__ float group_sum(float v) {
 }
 
 // NW wavefronts per block.  COHERENT: q and the output cross between blocks of the same launch.
+//
+// Lane mappings.  Scores: a group of G = HD/EPL lanes covers one K row with one 128-bit load per lane (RPI = 64/G rows per
+// wavefront load); the dot products are reduced inside the group with DPP.  P.V: a lane takes ONE dword of a V row, so the 64
+// lanes cover a whole row (or two rows of 32 dwords) and every lane accumulates its own output elements over the rows of
+// its wavefront: no reduction across lanes at the end (with 16 wavefronts a CU that alone would cost as much as the item).
 template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
-  static constexpr int EPL = 16 / sizeof(AT);  // elements per lane per 128-bit load
-  static constexpr int G = HD / EPL;           // lanes per cache row
-  static constexpr int RPI = 64 / G;           // rows per wavefront iteration
-  static_assert(G == 8 || G == 16 || G == 32, "the fold over row groups is written for 8, 16 or 32 lanes per row");
+  static constexpr int EPL = 16 / sizeof(AT);  // K: elements per lane per 128-bit load
+  static constexpr int G = HD / EPL;           // K: lanes per cache row
+  static constexpr int RPI = 64 / G;           // K: rows per wavefront load
+  static constexpr int KIT = (ATT_CHUNK_MAX + NW * RPI - 1) / (NW * RPI);   // K loads per lane for the longest chunk
+  static constexpr int EP = 4 / sizeof(AT);    // V: elements per dword
+  static constexpr int PIECES = HD / EP;       // V: dwords per row
+  static constexpr int LPR = PIECES < 64 ? PIECES : 64;   // V: lanes per row
+  static constexpr int RPV = 64 / LPR;         // V: rows per wavefront load (1 or 2)
+  static constexpr int IPR = PIECES / LPR;     // V: loads per row (1 or 2)
+  static constexpr int VROWS = (ATT_CHUNK_MAX + NW - 1) / NW;      // rows of the longest chunk per wavefront
+  static constexpr int VIT = (VROWS + RPV - 1) / RPV * IPR;        // V loads per lane for the longest chunk
+  static_assert(G == 8 || G == 16 || G == 32, "scores are reduced over 8, 16 or 32 lanes per row");
+  static_assert(RPV == 1 || RPV == 2, "a V row is 32, 64 or 128 dwords");
+  static_assert(NREP <= NW, "one wavefront per query head does the softmax");
+  static_assert(KIT <= 8 && VIT <= 32, "all rows of a chunk are requested up front: the block needs enough wavefronts");
   struct Smem {
     float sc[NREP][ATT_CHUNK_MAX];
-    float red[NREP][NW];
     __attribute__((aligned(16))) float o_part[NW][NREP][HD];   // every wavefront's partial output; summed in wavefront order
     float m_sh[NREP], l_sh[NREP];
     int is_last;
@@ -81,15 +96,15 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
   // Loads return in the order they were issued, and the block's barriers in front of the partial results wait for every
   // outstanding one: a caller with other loads to issue (weights of a following stage) issues them after this call.
   __device__ static void item(const AttnArgs &a, Smem &sm, int g, int split, int T, int chunk, int n_active) {
-    const int t0 = split * chunk, t1 = min(T, t0 + chunk), CH = t1 - t0;
+    const int t0 = split * chunk, t1 = min(T, t0 + chunk), CH = t1 - t0;   // t1 > t0: the item exists
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = NW * 64;
     const int sub = lane % G, grp = lane / G;
     const size_t row_stride = (size_t)a.n_kv_heads * HD;
     const AT *kbase = (const AT *)a.cache_k + (size_t)g * HD + (size_t)sub * EPL;
-    const AT *vbase = (const AT *)a.cache_v + (size_t)g * HD + (size_t)sub * EPL;
+    const AT *vbase = (const AT *)a.cache_v + (size_t)g * HD;
 
-    // the n_rep query rows of this kv head: requested once per block (16-byte pieces), ahead of the K and V rows, and handed
-    // to every lane through LDS
+    // ---- every request of the item goes out now: the query rows (once per block, 16-byte pieces), then this lane's K rows,
+    // then its V dwords.  They come back in that order.
     constexpr int QCH = NREP * HD / EPL;      // 16-byte pieces of the query rows
     u4_t qpiece = u4_t{0, 0, 0, 0};
     if (tid < QCH) {
@@ -101,236 +116,128 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
         qpiece = *(const u4_t *)qp;
       }
     }
-    // The K and V rows of this thread's first NPRE iterations are requested together, before anything is computed: a chunk is
-    // usually that short, and the launch is a chain of round trips, so V must not wait for the softmax.
-    constexpr int NPRE = 2;
-    u4_t kpre[NPRE], vpre[NPRE];
+    u4_t kreg[KIT];
 #pragma unroll
-    for (int i = 0; i < NPRE; i++) {
-      const int t = t0 + (wave + i * NW) * RPI + grp;
-      const size_t off = (size_t)(t < t1 ? t : t1 - 1) * row_stride;   // t1 > t0: the item exists
-      kpre[i] = *(const u4_t *)(kbase + off);
-      vpre[i] = *(const u4_t *)(vbase + off);
-    }
-
-    // a chunk with more rows than the up-front requests cover: its first batch of K rows is asked for before the first
-    // scores are computed
-    const int tb_v = t0 + (wave + NPRE * NW) * RPI + grp;
-    const bool more_v = CH > NPRE * NW * RPI;              // the same for the whole block
-    constexpr int NBATCH = 8;
-    u4_t kbat[NBATCH];
-    if (more_v) {
-#pragma unroll
-      for (int i = 0; i < NBATCH; i++) {
-        const int t = tb_v + i * NW * RPI;
-        kbat[i] = *(const u4_t *)(kbase + (size_t)(t < t1 ? t : t1 - 1) * row_stride);
+    for (int i = 0; i < KIT; i++) {
+      if (i * NW * RPI < CH) {                // the same for the whole block
+        const int t = t0 + (wave + i * NW) * RPI + grp;
+        kreg[i] = *(const u4_t *)(kbase + (size_t)(t < t1 ? t : t1 - 1) * row_stride);
       }
     }
-    // the query rows are here first (requested first): publish them, take this lane's slice
+    const int VR = (CH + NW - 1) / NW;        // rows of this chunk per wavefront: wavefront w has rows [w * VR, (w + 1) * VR)
+    const int vsel = lane / LPR, vcol = lane % LPR;
+    uint32_t vreg[VIT];
+#pragma unroll
+    for (int i = 0; i < VIT; i++) {
+      const int ri = i / IPR, part = i % IPR;
+      if (ri * RPV < VR) {                    // the same for the whole block
+        const int r = ri * RPV + vsel;
+        const int t = t0 + wave * VR + r;
+        const bool ok = r < VR && t < t1;
+        vreg[i] = *(const uint32_t *)(vbase + (size_t)(ok ? t : t1 - 1) * row_stride + (size_t)(vcol + LPR * part) * EP);
+      }
+    }
+
+    // ---- phase 1: scores of the chunk.  The query rows are here first: publish them, take this lane's slice.
     if (tid < QCH) ((u4_t *)sm.qs)[tid] = qpiece;
     lds_barrier();
     u4_t qv[NREP];
 #pragma unroll
     for (int j = 0; j < NREP; j++) qv[j] = ((const u4_t *)sm.qs)[j * G + sub];
-    // ---- phase 1: scores of the chunk.  fp16: packed dot products with float accumulation (the products are exact in float)
-    auto score_row = [&](u4_t raw, int t) {
 #pragma unroll
-      for (int j = 0; j < NREP; j++) {
-        float p = 0.0f;
-        if constexpr (sizeof(AT) == 2) {
+    for (int i = 0; i < KIT; i++) {
+      if (i * NW * RPI < CH) {
+        const int t = t0 + (wave + i * NW) * RPI + grp;
 #pragma unroll
-          for (int e = 0; e < 4; e++) p = __builtin_amdgcn_fdot2(as_h2(qv[j][e]), as_h2(raw[e]), p, false);
-        } else {
+        for (int j = 0; j < NREP; j++) {
+          float p = 0.0f;
+          if constexpr (sizeof(AT) == 2) {     // packed dot products with float accumulation (the products are exact in float)
 #pragma unroll
-          for (int e = 0; e < 4; e++) p = fmaf(__uint_as_float(qv[j][e]), __uint_as_float(raw[e]), p);
+            for (int e = 0; e < 4; e++) p = __builtin_amdgcn_fdot2(as_h2(qv[j][e]), as_h2(kreg[i][e]), p, false);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) p = fmaf(__uint_as_float(qv[j][e]), __uint_as_float(kreg[i][e]), p);
+          }
+          p = group_sum<G>(p);
+          if (sub == 0 && t < t1) sm.sc[j][t - t0] = p * a.scale;
         }
-        p = group_sum<G>(p);
-        if (sub == 0) sm.sc[j][t - t0] = p * a.scale;
-      }
-    };
-#pragma unroll
-    for (int i = 0; i < NPRE; i++) {
-      const int t = t0 + (wave + i * NW) * RPI + grp;
-      if (t < t1) score_row(kpre[i], t);
-    }
-    if (more_v) {
-#pragma unroll
-      for (int i = 0; i < NBATCH; i++) {
-        const int t = tb_v + i * NW * RPI;
-        if (t < t1) score_row(kbat[i], t);
-      }
-    }
-    // still longer chunks: the remaining rows in batches of NBATCH requests, so that an iteration does not wait a round trip
-    // of its own
-    for (int tb = tb_v + NBATCH * NW * RPI; tb < t1; tb += NBATCH * NW * RPI) {
-      u4_t raw[NBATCH];
-#pragma unroll
-      for (int i = 0; i < NBATCH; i++) {
-        const int t = tb + i * NW * RPI;
-        raw[i] = *(const u4_t *)(kbase + (size_t)(t < t1 ? t : t1 - 1) * row_stride);
-      }
-#pragma unroll
-      for (int i = 0; i < NBATCH; i++) {
-        const int t = tb + i * NW * RPI;
-        if (t < t1) score_row(raw[i], t);
-      }
-    }
-    // A chunk with more rows than the requests sent up front cover (several sequences, long contexts): the first batch of V
-    // rows is requested now, so that it travels while the softmax is computed.  The two barriers around the softmax wait
-    // for LDS traffic only; __syncthreads() would also wait for these requests.
-    u4_t vbat[NBATCH];
-    if (more_v) {
-#pragma unroll
-      for (int i = 0; i < NBATCH; i++) {
-        const int t = tb_v + i * NW * RPI;
-        vbat[i] = *(const u4_t *)(vbase + (size_t)(t < t1 ? t : t1 - 1) * row_stride);
       }
     }
     lds_barrier();
-    if (NREP <= NW) {
-      // Wavefront j does the whole softmax of head j by itself - maximum, exp, sum - with no barrier in between: lane i holds
-      // rows i, i + 64, ... of the chunk (one row per lane for the short chunks of a single sequence).
-      if (wave < NREP) {
-        const int j = wave;
-        constexpr int PL = ATT_CHUNK_MAX / 64;
-        float sv[PL];
-        float m = -INFINITY;
+    // Wavefront j does the whole softmax of head j by itself - maximum, exp, sum - with no barrier in between: lane i holds
+    // rows i, i + 64, ... of the chunk.
+    if (wave < NREP) {
+      const int j = wave;
+      constexpr int PL = ATT_CHUNK_MAX / 64;
+      float sv[PL];
+      float m = -INFINITY;
 #pragma unroll
-        for (int q = 0; q < PL; q++) {
-          const int i = lane + 64 * q;
-          sv[q] = (q * 64 < CH && i < CH) ? sm.sc[j][i] : -INFINITY;
-          m = fmaxf(m, sv[q]);
+      for (int q = 0; q < PL; q++) {
+        const int i = lane + 64 * q;
+        sv[q] = (q * 64 < CH && i < CH) ? sm.sc[j][i] : -INFINITY;
+        m = fmaxf(m, sv[q]);
+      }
+      m = wave_max(m);
+      float l = 0.0f;
+#pragma unroll
+      for (int q = 0; q < PL; q++) {
+        const int i = lane + 64 * q;
+        if (q * 64 < CH) {      // the same for the whole wavefront
+          const float e = i < CH ? exp_f32(sv[q] - m) : 0.0f;
+          if (i < CH) sm.sc[j][i] = e;
+          l += e;
         }
-        m = wave_max(m);
-        float l = 0.0f;
-#pragma unroll
-        for (int q = 0; q < PL; q++) {
-          const int i = lane + 64 * q;
-          if (q * 64 < CH) {      // the same for the whole wavefront
-            const float e = i < CH ? exp_f32(sv[q] - m) : 0.0f;
-            if (i < CH) sm.sc[j][i] = e;
-            l += e;
-          }
-        }
-        l = wave_sum(l);
-        if (lane == 0) { sm.m_sh[j] = m; sm.l_sh[j] = l; }
       }
-    } else {
-    // chunk maximum per head
-    {
-      float mx[NREP];
-#pragma unroll
-      for (int j = 0; j < NREP; j++) mx[j] = -INFINITY;
-      for (int i = tid; i < CH; i += nthreads)
-#pragma unroll
-        for (int j = 0; j < NREP; j++) mx[j] = fmaxf(mx[j], sm.sc[j][i]);
-#pragma unroll
-      for (int j = 0; j < NREP; j++) {
-        float w = wave_max(mx[j]);
-        if (lane == 0) sm.red[j][wave] = w;
-      }
-      __syncthreads();
-      if (tid < NREP) {
-        float w = sm.red[tid][0];
-        for (int i = 1; i < NW; i++) w = fmaxf(w, sm.red[tid][i]);
-        sm.m_sh[tid] = w;
-      }
-      __syncthreads();
-    }
-    // scores -> exp(s - m) in place, and their sum
-    {
-      float ls[NREP];
-#pragma unroll
-      for (int j = 0; j < NREP; j++) ls[j] = 0.0f;
-      for (int i = tid; i < CH; i += nthreads)
-#pragma unroll
-        for (int j = 0; j < NREP; j++) {
-          float e = exp_f32(sm.sc[j][i] - sm.m_sh[j]);
-          sm.sc[j][i] = e;
-          ls[j] += e;
-        }
-#pragma unroll
-      for (int j = 0; j < NREP; j++) {
-        float w = wave_sum(ls[j]);
-        if (lane == 0) sm.red[j][wave] = w;
-      }
-      __syncthreads();
-      if (tid < NREP) {
-        float w = 0.0f;
-        for (int i = 0; i < NW; i++) w += sm.red[tid][i];
-        sm.l_sh[tid] = w;
-      }
-      // the barrier below also orders the in-place exp writes before phase 2 reads them
-    }
+      l = wave_sum(l);
+      if (lane == 0) { sm.m_sh[j] = m; sm.l_sh[j] = l; }
     }
     lds_barrier();
 
-    // ---- phase 2: o[j][d] = sum_t p[j][t] * V[t][d]
-    float of[NREP][EPL];
+    // ---- phase 2: o[j][d] = sum_t p[j][t] * V[t][d] over the rows of this wavefront; this lane's elements are
+    // d = (vcol + LPR * part) * EP + e
+    float of[NREP][IPR][EP];
 #pragma unroll
     for (int j = 0; j < NREP; j++)
 #pragma unroll
-      for (int e = 0; e < EPL; e++) of[j][e] = 0.0f;
-    auto pv_row = [&](u4_t raw, int t) {
-      float vf[EPL];
-      if constexpr (sizeof(AT) == 2) {
+      for (int c = 0; c < IPR; c++)
 #pragma unroll
-        for (int e = 0; e < 4; e++) { h2_t h = as_h2(raw[e]); vf[2 * e] = (float)h[0]; vf[2 * e + 1] = (float)h[1]; }
-      } else {
+        for (int e = 0; e < EP; e++) of[j][c][e] = 0.0f;
 #pragma unroll
-        for (int e = 0; e < 4; e++) vf[e] = __uint_as_float(raw[e]);
-      }
+    for (int i = 0; i < VIT; i++) {
+      const int ri = i / IPR, part = i % IPR;
+      if (ri * RPV < VR) {
+        const int r = ri * RPV + vsel;
+        const int t = t0 + wave * VR + r;
+        const bool ok = r < VR && t < t1;
+        float vf[EP];
+        if constexpr (sizeof(AT) == 2) { const h2_t h = as_h2(vreg[i]); vf[0] = (float)h[0]; vf[1] = (float)h[1]; }
+        else vf[0] = __uint_as_float(vreg[i]);
 #pragma unroll
-      for (int j = 0; j < NREP; j++) {
-        const float p = sm.sc[j][t - t0];
+        for (int j = 0; j < NREP; j++) {
+          const float p = ok ? sm.sc[j][ok ? t - t0 : 0] : 0.0f;   // rows past the chunk: an existing row times zero
 #pragma unroll
-        for (int e = 0; e < EPL; e++) of[j][e] = fmaf(p, vf[e], of[j][e]);
-      }
-    };
-#pragma unroll
-    for (int i = 0; i < NPRE; i++) {
-      const int t = t0 + (wave + i * NW) * RPI + grp;
-      if (t < t1) pv_row(vpre[i], t);
-    }
-    if (more_v) {
-#pragma unroll
-      for (int i = 0; i < NBATCH; i++) {
-        const int t = tb_v + i * NW * RPI;
-        if (t < t1) pv_row(vbat[i], t);
+          for (int e = 0; e < EP; e++) of[j][part][e] = fmaf(p, vf[e], of[j][part][e]);
+        }
       }
     }
-    for (int tb = tb_v + NBATCH * NW * RPI; tb < t1; tb += NBATCH * NW * RPI) {
-      u4_t raw[NBATCH];
-#pragma unroll
-      for (int i = 0; i < NBATCH; i++) {
-        const int t = tb + i * NW * RPI;
-        raw[i] = *(const u4_t *)(vbase + (size_t)(t < t1 ? t : t1 - 1) * row_stride);
-      }
-#pragma unroll
-      for (int i = 0; i < NBATCH; i++) {
-        const int t = tb + i * NW * RPI;
-        if (t < t1) pv_row(raw[i], t);
-      }
-    }
-    // lanes with the same `sub` hold different rows: fold the RPI groups of the wavefront together
-#pragma unroll
-    for (int j = 0; j < NREP; j++)
-#pragma unroll
-      for (int e = 0; e < EPL; e++) {
-        float v = of[j][e];
-        if constexpr (G <= 8) v += dpp_f<0x128>(v);    // row_ror:8: lane l ^ 8 of the same 16-lane row
-        if constexpr (G <= 16) v = add_xor16(v);
-        v = add_xor32(v);
-        of[j][e] = v;
-      }
-    // every wavefront leaves its partial output in a slot of its own (16-byte stores), one barrier, then each element is the
-    // sum over the slots in wavefront order: independent reads, one LDS round trip (folding slot into slot would be a chain
-    // of read-add-write round trips, one per element)
-    if (grp == 0) {
+    // two rows per load: the halves of the wavefront hold different rows of the same elements
+    if constexpr (RPV == 2) {
 #pragma unroll
       for (int j = 0; j < NREP; j++)
 #pragma unroll
-        for (int e = 0; e < EPL; e += 4) *(f4_t *)&sm.o_part[wave][j][sub * EPL + e] = f4_t{of[j][e], of[j][e + 1], of[j][e + 2], of[j][e + 3]};
+        for (int c = 0; c < IPR; c++)
+#pragma unroll
+          for (int e = 0; e < EP; e++) of[j][c][e] = add_xor32(of[j][c][e]);
+    }
+    // every wavefront leaves its partial output in a slot of its own, one barrier, then each element is the sum over the
+    // slots in wavefront order: independent reads, one LDS round trip
+    if (vsel == 0) {
+#pragma unroll
+      for (int j = 0; j < NREP; j++)
+#pragma unroll
+        for (int c = 0; c < IPR; c++)
+#pragma unroll
+          for (int e = 0; e < EP; e++) sm.o_part[wave][j][(vcol + LPR * c) * EP + e] = of[j][c][e];
     }
     lds_barrier();
     constexpr int SLOTS = NW;
