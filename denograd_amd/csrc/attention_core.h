@@ -94,8 +94,12 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
   // T visible positions cut into chunks of `chunk` rows (n_active of them); this call handles chunk `split` of kv head g.
   // Must be called by every thread of the block (it contains barriers).
   // Loads return in the order they were issued, and the block's barriers in front of the partial results wait for every
-  // outstanding one: a caller with other loads to issue (weights of a following stage) issues them after this call.
-  __device__ static void item(const AttnArgs &a, Smem &sm, int g, int split, int T, int chunk, int n_active) {
+  // outstanding one: a caller with other loads to issue (weights of a following stage) passes them as `then`, which is
+  // called exactly once, as soon as nothing the item still waits for can end up behind them: after the block has published
+  // its partial results, or, in the block that merges, right after the merge's own requests.
+  struct Nothing { __device__ __forceinline__ void operator()() const {} };
+  __device__ static void item(const AttnArgs &a, Smem &sm, int g, int split, int T, int chunk, int n_active) { item(a, sm, g, split, T, chunk, n_active, Nothing()); }
+  template <typename Then> __device__ static __forceinline__ void item(const AttnArgs &a, Smem &sm, int g, int split, int T, int chunk, int n_active, Then then) {
     const int t0 = split * chunk, t1 = min(T, t0 + chunk), CH = t1 - t0;   // t1 > t0: the item exists
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = NW * 64;
     const int sub = lane % G, grp = lane / G;
@@ -261,7 +265,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       sm.is_last = (old == n_active - 1);
     }
     __syncthreads();
-    if (!sm.is_last) return;
+    if (!sm.is_last) { then(); return; }
     // merge.  Every thread owns two neighbouring output elements and requests their partial sums of the first MB chunks
     // right away; while those travel, one wavefront per query head fetches the per-chunk (m, l), turns them into weights
     // exp(m_s - M) and 1/L in LDS; then the sums are folded in chunk order.  One round trip for up to MB chunks.
@@ -274,15 +278,19 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
     const int p0 = tid < NPAIR ? tid : 0;        // threads beyond the pairs request pair 0 again (their result is not stored)
     const int j0 = (2 * p0) / HD, d0 = (2 * p0) % HD;
     const float *po0 = base + (size_t)j0 * (HD + 2) + d0;
+    constexpr int MSL = ATT_CHUNK_MAX / 64;   // chunks per lane
+    uint64_t mls[MSL];                         // wavefront j < NREP: (m, l) of this lane's chunks of head j, requested in one go
+    if (wave < NREP) {
+#pragma unroll
+      for (int i = 0; i < MSL; i++)
+        if (i * 64 < n_active) mls[i] = ld_pair(base + (size_t)wave * (HD + 2) + HD, lane + i * 64);   // same test for the whole wavefront
+    }
     uint64_t part[MB];
 #pragma unroll
     for (int u = 0; u < MB; u++) part[u] = ld_pair(po0, u);
-    constexpr int MSL = ATT_CHUNK_MAX / 64;   // chunks per lane
-    for (int j = wave; j < NREP; j += NW) {
-      uint64_t mls[MSL];                       // (m, l) of this lane's chunks, all requested in one go
-#pragma unroll
-      for (int i = 0; i < MSL; i++)
-        if (i * 64 < n_active) mls[i] = ld_pair(base + (size_t)j * (HD + 2) + HD, lane + i * 64);   // same test for the whole wavefront
+    then();
+    if (wave < NREP) {
+      const int j = wave;
       float M = -INFINITY;
 #pragma unroll
       for (int i = 0; i < MSL; i++)

@@ -50,16 +50,20 @@ __global__ __launch_bounds__(AW_THREADS) void attn_wo_kernel(AttnArgs at, GemvAr
     const int n_active = (T + chunk - 1) / chunk;
     const int id = blockIdx.x;
     has_item = id < at.n_kv_heads * n_active;
-    if (has_item) A::item(at, sm, id % at.n_kv_heads, id / at.n_kv_heads, T, chunk, n_active);
+    // This wavefront's first wo item is requested as soon as the attention item lets it (attention_core.h: loads return in
+    // order and the item's barriers wait for every outstanding one, so weights requested earlier would sit in front of the
+    // rows and partial results the item waits for): when the block has published its chunk, or, in the block that merges,
+    // behind the merge's requests, so that the weights travel while the merge computes.
+    if (has_item) A::item(at, sm, id % at.n_kv_heads, id / at.n_kv_heads, T, chunk, n_active, [&]() { if (preloaded) G::load_item(a, buf, grp, 0, 0); });
   } else if (blockIdx.x == 0 && threadIdx.x == 0) {
     st_coherent(a.err, 1);   // no attention row will come for such a position
   }
-  // This wavefront's first wo item.  Blocks with an attention item ask for it now, when the item is done: loads return in
-  // order and the item's barriers wait for every outstanding one, so weights requested earlier would sit in front of the
-  // rows and partial results the item waits for.  The other blocks give the items' small requests a head start before they
-  // flood the memory system with theirs; either way the weights are there before the attention row is.
-  if (!has_item) __builtin_amdgcn_s_sleep(64);
-  if (preloaded) G::load_item(a, buf, grp, 0, 0);
+  // The other blocks give the items' small requests a head start before they flood the memory system with theirs; either
+  // way the weights are there before the attention row is.
+  if (!has_item) {
+    __builtin_amdgcn_s_sleep(64);
+    if (preloaded) G::load_item(a, buf, grp, 0, 0);
+  }
   __syncthreads();   // the LDS of the attention item is done with
   G::run(a, (AT *)smem, red, lut, buf, preloaded, 0);
 }
