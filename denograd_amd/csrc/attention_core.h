@@ -40,6 +40,7 @@ struct AttnArgs {
   const int32_t *st;
   void *out;
   int *counters;   // [n_kv_heads], zero before the first launch; the merging block leaves them zero
+  int *err = nullptr;   // optional: set to 1 when the merging block's bounded wait for the other chunks ran out
   float *partial;  // [n_kv_heads][nsplit][n_rep][HD + 2]
   int n_kv_heads, nsplit, max_context;
   float scale;     // float(1 / sqrt(head_dim)) (tensor.ts:3923 `.div(Math.sqrt(d))` = mul by the folded reciprocal)
@@ -87,7 +88,6 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
     float sc[NREP][ATT_CHUNK_MAX];
     __attribute__((aligned(16))) float o_part[NW][NREP][HD];   // every wavefront's partial output; summed in wavefront order
     float m_sh[NREP], l_sh[NREP];
-    int is_last;
     __attribute__((aligned(16))) AT qs[NREP][HD];   // the query rows of the kv head
   };
 
@@ -95,8 +95,8 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
   // Must be called by every thread of the block (it contains barriers).
   // Loads return in the order they were issued, and the block's barriers in front of the partial results wait for every
   // outstanding one: a caller with other loads to issue (weights of a following stage) passes them as `then`, which is
-  // called exactly once, as soon as nothing the item still waits for can end up behind them: after the block has published
-  // its partial results, or, in the block that merges, right after the merge's own requests.
+  // called exactly once, when nothing the item still waits for can end up behind them: after the block has published its
+  // partial results (and, in the block of chunk 0, merged the kv head).
   struct Nothing { __device__ __forceinline__ void operator()() const {} };
   __device__ static void item(const AttnArgs &a, Smem &sm, int g, int split, int T, int chunk, int n_active) { item(a, sm, g, split, T, chunk, n_active, Nothing()); }
   template <typename Then> __device__ static __forceinline__ void item(const AttnArgs &a, Smem &sm, int g, int split, int T, int chunk, int n_active, Then then) {
@@ -258,14 +258,26 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       st_coherent(&mine[tid * (HD + 2) + HD + 1], sm.l_sh[tid]);
     }
 
-    // ---- publish, and let the last chunk of this kv head merge
+    // ---- publish.  The block of chunk 0 merges the chunks of its kv head; the others count themselves in and are done.
     __syncthreads();  // every coherent store of the block has been acknowledged
-    if (tid == 0) {
-      int old = __hip_atomic_fetch_add(&a.counters[g], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      sm.is_last = (old == n_active - 1);
+    if (split != 0) {
+      if (tid == 0) __hip_atomic_fetch_add(&a.counters[g], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // nobody waits for the answer
+      then();
+      return;
     }
-    __syncthreads();
-    if (!sm.is_last) { then(); return; }
+    if (n_active > 1) {
+      if (tid == 0) {
+        // The other chunks' blocks never wait for anything before they count themselves in, and the launch keeps them all on the
+        // device, so this wait ends; it is bounded all the same and reports through the error word where one is given.
+        int it = 0;
+        while (ld_coherent(&a.counters[g]) != n_active - 1) {
+          if (++it > (1 << 20)) { if (a.err != nullptr) st_coherent(a.err, 1); break; }
+          __builtin_amdgcn_s_sleep(2);
+        }
+        __hip_atomic_store(&a.counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // zero again for the next launch
+      }
+      __syncthreads();
+    }
     // merge.  Every thread owns two neighbouring output elements and requests their partial sums of the first MB chunks
     // right away; while those travel, one wavefront per query head fetches the per-chunk (m, l), turns them into weights
     // exp(m_s - M) and 1/L in LDS; then the sums are folded in chunk order.  One round trip for up to MB chunks.
@@ -288,7 +300,6 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
     uint64_t part[MB];
 #pragma unroll
     for (int u = 0; u < MB; u++) part[u] = ld_pair(po0, u);
-    then();
     if (wave < NREP) {
       const int j = wave;
       float M = -INFINITY;
@@ -338,7 +349,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       finish(2 * p, Oa);
       finish(2 * p + 1, Ob);
     }
-    if (tid == 0) __hip_atomic_store(&a.counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    then();
   }
 };
 

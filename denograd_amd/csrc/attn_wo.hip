@@ -40,9 +40,12 @@ __global__ __launch_bounds__(AW_THREADS) void attn_wo_kernel(AttnArgs at, GemvAr
   at.out_tag = tag;                                 // row has it (another layer, or another position of the same layer)
   a.x_tag = tag;
 
+  // Blocks [0, n_kv_heads) run chunk 0 of a kv head and merge that head's chunks; they take no part in wo (the merged row is
+  // what everybody else waits for, and their weights would arrive last).  The wo rows are shared by the other blocks.
   GemvBuf buf;
-  const int wave = threadIdx.x >> 6, grp = blockIdx.x * AW_WAVES + wave;
-  const bool preloaded = grp < G::ngroups(a);
+  const int wo_blk = (int)blockIdx.x - at.n_kv_heads, wo_nblk = (int)gridDim.x - at.n_kv_heads;
+  const int wave = threadIdx.x >> 6, grp = wo_blk * AW_WAVES + wave;
+  const bool preloaded = wo_blk >= 0 && grp < G::ngroups(a);
   bool has_item = false;
   if (pos >= 0 && pos < at.max_context) {
     const int T = pos + 1;
@@ -64,8 +67,9 @@ __global__ __launch_bounds__(AW_THREADS) void attn_wo_kernel(AttnArgs at, GemvAr
     __builtin_amdgcn_s_sleep(64);
     if (preloaded) G::load_item(a, buf, grp, 0, 0);
   }
+  if (wo_blk < 0) return;
   __syncthreads();   // the LDS of the attention item is done with
-  G::run(a, (AT *)smem, red, lut, buf, preloaded, 0);
+  G::run(a, (AT *)smem, red, lut, buf, preloaded, 0, wo_blk, wo_nblk);
 }
 
 static int aw_nsplit(int max_context) { return att_max_chunks(max_context); }
@@ -90,7 +94,7 @@ template <int KIND, int HD> static int aw_capacity(int n_rep, size_t lds, int *o
 }
 
 template <int KIND, int HD> static int launch_attn_wo(const AttnArgs &at, const GemvArgs &a, int n_rep, int layer, int out_f, int *query_capacity) {
-  const int ngroups = (out_f + 1) / 2, need = (ngroups + AW_WAVES - 1) / AW_WAVES;
+  const int ngroups = (out_f + 1) / 2, need = (ngroups + AW_WAVES - 1) / AW_WAVES + at.n_kv_heads;   // the merging blocks do no wo rows
   const int cap = state().cu_count * (16 / AW_WAVES);
   int blocks = need < cap ? need : cap;
   const int items = at.n_kv_heads * at.nsplit;
@@ -154,6 +158,7 @@ static int attn_wo_impl(const void *q, const void *cache_k, const void *cache_v,
   at.n_kv_heads = n_kv_heads; at.nsplit = aw_nsplit(max_context); at.max_context = max_context;
   at.scale = (float)(1.0 / sqrt((double)head_dim));
   at.out_tagged = (uint32_t *)(ws + 512 + (size_t)n_heads * 256 * (head_dim + 2) * sizeof(float));
+  at.err = (int *)(ws + 256);
   GemvArgs a = {};
   a.w0 = wo; a.s0 = so; a.rows0 = dim; a.in_f = qdim; a.norm_w = nullptr; a.eps = 0.0f;
   a.inv_d = (float)(1.0 / (double)qdim); a.y = y; a.residual = residual;

@@ -633,14 +633,16 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
   // xs: LDS for in_f activations; red: LDS float[blockDim/64]; lut: LDS float[16] (NF4 code book, written here), and for
   // NF4 weights with fp16 activations NF4_LUT_WORDS words (the table of code pairs behind it)
   // EARLY_X: the input row exists when the kernel starts (it is not produced inside this launch): request it first.
+  // blk / nblk: this block's index among the nblk blocks that share the rows (the whole grid unless the caller says otherwise).
   template <bool EARLY_X = false>
-  __device__ static __forceinline__ void run(const GemvArgs &a, AT *xs, float *red, float *lut, Buf &bufA, bool preloaded, int pos) {
+  __device__ static __forceinline__ void run(const GemvArgs &a, AT *xs, float *red, float *lut, Buf &bufA, bool preloaded, int pos, int blk = blockIdx.x,
+                                             int nblk = gridDim.x) {
     const int wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
-    const int ng = ngroups(a), nb = nbatch(a), gstride = gridDim.x * nw;
+    const int ng = ngroups(a), nb = nbatch(a), gstride = nblk * nw;
     XStage xst;
     if constexpr (EARLY_X) stage_x_issue<AT>(a, xst);
     fill_lut(lut);
-    int grp = blockIdx.x * nw + wave, b = 0;
+    int grp = blk * nw + wave, b = 0;
     if (!preloaded && grp < ng) load_item(a, bufA, grp, 0, pos);
     auto advance = [&](int &g, int &bb) {
       if (++bb == nb) { bb = 0; g += gstride; }
