@@ -23,7 +23,7 @@ int fail(const char *fmt, ...);
 int fail_hip(hipError_t e, const char *what);
 
 // per-kernel timing with HIP events on the library stream (off unless jsgrad_hip_profile(1))
-enum { PROF_EMBED = 0, PROF_RMSNORM, PROF_LINEAR, PROF_QKV_ROPE, PROF_ATTN, PROF_FFN_GATE, PROF_ARGMAX, PROF_STEP, PROF_GEMM, PROF_ATTN_PREFILL, PROF_ATTN_WO, PROF_READ, PROF_SAMPLE, PROF_KINDS };
+enum { PROF_EMBED = 0, PROF_RMSNORM, PROF_LINEAR, PROF_QKV_ROPE, PROF_ATTN, PROF_FFN_GATE, PROF_ARGMAX, PROF_STEP, PROF_GEMM, PROF_ATTN_PREFILL, PROF_ATTN_WO, PROF_READ, PROF_SAMPLE, PROF_FFN, PROF_KINDS };
 // Event pair for the next launch of `kind`, or false when profiling is off (or capturing, or out of slots).  The pair
 // is handed to hipExtLaunchKernelGGL, which stamps it with the dispatch's own begin/end times, so the elapsed time is
 // the kernel alone: no marker packets, no launch latency.

@@ -34,6 +34,10 @@ struct GemvArgs {
   const uint32_t *x_tagged = nullptr;
   uint32_t x_tag = 0;
   int *err = nullptr;
+  // when set, EPI_STORE / EPI_SWIGLU write their output row here as tagged words (value | y_tag << 16) instead of to y, for
+  // blocks of the same launch that take it as their x_tagged
+  uint32_t *y_tagged = nullptr;
+  uint32_t y_tag = 0;
 };
 
 // ---- weight formats: VEC elements per 16-byte load --------------------------------------------
@@ -589,13 +593,18 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
         if (lane == r && r0 + r < mrows) {
           float v = val[0][r];
           if (has_res) v = Act<AT>::rn(extra_of<AT>(buf, r) + v);
-          store_out(y + r0 + r, v);
+          if (a.y_tagged != nullptr) tw_store(a.y_tagged + r0 + r, a.y_tag, v);
+          else store_out(y + r0 + r, v);
         }
     } else if constexpr (EPI == EPI_SWIGLU) {
       AT *g = (AT *)a.y;
 #pragma unroll
       for (int r = 0; r < ROWS; r++)
-        if (lane == r && r0 + r < mrows) store_out(g + r0 + r, Act<AT>::rn(silu_act<AT>(val[0][r]) * val[1][r]));
+        if (lane == r && r0 + r < mrows) {
+          const float v = Act<AT>::rn(silu_act<AT>(val[0][r]) * val[1][r]);
+          if (a.y_tagged != nullptr) tw_store(a.y_tagged + r0 + r, a.y_tag, v);
+          else store_out(g + r0 + r, v);
+        }
     } else {
       if (pos < 0 || pos >= a.max_context) return;  // never write outside the cache
       if (w.m == 2) {  // value rows: plain copy into the cache row
