@@ -52,10 +52,9 @@ def linear_bytes(cfg, out_f, in_f):
     return out_f * in_f * 2
 
 
-def kernel_bytes(cfg, T, attn_wo=False, ffn=False):
+def kernel_bytes(cfg, T, attn_wo=False):
     """algorithmic HBM bytes per decode step of each kernel family at T visible positions; attn_wo: attention and wo of a
-    layer are one launch (their bytes move from `attn_decode` and `linear` to `attn_wo`); ffn: w1 / w3 / w2 of a layer are
-    one launch (bytes move from `ffn_gate` and `linear` to `ffn`)"""
+    layer are one launch (their bytes move from `attn_decode` and `linear` to `attn_wo`)"""
     from denograd_amd import synthetic
     d, V, L = cfg["dim"], cfg["vocab_size"], cfg["n_layers"]
     shp = synthetic.linear_shapes(cfg)
@@ -72,13 +71,10 @@ def kernel_bytes(cfg, T, attn_wo=False, ffn=False):
     if attn_wo:
         out["attn_wo"] = out.pop("attn_decode") + L * lb("attention.wo")
         out["linear"] -= L * lb("attention.wo")
-    if ffn:
-        out["ffn"] = out.pop("ffn_gate") + L * lb("feed_forward.w2")
-        out["linear"] -= L * lb("feed_forward.w2")
     return out
 
 
-def read_only_launches(lib, cfg, T, attn_wo, ffn=False, reps=12):
+def read_only_launches(lib, cfg, T, attn_wo, reps=12):
     """Time jsgrad_hip_read_probe at the byte count of every weight-streaming launch of one decode step (cold data: the
     source window moves through 1 GiB).  Returns ms per step per kernel family, their sum, and the per-size table."""
     from denograd_amd import ffi, synthetic
@@ -100,9 +96,7 @@ def read_only_launches(lib, cfg, T, attn_wo, ffn=False, reps=12):
     else:
         launches["linear"].append((L, lb("attention.wo")))
         launches["attn_decode"] = [(L, kv)]
-    if ffn:
-        launches["ffn"] = [(L, launches.pop("ffn_gate")[0][1] + lb("feed_forward.w2"))]
-        launches["linear"] = [x for x in launches["linear"] if x != (L, lb("feed_forward.w2"))]
+
     span = 1 << 30
     src, sink = Tensor.empty((span,), "uint8"), Tensor.zeros((4,), "uint8")
     check(lib.jsgrad_hip_memset(src.ptr, 1, span))
@@ -231,7 +225,7 @@ def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=Tru
         if m.forward_jit is not None:
             m.forward_jit.reset()
     fam = per_op if fused else kinds
-    kb = kernel_bytes(cfg, llm.start_pos, attn_wo="attn_wo" in fam, ffn="ffn" in fam)
+    kb = kernel_bytes(cfg, llm.start_pos, attn_wo="attn_wo" in fam)
     for kname, b_ in kb.items():
         k = fam[kname]
         k["bytes_per_step"] = int(b_)
@@ -240,7 +234,7 @@ def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=Tru
     bytes_tok = synthetic.weight_bytes_per_token(cfg) + synthetic.kv_bytes_per_position(cfg) * t_avg
     # The measuring stick: a launch that only reads as many bytes as each weight-streaming launch of the step moves (cold
     # data, same event timing).  What the step would take if its launches did nothing but read.
-    read_only = read_only_launches(lib, cfg, llm.start_pos, "attn_wo" in fam, "ffn" in fam)
+    read_only = read_only_launches(lib, cfg, llm.start_pos, "attn_wo" in fam)
     for kname, r in read_only["families"].items():
         if kname in fam:
             fam[kname]["read_only_ms_per_step"] = r
@@ -271,12 +265,12 @@ def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=Tru
         fam["linear"]["per_matrix"] = {
             "lm_head": {"launches_per_step": 1, "bytes_per_launch": int(head_b), "avg_us_per_launch": round(1e3 * head_ms, 2), "GBps": round(head_b / (head_ms * 1e-3) / 1e9, 1)}}
         if rest_n > 0:
-            rest_name = "+".join(n for n, there in (("wo", "attn_wo" not in fam), ("w2", "ffn" not in fam)) if there)
+            rest_name = "w2" if "attn_wo" in fam else "wo+w2"
             fam["linear"]["per_matrix"][rest_name] = {"launches_per_step": rest_n, "bytes_per_launch": int(rest_b / rest_n), "avg_us_per_launch": round(1e3 * rest_ms / rest_n, 2),
                                                       "GBps": round(rest_b / (rest_ms * 1e-3) / 1e9, 1)}
         # the dominant kernel: the weight-streaming family the step spends the most time in
         dom = max((k for k in kb if k in fam), key=lambda k: fam[k]["ms_per_step"])
-        kern = {"linear": "gemv_kernel<EPI_STORE> (lm_head and the layer matrices that are launches of their own)", "ffn": "ffn_kernel (ffn_norm + w1, w3 + SwiGLU + w2 + residual)", "ffn_gate": "gemv_kernel<EPI_SWIGLU> (ffn_norm + w1, w3 + SwiGLU)",
+        kern = {"linear": "gemv_kernel<EPI_STORE> (lm_head and the layer matrices that are launches of their own)", "ffn_gate": "gemv_kernel<EPI_SWIGLU> (ffn_norm + w1, w3 + SwiGLU)",
                 "qkv_rope": "gemv_kernel<EPI_ROPE_KV> (attention_norm + wq, wk, wv + rotary + cache write)",
                 "attn_wo": "attn_wo_kernel (decode attention + wo + residual)", "attn_decode": "attn_decode_kernel"}[dom]
         achieved = fam[dom]["GBps"]

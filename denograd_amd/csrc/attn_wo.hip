@@ -44,7 +44,7 @@ __global__ __launch_bounds__(AW_THREADS) void attn_wo_kernel(AttnArgs at, GemvAr
   // what everybody else waits for, and their weights would arrive last).  The wo rows are shared by the other blocks.
   GemvBuf buf;
   const int wo_blk = (int)blockIdx.x - at.n_kv_heads, wo_nblk = (int)gridDim.x - at.n_kv_heads;
-  const int wave = threadIdx.x >> 6, grp = wo_blk * AW_WAVES + wave;
+  const int grp = G::first_group(wo_blk, wo_nblk);
   const bool preloaded = wo_blk >= 0 && grp < G::ngroups(a);
   bool has_item = false;
   if (pos >= 0 && pos < at.max_context) {

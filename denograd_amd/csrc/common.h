@@ -23,7 +23,7 @@ int fail(const char *fmt, ...);
 int fail_hip(hipError_t e, const char *what);
 
 // per-kernel timing with HIP events on the library stream (off unless jsgrad_hip_profile(1))
-enum { PROF_EMBED = 0, PROF_RMSNORM, PROF_LINEAR, PROF_QKV_ROPE, PROF_ATTN, PROF_FFN_GATE, PROF_ARGMAX, PROF_STEP, PROF_GEMM, PROF_ATTN_PREFILL, PROF_ATTN_WO, PROF_READ, PROF_SAMPLE, PROF_FFN, PROF_KINDS };
+enum { PROF_EMBED = 0, PROF_RMSNORM, PROF_LINEAR, PROF_QKV_ROPE, PROF_ATTN, PROF_FFN_GATE, PROF_ARGMAX, PROF_STEP, PROF_GEMM, PROF_ATTN_PREFILL, PROF_ATTN_WO, PROF_READ, PROF_SAMPLE, PROF_KINDS };
 // Event pair for the next launch of `kind`, or false when profiling is off (or capturing, or out of slots).  The pair
 // is handed to hipExtLaunchKernelGGL, which stamps it with the dispatch's own begin/end times, so the elapsed time is
 // the kernel alone: no marker packets, no launch latency.
@@ -166,6 +166,35 @@ __device__ __forceinline__ float row8_sum(float v) {
   v += dpp_f<0x141>(v);
   return v;
 }
+
+// ---------------------------------------------------------------- time stamps inside kernels (diagnostic builds only)
+// `make TRACE=1` compiles the stamps in: thread 0 of a traced block stores the 100 MHz device clock into a per-translation-unit
+// table, which the unit's *_trace entry point copies to the host.  Row 0: block JSG_TRACE_BLOCK (default 0), row 1: whatever
+// code path names it explicitly, row 2: the last block of the grid.  Normal builds contain none of this.
+#ifdef JSG_TRACE
+#ifndef JSG_TRACE_BLOCK
+#define JSG_TRACE_BLOCK 0
+#endif
+static __device__ unsigned long long g_trace[3][32];
+__device__ __forceinline__ int trace_row() { return blockIdx.x == JSG_TRACE_BLOCK ? 0 : (blockIdx.x == gridDim.x - 1 ? 2 : -1); }
+__device__ __forceinline__ void trace_stamp(int row, int slot) {
+  if (row >= 0 && threadIdx.x == 0) g_trace[row][slot] = __builtin_amdgcn_s_memrealtime();
+}
+#define JSG_STAMP(slot) jsg::trace_stamp(jsg::trace_row(), slot)
+#define JSG_STAMP_ROW(row, slot) jsg::trace_stamp(row, slot)
+#define JSG_TRACE_ENTRY(name)                                                                              \
+  extern "C" int name(unsigned long long *host_out) {                                                      \
+    JSG_HIP(hipStreamSynchronize(jsg::state().stream));                                                    \
+    JSG_HIP(hipMemcpyFromSymbol(host_out, HIP_SYMBOL(jsg::g_trace), sizeof(jsg::g_trace)));                  \
+    unsigned long long z[3][32] = {};                                                                      \
+    JSG_HIP(hipMemcpyToSymbol(HIP_SYMBOL(jsg::g_trace), z, sizeof(z)));                                     \
+    return 0;                                                                                              \
+  }
+#else
+#define JSG_STAMP(slot) ((void)0)
+#define JSG_STAMP_ROW(row, slot) ((void)0)
+#define JSG_TRACE_ENTRY(name)
+#endif
 
 // ---------------------------------------------------------------- tagged words: data that is its own flag
 // A row that blocks of one launch hand to each other: one 32-bit word per element, the fp16 value below, a version tag

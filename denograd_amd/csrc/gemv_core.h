@@ -34,10 +34,6 @@ struct GemvArgs {
   const uint32_t *x_tagged = nullptr;
   uint32_t x_tag = 0;
   int *err = nullptr;
-  // when set, EPI_STORE / EPI_SWIGLU write their output row here as tagged words (value | y_tag << 16) instead of to y, for
-  // blocks of the same launch that take it as their x_tagged
-  uint32_t *y_tagged = nullptr;
-  uint32_t y_tag = 0;
 };
 
 // ---- weight formats: VEC elements per 16-byte load --------------------------------------------
@@ -213,14 +209,18 @@ template <typename AT, bool COHERENT> __device__ __forceinline__ void stage_x(co
       // blocks that are still producing it.  Eight words spread over the row are watched by one wavefront until they carry
       // the tag (a hint that the row is about there); what decides is the check of every word below.
       if (tid < 64) {
-        const int probe = (tid & 7) * (n / 8);
+        // eight elements spread over the row (a row made of parts that different blocks finish, such as the heads of an
+        // attention row) and the last eight (a row dealt in order to its producers' wavefronts: what is written last)
+        const int probe = (tid & 8) ? n - 8 + (tid & 7) : (tid & 7) * (n / 8);
         for (int it = 0; it < (1 << 18); it++) {
           const uint32_t w = (uint32_t)ld_coherent((const int *)a.x_tagged + probe);
           if (__all((w >> 16) == a.x_tag)) break;
           __builtin_amdgcn_s_sleep(8);
         }
       }
-      __syncthreads();
+      JSG_STAMP(2);
+      lds_barrier();   // only "the probe is through": requests of this wavefront that are in flight stay in flight
+      JSG_STAMP(3);
       // all chunks of a thread are asked for together, again and again until every one carries the tag: one round trip
       // when the row is there, instead of one per chunk
       constexpr int NCH = 2;
@@ -235,6 +235,7 @@ template <typename AT, bool COHERENT> __device__ __forceinline__ void stage_x(co
           }
           if (ok) break;
           if (it > (1 << 18)) { st_coherent(a.err, 1); break; }
+          __builtin_amdgcn_s_sleep(4);   // not there yet: leave the memory system to those who are producing it
         }
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
@@ -246,6 +247,7 @@ template <typename AT, bool COHERENT> __device__ __forceinline__ void stage_x(co
       for (int c = tid; c < nchunks; c += nt) xl[c] = ldx(c);
     }
     __syncthreads();
+    JSG_STAMP(4);
     return;
   }
   const u4_t *wg = (const u4_t *)a.norm_w;
@@ -458,6 +460,12 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
   // LDS elements the staged x needs: in_f rounded up to whole batches (host side)
   static int x_elems(int in_f) { return (((in_f + STEP - 1) / STEP + UNROLL - 1) / UNROLL) * UNROLL * STEP; }
 
+  // Row groups are dealt to wavefronts block by block: wavefront w of block blk (of nblk) takes groups blk + nblk * (w + nw * i),
+  // i = 0, 1, ...  All blocks then have the same number of groups to within one, whatever the number of wavefronts per
+  // block, so they finish together (dealt wavefront by wavefront over the whole grid, the last blocks would be short of work
+  // whenever the groups do not fill every wavefront of the grid equally).
+  __device__ static __forceinline__ int first_group(int blk, int nblk) { return blk + nblk * (int)(threadIdx.x >> 6); }
+
   // issue the loads of item (grp, b)
   __device__ static __forceinline__ void load_item(const GemvArgs &a, Buf &buf, int grp, int b, int pos) {
     const int lane = threadIdx.x & 63, in_f = a.in_f;
@@ -504,7 +512,7 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
 
   // the first item of this wavefront, requested ahead of run()
   __device__ static __forceinline__ void prefetch(const GemvArgs &a, Buf &buf, int pos) {
-    const int grp = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int grp = first_group(blockIdx.x, gridDim.x);
     if (grp < ngroups(a)) load_item(a, buf, grp, 0, pos);
   }
 
@@ -515,7 +523,7 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
   template <int DEPTH> __device__ static __forceinline__ void touch(const GemvArgs &a, int first, uint32_t (&t)[DEPTH]) {
     const int lane = threadIdx.x & 63, nw = blockDim.x >> 6;
     const int ng = ngroups(a), nb = nbatch(a), gstride = gridDim.x * nw;
-    int grp = blockIdx.x * nw + (threadIdx.x >> 6), b = 0;
+    int grp = first_group(blockIdx.x, gridDim.x), b = 0;
     const int v = lane >> 3, line = lane & 7;
     const int u = v / (NM * ROWS), j = (v / ROWS) % NM, r = v % ROWS;
     for (int i = 0; i < first; i++)
@@ -593,18 +601,13 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
         if (lane == r && r0 + r < mrows) {
           float v = val[0][r];
           if (has_res) v = Act<AT>::rn(extra_of<AT>(buf, r) + v);
-          if (a.y_tagged != nullptr) tw_store(a.y_tagged + r0 + r, a.y_tag, v);
-          else store_out(y + r0 + r, v);
+          store_out(y + r0 + r, v);
         }
     } else if constexpr (EPI == EPI_SWIGLU) {
       AT *g = (AT *)a.y;
 #pragma unroll
       for (int r = 0; r < ROWS; r++)
-        if (lane == r && r0 + r < mrows) {
-          const float v = Act<AT>::rn(silu_act<AT>(val[0][r]) * val[1][r]);
-          if (a.y_tagged != nullptr) tw_store(a.y_tagged + r0 + r, a.y_tag, v);
-          else store_out(g + r0 + r, v);
-        }
+        if (lane == r && r0 + r < mrows) store_out(g + r0 + r, Act<AT>::rn(silu_act<AT>(val[0][r]) * val[1][r]));
     } else {
       if (pos < 0 || pos >= a.max_context) return;  // never write outside the cache
       if (w.m == 2) {  // value rows: plain copy into the cache row
@@ -651,7 +654,7 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
     XStage xst;
     if constexpr (EARLY_X) stage_x_issue<AT>(a, xst);
     fill_lut(lut);
-    int grp = blk * nw + wave, b = 0;
+    int grp = first_group(blk, nblk), b = 0;
     if (!preloaded && grp < ng) load_item(a, bufA, grp, 0, pos);
     auto advance = [&](int &g, int &bb) {
       if (++bb == nb) { bb = 0; g += gstride; }

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libjsgrad_hip.so")
 
 F32, F16, BF16 = 0, 1, 2
 W_F32, W_F16, W_I8, W_NF4 = 0, 1, 2, 3
-PROF_KINDS = {"embed": 0, "rmsnorm": 1, "linear": 2, "qkv_rope": 3, "attn_decode": 4, "ffn_gate": 5, "argmax": 6, "decode_step": 7, "gemm": 8, "attn_prefill": 9, "attn_wo": 10, "read_probe": 11, "sample": 12, "ffn": 13}
+PROF_KINDS = {"embed": 0, "rmsnorm": 1, "linear": 2, "qkv_rope": 3, "attn_decode": 4, "ffn_gate": 5, "argmax": 6, "decode_step": 7, "gemm": 8, "attn_prefill": 9, "attn_wo": 10, "read_probe": 11, "sample": 12}
 
 
 class HipError(RuntimeError):
@@ -66,9 +66,6 @@ SIGNATURES: dict[str, tuple[list, object]] = {
     "jsgrad_hip_attn_wo_items": ([_i32, _i32], _i32),
     "jsgrad_hip_attn_wo_fits": ([_i32, _i32, _i32, _i32, _i32, _i32, C.POINTER(_i32), C.POINTER(_i32)], _i32),
     "jsgrad_hip_ffn_gate": ([_i32, _vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _i32, _i32, _i32], _i32),
-    "jsgrad_hip_ffn_workspace_bytes": ([_i32], _sz),
-    "jsgrad_hip_ffn": ([_i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _i32, _i32, _vp, _vp, _i32], _i32),
-    "jsgrad_hip_ffn_status": ([_vp, C.POINTER(_i32)], _i32),
     "jsgrad_hip_argmax": ([_vp, _i32, _vp, _vp, _i32, _i32, _i32], _i32),
     "jsgrad_hip_embed_rows": ([_i32, _vp, _vp, _vp, _i32, _vp, _i32, _i32], _i32),
     "jsgrad_hip_rmsnorm_rows": ([_vp, _vp, _vp, _i32, _i32, _f32], _i32),

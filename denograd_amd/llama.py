@@ -94,14 +94,9 @@ class FeedForward:
         self.w2 = linear(hidden_dim, dim, False)
         self.w3 = linear(dim, hidden_dim, False)  # the gate in Gated Linear Unit
 
-    def call(self, x: Tensor, norm: RMSNorm, ctx: "_Scratch", out: Tensor, state: Tensor | None = None, layer_id: int | None = None) -> Tensor:
+    def call(self, x: Tensor, norm: RMSNorm, ctx: "_Scratch", out: Tensor) -> Tensor:
         """out = x + w2( silu(w1 n) * (w3 n) ), n = norm(x)  (SwiGLU, llama.ts:108-110 with the residual of :126)."""
         sp = lambda l: l.scale.ptr if l.scale is not None else None
-        if ctx.fuse_ffn and state is not None and layer_id is not None:
-            # both matrices in one launch: w2's weights are on their way while the gate row is still being finished
-            check(ffi.load().jsgrad_hip_ffn(self.w1.kind, self.w1.weight.ptr, sp(self.w1), self.w3.weight.ptr, sp(self.w3), self.w2.weight.ptr, sp(self.w2),
-                                            x.ptr, norm.weight.ptr, norm.eps, out.ptr, self.dim, self.hidden_dim, state.ptr, ctx.ffn_ws.ptr, layer_id))
-            return out
         check(ffi.load().jsgrad_hip_ffn_gate(self.w1.kind, self.w1.weight.ptr, sp(self.w1), self.w3.weight.ptr, sp(self.w3), x.ptr, norm.weight.ptr, norm.eps,
                                              ctx.g.ptr, self.dim, self.hidden_dim, act_code(x.dtype)))
         return self.w2.call(ctx.g, out=out, residual=x)
@@ -124,7 +119,7 @@ class TransformerBlock:
 
     def call(self, x: Tensor, state: Tensor, freqs_cis: Tensor, ctx: "_Scratch") -> Tensor:
         h = self.attention.call(x, state, freqs_cis, self.attention_norm, ctx)     # ctx.h2
-        return self.feed_forward.call(h, self.ffn_norm, ctx, out=x, state=state, layer_id=self.attention.layer_id)   # back into x
+        return self.feed_forward.call(h, self.ffn_norm, ctx, out=x)                # back into x
 
     def call_rows(self, x: Tensor, bsz: int, seqlen: int, start_pos: int, state: Tensor, freqs_cis: Tensor, rows: "_RowScratch") -> Tensor:
         """TransformerBlock.call (llama.ts:124-127) on x [bsz*seqlen, dim]; the result is written back into x."""
@@ -159,15 +154,9 @@ class _Scratch:
         self.logits = Tensor.empty((vocab,), dtype, device)
         nbytes = ffi.load().jsgrad_hip_attn_workspace_bytes(n_heads, n_kv_heads, head_dim)
         self.workspace = Tensor.zeros((nbytes,), "uint8", device)
-        # attention + wo as one launch, w1 / w3 / w2 as one launch (set up by Transformer._prepare when the model qualifies)
+        # attention + wo as one launch (set up by Transformer._prepare when the model qualifies)
         self.fuse_attn_wo = False
         self.attn_wo_ws: Tensor | None = None
-        self.fuse_ffn = False
-        self.ffn_ws: Tensor | None = None
-
-    def enable_ffn(self, hidden: int, device: str) -> None:
-        self.ffn_ws = Tensor.zeros((ffi.load().jsgrad_hip_ffn_workspace_bytes(hidden),), "uint8", device)
-        self.fuse_ffn = True
 
     def enable_attn_wo(self, n_heads: int, n_kv_heads: int, head_dim: int, device: str) -> None:
         nbytes = ffi.load().jsgrad_hip_attn_wo_workspace_bytes(n_heads, n_kv_heads, head_dim)
@@ -183,8 +172,6 @@ class _Scratch:
         if self.attn_wo_ws is not None:
             ws = self.attn_wo_ws
             check(ffi.load().jsgrad_hip_memset(ws.ptr + ws.nbytes - self._tagged_row_bytes, 0, self._tagged_row_bytes))
-        if self.ffn_ws is not None:      # the gate row of the fused feed-forward launch is tagged the same way
-            check(ffi.load().jsgrad_hip_memset(self.ffn_ws.ptr + 256, 0, self.ffn_ws.nbytes - 256))
 
 
 class _RowScratch:
@@ -297,7 +284,7 @@ class TinyJit:
 class Transformer:
     def __init__(self, dim: int, hidden_dim: int, n_heads: int, n_layers: int, norm_eps: float, vocab_size: int, linear=Linear, embedding=Embedding,
                  n_kv_heads: int | None = None, rope_theta: float = 10000, max_context: int = 1024, jit: bool = True, feed_forward=FeedForward, device: str = "HIP",
-                 fused_step: bool = False, fuse_attn_wo: bool = True, fuse_ffn: bool = True):
+                 fused_step: bool = False, fuse_attn_wo: bool = True):
         self.dim, self.hidden_dim, self.n_heads, self.vocab_size, self.max_context = dim, hidden_dim, n_heads, vocab_size, max_context
         self.n_kv_heads = n_kv_heads if n_kv_heads is not None else n_heads
         self.rope_theta, self.device = rope_theta, device
@@ -316,7 +303,6 @@ class Transformer:
         # False: one launch per fused op (the faster of the two today); True: the whole step as one persistent kernel
         self.fused_step = fused_step
         self.fuse_attn_wo = fuse_attn_wo   # attention and wo of a layer as one launch, where the model qualifies
-        self.fuse_ffn = fuse_ffn           # w1 / w3 / w2 of a layer as one launch, where the model qualifies
         self._fused: _FusedStep | None = None
         self._rows: _RowScratch | None = None
         # sampling (llama.ts:131-185): (temperature, top_k, top_p, alpha_f, alpha_p) of the current calls; greedy until told otherwise
@@ -338,11 +324,7 @@ class Transformer:
         the host waits for the device anyway (the per-token read of Llama3._call, the end of Llama3.generate)."""
         if self.attn_wo_error():
             raise ffi.HipError("a fused attention + wo launch gave up waiting for its attention row; results after that launch are invalid")
-        if self._ctx is not None and self._ctx.ffn_ws is not None:
-            e = C.c_int(0)
-            check(ffi.load().jsgrad_hip_ffn_status(self._ctx.ffn_ws.ptr, C.byref(e)))
-            if e.value:
-                raise ffi.HipError("a fused feed-forward launch gave up waiting for its gate row; results after that launch are invalid")
+
 
     # ---- plumbing
     @property
@@ -365,10 +347,6 @@ class Transformer:
                     and self.n_heads // self.n_kv_heads in (1, 2, 3, 4) and self.max_context <= 64 * 256 and self.n_heads * hd * 2 <= 64 * 1024
                     and self.n_kv_heads <= 64 and attn_wo_fits(self.n_heads, self.n_kv_heads, hd, self.max_context, wo.kind, self.dim)):
                 self._ctx.enable_attn_wo(self.n_heads, self.n_kv_heads, hd, self.device)
-            ff = self.layers[0].feed_forward
-            if (self.fuse_ffn and self.dtype == "float16" and isinstance(ff, FeedForward) and ff.w1.kind in (ffi.W_F16, ffi.W_I8) and ff.w2.kind == ff.w1.kind
-                    and 2 <= len(self.layers) <= 128 and self.dim % 16 == 0 and self.hidden_dim % 16 == 0 and self.hidden_dim * 2 <= 64 * 1024):
-                self._ctx.enable_ffn(self.hidden_dim, self.device)
             if self.fused_step:
                 self._fused = _FusedStep(self, self._ctx, self._fused_mode())      # raises NotImplementedError for models it was not built for
         return self._ctx

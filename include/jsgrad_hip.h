@@ -268,18 +268,6 @@ size_t jsgrad_hip_attn_wo_workspace_bytes(int n_heads, int n_kv_heads, int head_
 int jsgrad_hip_attn_wo(const void *q, const void *cache_k, const void *cache_v, const int32_t *state, void *workspace, int n_heads, int n_kv_heads,
                        int head_dim, int max_context, int kind, const void *wo, const void *wo_scale, int dim, const void *residual, void *y, int layer);
 int jsgrad_hip_attn_wo_status(const void *workspace, int *host_out_error);
-/* jsgrad_hip_ffn_gate followed by jsgrad_hip_linear(w2, residual = x) of one layer as ONE launch (FeedForward.call,
- * models/llama.ts:108-110, and the residual add of :126): y[dim] = x + w2 . (silu(w1 n) * (w3 n)), n = RMSNorm(x).  Every
- * wavefront requests its first w2 weights as soon as it is done with its rows of w1 / w3, and the gate row reaches all blocks
- * inside the launch.  fp16 activations, fp16 or int8 weights.  state: the device {token, start_pos} words (the position and
- * `layer`, 0..127, tell launches that share a workspace apart).  workspace: jsgrad_hip_ffn_workspace_bytes(hidden) bytes,
- * zero-filled once before first use, one per model.  The wait inside the launch is bounded; jsgrad_hip_ffn_status reads
- * whether one ever ran out. */
-size_t jsgrad_hip_ffn_workspace_bytes(int hidden);
-int jsgrad_hip_ffn(int kind, const void *w1, const void *s1, const void *w3, const void *s3, const void *w2, const void *s2, const void *x,
-                   const void *norm_weight, float eps, void *y, int dim, int hidden, const int32_t *state, void *workspace, int layer);
-int jsgrad_hip_ffn_status(const void *workspace, int *host_out_error);
-
 /* Launch geometry of jsgrad_hip_attn_wo.  _items: blocks that run an attention item (kv heads x chunks of max_context; plain
  * arithmetic, needs no device).  _fits: that number and the number of blocks of the kernel the device holds at once; a launch
  * with more items than that is refused by jsgrad_hip_attn_wo (blocks that are done wait on the device for the attention row,
