@@ -4,11 +4,11 @@
 
 namespace jsg {
 
-constexpr int ATT_THREADS = 1024;   // 16 wavefronts work on an item (attention_core.h requests every row of a chunk up front)
-
-template <typename AT, int HD, int NREP>
-__global__ __launch_bounds__(ATT_THREADS) void attn_decode_kernel(AttnArgs a) {
-  typedef Attn<AT, HD, NREP, ATT_THREADS / 64, false> A;
+// One sequence: blocks of 16 wavefronts (an item is a chain of dependent steps the whole launch waits for).  Several sequences:
+// blocks of 8 wavefronts with chunks of at most 128 rows, several blocks per CU, so that the chains of different items overlap.
+template <typename AT, int HD, int NREP, int NW>
+__global__ __launch_bounds__(NW * 64) void attn_decode_kernel(AttnArgs a) {
+  typedef Attn<AT, HD, NREP, NW, false> A;
   __shared__ typename A::Smem sm;
   const int g = blockIdx.x, split = blockIdx.y;
   if (const int z = blockIdx.z) {   // sequence z of a batch: same position, its own rows of q / out / cache / workspace
@@ -22,23 +22,20 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_decode_kernel(AttnArgs a) {
   const int pos = a.st[1];
   if (pos < 0 || pos >= a.max_context) return;
   const int T = pos + 1;
-  const int chunk = att_chunk_rows(T, a.nsplit);  // <= ATT_CHUNK_MAX, checked on the host against max_context
+  const int chunk = att_chunk_rows(T, a.nsplit, A::CHUNK_CAP);  // the host sized nsplit for this cap
   const int n_active = (T + chunk - 1) / chunk;
   if (split >= n_active) return;
   A::item(a, sm, g, split, T, chunk, n_active);
 }
 
-// chunks the grid and the workspace provide: what the chunk policy can ask for at any T up to max_context
-static int nsplit_for(int max_context, int heads_x_batch) {
-  (void)heads_x_batch;
-  return att_max_chunks(max_context);
-}
+constexpr int ATT_NW_ONE = 16, ATT_NW_MANY = 8;
+static int att_cap(int nw) { return nw * 16 < ATT_CHUNK_MAX ? nw * 16 : ATT_CHUNK_MAX; }
 
-template <typename AT, int HD> static int launch_attn(const AttnArgs &a, int n_rep, int batch = 1) {
-  dim3 grid(a.n_kv_heads, a.nsplit, batch), block(ATT_THREADS);
+template <typename AT, int HD, int NW> static int launch_attn_nw(const AttnArgs &a, int n_rep, int batch) {
+  dim3 grid(a.n_kv_heads, a.nsplit, batch), block(NW * 64);
 #define JSG_REP(N)                                                                                   \
   case N:                                                                                            \
-    JSG_LAUNCH(PROF_ATTN, (attn_decode_kernel<AT, HD, N>), grid, block, 0, a);                         \
+    JSG_LAUNCH(PROF_ATTN, (attn_decode_kernel<AT, HD, N, NW>), grid, block, 0, a);                     \
     break;
   switch (n_rep) {
     JSG_REP(1) JSG_REP(2) JSG_REP(3) JSG_REP(4) JSG_REP(8)
@@ -46,6 +43,10 @@ template <typename AT, int HD> static int launch_attn(const AttnArgs &a, int n_r
   }
 #undef JSG_REP
   return 0;
+}
+// nw: ATT_NW_ONE or ATT_NW_MANY, the shape a.nsplit was sized for
+template <typename AT, int HD> static int launch_attn(const AttnArgs &a, int n_rep, int batch = 1, int nw = ATT_NW_ONE) {
+  return nw == ATT_NW_MANY ? launch_attn_nw<AT, HD, ATT_NW_MANY>(a, n_rep, batch) : launch_attn_nw<AT, HD, ATT_NW_ONE>(a, n_rep, batch);
 }
 
 // ---- the variant that allocates nothing: its workspace is a file-scope device array
@@ -94,13 +95,15 @@ int jsgrad_hip_attn_decode_batch(const void *q, const void *cache_k, const void 
   a.q = q; a.cache_k = cache_k; a.cache_v = cache_v; a.st = st; a.out = out;
   a.counters = (int *)workspace;                                   // [batch][n_kv_heads], densely packed
   a.partial = (float *)((char *)workspace + (size_t)batch * counter_bytes);
-  a.n_kv_heads = n_kv_heads; a.nsplit = nsplit_for(max_context, n_kv_heads * batch); a.max_context = max_context;
+  // several sequences: the smaller block shape, while its chunk length can cover the context with the chunks the merge indexes
+  const int nw = (batch > 1 && max_context <= att_cap(ATT_NW_MANY) * att_cap(ATT_NW_MANY)) ? ATT_NW_MANY : ATT_NW_ONE;
+  a.n_kv_heads = n_kv_heads; a.nsplit = att_max_chunks(max_context, att_cap(nw)); a.max_context = max_context;
   a.scale = (float)(1.0 / sqrt((double)head_dim));
   a.q_bstride = (size_t)n_heads * head_dim * sizeof(_Float16);
   a.cache_bstride = (size_t)max_context * n_kv_heads * head_dim * sizeof(_Float16);
   a.partial_bstride = (size_t)n_heads * 256 * (head_dim + 2);
   const int n_rep = n_heads / n_kv_heads;
-  return head_dim == 64 ? launch_attn<_Float16, 64>(a, n_rep, batch) : launch_attn<_Float16, 128>(a, n_rep, batch);
+  return head_dim == 64 ? launch_attn<_Float16, 64>(a, n_rep, batch, nw) : launch_attn<_Float16, 128>(a, n_rep, batch, nw);
 }
 
 size_t jsgrad_hip_attn_decode_static_max_bytes(void) { return NOALLOC_SCRATCH_BYTES; }
@@ -112,7 +115,7 @@ int jsgrad_hip_attn_decode_static(const void *q, const void *cache_k, const void
   JSG_REQUIRE(n_heads > 0 && n_kv_heads > 0 && max_context > 0, "jsgrad_hip_attn_decode_static: n_heads %d / n_kv_heads %d / max_context %d", n_heads, n_kv_heads, max_context);
   JSG_REQUIRE(max_context <= 256 * ATT_CHUNK_MAX, "jsgrad_hip_attn_decode_static: max_context %d exceeds %d", max_context, 256 * ATT_CHUNK_MAX);
   // counters [0, 256), then one partial result per (head, chunk): only the chunks this max_context can produce are needed
-  const size_t need = 256 + (size_t)n_heads * nsplit_for(max_context, 1) * ((size_t)head_dim + 2) * sizeof(float);
+  const size_t need = 256 + (size_t)n_heads * att_max_chunks(max_context) * ((size_t)head_dim + 2) * sizeof(float);
   JSG_REQUIRE(need <= NOALLOC_SCRATCH_BYTES,
               "jsgrad_hip_attn_decode_static: %d heads of %d at max_context %d need %zu bytes of workspace, the built-in one holds %zu; use jsgrad_hip_attn_decode "
               "with a workspace of its own", n_heads, head_dim, max_context, need, (size_t)NOALLOC_SCRATCH_BYTES);
@@ -142,7 +145,7 @@ int jsgrad_hip_attn_decode(const void *q, const void *cache_k, const void *cache
   a.q = q; a.cache_k = cache_k; a.cache_v = cache_v; a.st = st; a.out = out;
   a.counters = (int *)workspace;
   a.partial = (float *)((char *)workspace + 256);
-  a.n_kv_heads = n_kv_heads; a.nsplit = nsplit_for(max_context, 1); a.max_context = max_context;
+  a.n_kv_heads = n_kv_heads; a.nsplit = att_max_chunks(max_context); a.max_context = max_context;
   a.scale = (float)(1.0 / sqrt((double)head_dim));
   const int n_rep = n_heads / n_kv_heads;
   if (act == JSGRAD_F16) return head_dim == 64 ? launch_attn<_Float16, 64>(a, n_rep) : launch_attn<_Float16, 128>(a, n_rep);

@@ -21,14 +21,19 @@ constexpr int ATT_CHUNK_MAX = 256;  // positions per item held in LDS; also the 
 // fetches one partial result per chunk, so chunks are few and long rather than many and short: 64 rows up to 512 positions,
 // 128 up to 2048, 256 beyond (at most 8 / 16 / T/256 chunks per kv head).
 // `nsplit` chunks is what the workspace and the grid provide: the chunk grows if T would need more.
-__host__ __device__ __forceinline__ int att_chunk_rows(int T, int nsplit) {
-  int c = T <= 512 ? 64 : (T <= 2048 ? 128 : 256);
+// `cap`: the longest chunk the block shape can take (16 rows per wavefront, at most ATT_CHUNK_MAX).
+__host__ __device__ __forceinline__ int att_policy_rows(int T, int cap) {
+  const int c = T <= 512 ? 64 : (T <= 2048 ? 128 : 256);
+  return c < cap ? c : cap;
+}
+__host__ __device__ __forceinline__ int att_chunk_rows(int T, int nsplit, int cap = ATT_CHUNK_MAX) {
+  const int c = att_policy_rows(T, cap);
   const int need = (T + nsplit - 1) / nsplit;
   return c < need ? need : c;
 }
 // chunks a launch must provide for every T up to max_context (the count is not monotonic in T across the policy's steps)
-__host__ __device__ __forceinline__ int att_max_chunks(int max_context) {
-  auto n = [](int T) { const int c = T <= 512 ? 64 : (T <= 2048 ? 128 : 256); return (T + c - 1) / c; };
+__host__ __device__ __forceinline__ int att_max_chunks(int max_context, int cap = ATT_CHUNK_MAX) {
+  auto n = [cap](int T) { const int c = att_policy_rows(T, cap); return (T + c - 1) / c; };
   int m = n(max_context < 512 ? max_context : 512);
   if (max_context > 512) { const int v = n(max_context < 2048 ? max_context : 2048); m = v > m ? v : m; }
   if (max_context > 2048) { const int v = n(max_context); m = v > m ? v : m; }
@@ -72,20 +77,24 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
   static constexpr int EPL = 16 / sizeof(AT);  // K: elements per lane per 128-bit load
   static constexpr int G = HD / EPL;           // K: lanes per cache row
   static constexpr int RPI = 64 / G;           // K: rows per wavefront load
-  static constexpr int KIT = (ATT_CHUNK_MAX + NW * RPI - 1) / (NW * RPI);   // K loads per lane for the longest chunk
+  // Every row of a chunk is requested up front, 16 rows per wavefront at most: the longest chunk this block shape takes.
+  // Sixteen wavefronts (one sequence: few items, each a chain of dependent steps that the launch waits for) take 256 rows;
+  // smaller blocks (many sequences: many items, several blocks per CU overlapping their chains) take shorter chunks.
+  static constexpr int CHUNK_CAP = NW * 16 < ATT_CHUNK_MAX ? NW * 16 : ATT_CHUNK_MAX;
+  static constexpr int KIT = (CHUNK_CAP + NW * RPI - 1) / (NW * RPI);   // K loads per lane for the longest chunk
   static constexpr int EP = 4 / sizeof(AT);    // V: elements per dword
   static constexpr int PIECES = HD / EP;       // V: dwords per row
   static constexpr int LPR = PIECES < 64 ? PIECES : 64;   // V: lanes per row
   static constexpr int RPV = 64 / LPR;         // V: rows per wavefront load (1 or 2)
   static constexpr int IPR = PIECES / LPR;     // V: loads per row (1 or 2)
-  static constexpr int VROWS = (ATT_CHUNK_MAX + NW - 1) / NW;      // rows of the longest chunk per wavefront
+  static constexpr int VROWS = (CHUNK_CAP + NW - 1) / NW;          // rows of the longest chunk per wavefront
   static constexpr int VIT = (VROWS + RPV - 1) / RPV * IPR;        // V loads per lane for the longest chunk
   static_assert(G == 8 || G == 16 || G == 32, "scores are reduced over 8, 16 or 32 lanes per row");
   static_assert(RPV == 1 || RPV == 2, "a V row is 32, 64 or 128 dwords");
   static_assert(NREP <= NW, "one wavefront per query head does the softmax");
   static_assert(KIT <= 8 && VIT <= 32, "all rows of a chunk are requested up front: the block needs enough wavefronts");
   struct Smem {
-    float sc[NREP][ATT_CHUNK_MAX];
+    float sc[NREP][CHUNK_CAP];   // scores / probabilities of the chunk; in the merge, the weights of up to CHUNK_CAP chunks
     __attribute__((aligned(16))) float o_part[NW][NREP][HD];   // every wavefront's partial output; summed in wavefront order
     float m_sh[NREP], l_sh[NREP];
     __attribute__((aligned(16))) AT qs[NREP][HD];   // the query rows of the kv head
@@ -172,7 +181,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
     // rows i, i + 64, ... of the chunk.
     if (wave < NREP) {
       const int j = wave;
-      constexpr int PL = ATT_CHUNK_MAX / 64;
+      constexpr int PL = (CHUNK_CAP + 63) / 64;
       float sv[PL];
       float m = -INFINITY;
 #pragma unroll
@@ -290,7 +299,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
     const int p0 = tid < NPAIR ? tid : 0;        // threads beyond the pairs request pair 0 again (their result is not stored)
     const int j0 = (2 * p0) / HD, d0 = (2 * p0) % HD;
     const float *po0 = base + (size_t)j0 * (HD + 2) + d0;
-    constexpr int MSL = ATT_CHUNK_MAX / 64;   // chunks per lane
+    constexpr int MSL = (CHUNK_CAP + 63) / 64;   // chunks per lane (the host keeps n_active <= CHUNK_CAP)
     uint64_t mls[MSL];                         // wavefront j < NREP: (m, l) of this lane's chunks of head j, requested in one go
     if (wave < NREP) {
 #pragma unroll
@@ -313,7 +322,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
         const int s_ = lane + i * 64;
         if (s_ < n_active) {
           const float w = exp_f32(__uint_as_float((uint32_t)mls[i]) - M);
-          sm.sc[j][s_] = w;  // n_active <= nsplit <= ATT_CHUNK_MAX
+          sm.sc[j][s_] = w;  // n_active <= nsplit <= CHUNK_CAP
           L = fmaf(__uint_as_float((uint32_t)(mls[i] >> 32)), w, L);
         }
       }

@@ -557,7 +557,7 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
 
   // consume item (grp, b) from buf; on the last batch of the group: cross-lane sum, scale, cast, epilogue
   __device__ static __forceinline__ void use_item(const GemvArgs &a, const Buf &buf, int grp, int b, float (&acc)[NM][ROWS], const AT *xs, const float *lut, int pos) {
-    const int lane = threadIdx.x & 63, in_f = a.in_f;
+    const int lane = threadIdx.x & 63;
     const Where w = locate(a, grp);
     if (b == 0) {
 #pragma unroll
