@@ -649,7 +649,7 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
   template <bool EARLY_X = false>
   __device__ static __forceinline__ void run(const GemvArgs &a, AT *xs, float *red, float *lut, Buf &bufA, bool preloaded, int pos, int blk = blockIdx.x,
                                              int nblk = gridDim.x) {
-    const int wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int nw = blockDim.x >> 6;
     const int ng = ngroups(a), nb = nbatch(a), gstride = nblk * nw;
     XStage xst;
     if constexpr (EARLY_X) stage_x_issue<AT>(a, xst);

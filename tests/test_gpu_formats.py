@@ -174,10 +174,10 @@ def test_gguf_checkpoint_loads_to_the_same_model(tmp_path):
     direct_sd = {k: want[inv[k]].astype(np.float16) for k in sd if k != "output.weight"}
     direct_sd["output.weight"] = direct_sd["tok_embeddings.weight"]
     direct = Llama3.from_config(CFG).load_weights(direct_sd)
-    loaded = Llama3(quantize="float16", max_context=CFG["max_context"], args={k: CFG[k] for k in ("dim", "hidden_dim", "n_heads", "n_kv_heads", "n_layers", "norm_eps", "rope_theta", "vocab_size")}).load(path)
+    loaded = Llama3(quantize="float16", temperature=0.0, max_context=CFG["max_context"], args={k: CFG[k] for k in ("dim", "hidden_dim", "n_heads", "n_kv_heads", "n_layers", "norm_eps", "rope_theta", "vocab_size")}).load(path)
     assert loaded.model.dtype == "float16"
     assert _tokens(loaded) == _tokens(direct)
     # and through the int8 quantiser: the same codes as quantising the dequantised values directly
-    q_loaded = Llama3(quantize="int8", max_context=CFG["max_context"], args=loaded.params).load(path)
-    q_direct = Llama3(quantize="int8", max_context=CFG["max_context"], args=loaded.params).load_weights(direct_sd)
+    q_loaded = Llama3(quantize="int8", temperature=0.0, max_context=CFG["max_context"], args=loaded.params).load(path)
+    q_direct = Llama3(quantize="int8", temperature=0.0, max_context=CFG["max_context"], args=loaded.params).load_weights(direct_sd)
     assert _tokens(q_loaded) == _tokens(q_direct)
