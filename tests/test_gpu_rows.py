@@ -306,7 +306,13 @@ def test_attn_decode_batch_equals_per_sequence(hip):
     for b in range(B):
         o = Tensor.empty((H * hd,), "float16")
         check(hip.jsgrad_hip_attn_decode(tq.ptr + b * H * hd * 2, tk.ptr + b * row, tv.ptr + b * row, st.ptr, o.ptr, ws.ptr, H, KV, hd, ctx, ffi.F16))
-        assert np.array_equal(ob.numpy()[b].view(np.uint16), o.numpy().view(np.uint16)), b
+        # the two launches cut the positions into chunks of different lengths (several sequences: shorter chunks, smaller
+        # blocks), so the float sums differ in their last bits: the same values to an fp16 ulp, and mostly the same bits
+        got, one = ob.numpy()[b].astype(np.float32), o.numpy().astype(np.float32)
+        assert np.all(np.abs(got - one) <= np.spacing(np.abs(one).astype(np.float16)).astype(np.float32)), b
+        assert np.mean(got == one) > 0.9, b
+    ref = attention_ref(q, ck, cv, B, 1, pos, H, KV, hd)
+    assert np.allclose(ob.numpy().astype(np.float64), ref, rtol=1e-2, atol=1e-2) and np.max(np.abs(ob.numpy().astype(np.float64) - ref)) < 4e-3
 
 
 def test_row_companions_bit_exact(hip):
