@@ -1,17 +1,34 @@
 // Stand-alone decode attention kernel: grid (n_kv_heads, NSPLIT), one work item per block (see attention_core.h).
 // NSPLIT is fixed from max_context, so the grid does not depend on T and a captured graph replays unchanged while T grows.
 #include "attention_core.h"
+#include "attention_stream.h"
 
 namespace jsg {
 
-// One sequence: blocks of 16 wavefronts (an item is a chain of dependent steps the whole launch waits for).  Several sequences:
-// blocks of 8 wavefronts with chunks of at most 128 rows, several blocks per CU, so that the chains of different items overlap.
-template <typename AT, int HD, int NREP, int NW>
-__global__ __launch_bounds__(NW * 64) void attn_decode_kernel(AttnArgs a) {
-  typedef Attn<AT, HD, NREP, NW, false> A;
+// One sequence (or few): blocks of 16 wavefronts, an item's rows requested up front (attention_core.h).
+constexpr int ATT_NW = 16;
+template <typename AT, int HD, int NREP>
+__global__ __launch_bounds__(ATT_NW * 64) void attn_decode_kernel(AttnArgs a) {
+  typedef Attn<AT, HD, NREP, ATT_NW, false> A;
   __shared__ typename A::Smem sm;
   const int g = blockIdx.x, split = blockIdx.y;
-  if (const int z = blockIdx.z) {   // sequence z of a batch: same position, its own rows of q / out / cache / workspace
+  const int pos = a.st[1];
+  if (pos < 0 || pos >= a.max_context) return;
+  const int T = pos + 1;
+  const int chunk = att_chunk_rows(T, a.nsplit);  // <= ATT_CHUNK_MAX, checked on the host against max_context
+  const int n_active = (T + chunk - 1) / chunk;
+  if (split >= n_active) return;
+  A::item(a, sm, g, split, T, chunk, n_active);
+}
+
+// Many sequences at the same position (grid z): blocks of 4 wavefronts that stream their rows (attention_stream.h).
+constexpr int ATT_STREAM_NW = 4;
+template <int HD, int NREP>
+__global__ __launch_bounds__(ATT_STREAM_NW * 64) void attn_decode_stream_kernel(AttnArgs a) {
+  typedef AttnStream<_Float16, HD, NREP, ATT_STREAM_NW, false> A;
+  __shared__ typename A::Smem sm;
+  const int g = blockIdx.x, split = blockIdx.y;
+  if (const int z = blockIdx.z) {   // sequence z: its own rows of q / out / cache / workspace
     a.q = (const char *)a.q + z * a.q_bstride;
     a.out = (char *)a.out + z * a.q_bstride;
     a.cache_k = (const char *)a.cache_k + z * a.cache_bstride;
@@ -22,20 +39,29 @@ __global__ __launch_bounds__(NW * 64) void attn_decode_kernel(AttnArgs a) {
   const int pos = a.st[1];
   if (pos < 0 || pos >= a.max_context) return;
   const int T = pos + 1;
-  const int chunk = att_chunk_rows(T, a.nsplit, A::CHUNK_CAP);  // the host sized nsplit for this cap
+  const int chunk = att_stream_chunk_rows(T, a.nsplit);  // <= ATT_CHUNK_MAX, checked on the host against max_context
   const int n_active = (T + chunk - 1) / chunk;
   if (split >= n_active) return;
   A::item(a, sm, g, split, T, chunk, n_active);
 }
 
-constexpr int ATT_NW_ONE = 16, ATT_NW_MANY = 8;
-static int att_cap(int nw) { return nw * 16 < ATT_CHUNK_MAX ? nw * 16 : ATT_CHUNK_MAX; }
+// splits of the streaming launch: enough that a chunk fits the LDS score buffer, no more than the merge can index there, and
+// about 8 blocks per CU: the sequences fill the chip by themselves, every extra split only adds its fixed cost (query load,
+// partial store, counter, merge)
+static int stream_nsplit(int max_context, int heads_x_batch) {
+  int by_lds = (max_context + ATT_CHUNK_MAX - 1) / ATT_CHUNK_MAX;
+  int wanted = (max_context + 31) / 32;
+  if (wanted > 64) wanted = 64;
+  const int fill = (2048 + heads_x_batch - 1) / heads_x_batch;
+  if (wanted > fill) wanted = fill;
+  return by_lds > wanted ? by_lds : wanted;
+}
 
-template <typename AT, int HD, int NW> static int launch_attn_nw(const AttnArgs &a, int n_rep, int batch) {
-  dim3 grid(a.n_kv_heads, a.nsplit, batch), block(NW * 64);
+template <typename AT, int HD> static int launch_attn(const AttnArgs &a, int n_rep) {
+  dim3 grid(a.n_kv_heads, a.nsplit, 1), block(ATT_NW * 64);
 #define JSG_REP(N)                                                                                   \
   case N:                                                                                            \
-    JSG_LAUNCH(PROF_ATTN, (attn_decode_kernel<AT, HD, N, NW>), grid, block, 0, a);                     \
+    JSG_LAUNCH(PROF_ATTN, (attn_decode_kernel<AT, HD, N>), grid, block, 0, a);                         \
     break;
   switch (n_rep) {
     JSG_REP(1) JSG_REP(2) JSG_REP(3) JSG_REP(4) JSG_REP(8)
@@ -44,9 +70,18 @@ template <typename AT, int HD, int NW> static int launch_attn_nw(const AttnArgs 
 #undef JSG_REP
   return 0;
 }
-// nw: ATT_NW_ONE or ATT_NW_MANY, the shape a.nsplit was sized for
-template <typename AT, int HD> static int launch_attn(const AttnArgs &a, int n_rep, int batch = 1, int nw = ATT_NW_ONE) {
-  return nw == ATT_NW_MANY ? launch_attn_nw<AT, HD, ATT_NW_MANY>(a, n_rep, batch) : launch_attn_nw<AT, HD, ATT_NW_ONE>(a, n_rep, batch);
+template <int HD> static int launch_attn_stream(const AttnArgs &a, int n_rep, int batch) {
+  dim3 grid(a.n_kv_heads, a.nsplit, batch), block(ATT_STREAM_NW * 64);
+#define JSG_REP(N)                                                                                   \
+  case N:                                                                                            \
+    JSG_LAUNCH(PROF_ATTN, (attn_decode_stream_kernel<HD, N>), grid, block, 0, a);                      \
+    break;
+  switch (n_rep) {
+    JSG_REP(1) JSG_REP(2) JSG_REP(3) JSG_REP(4) JSG_REP(8)
+    default: return fail("jsgrad_hip_attn_decode_batch: n_heads/n_kv_heads = %d is not one of 1,2,3,4,8", n_rep);
+  }
+#undef JSG_REP
+  return 0;
 }
 
 // ---- the variant that allocates nothing: its workspace is a file-scope device array
@@ -95,15 +130,13 @@ int jsgrad_hip_attn_decode_batch(const void *q, const void *cache_k, const void 
   a.q = q; a.cache_k = cache_k; a.cache_v = cache_v; a.st = st; a.out = out;
   a.counters = (int *)workspace;                                   // [batch][n_kv_heads], densely packed
   a.partial = (float *)((char *)workspace + (size_t)batch * counter_bytes);
-  // several sequences: the smaller block shape, while its chunk length can cover the context with the chunks the merge indexes
-  const int nw = (batch > 1 && max_context <= att_cap(ATT_NW_MANY) * att_cap(ATT_NW_MANY)) ? ATT_NW_MANY : ATT_NW_ONE;
-  a.n_kv_heads = n_kv_heads; a.nsplit = att_max_chunks(max_context, att_cap(nw)); a.max_context = max_context;
+  a.n_kv_heads = n_kv_heads; a.nsplit = stream_nsplit(max_context, n_kv_heads * batch); a.max_context = max_context;
   a.scale = (float)(1.0 / sqrt((double)head_dim));
   a.q_bstride = (size_t)n_heads * head_dim * sizeof(_Float16);
   a.cache_bstride = (size_t)max_context * n_kv_heads * head_dim * sizeof(_Float16);
   a.partial_bstride = (size_t)n_heads * 256 * (head_dim + 2);
   const int n_rep = n_heads / n_kv_heads;
-  return head_dim == 64 ? launch_attn<_Float16, 64>(a, n_rep, batch, nw) : launch_attn<_Float16, 128>(a, n_rep, batch, nw);
+  return head_dim == 64 ? launch_attn_stream<64>(a, n_rep, batch) : launch_attn_stream<128>(a, n_rep, batch);
 }
 
 size_t jsgrad_hip_attn_decode_static_max_bytes(void) { return NOALLOC_SCRATCH_BYTES; }

@@ -91,7 +91,6 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
   static constexpr int VIT = (VROWS + RPV - 1) / RPV * IPR;        // V loads per lane for the longest chunk
   static_assert(G == 8 || G == 16 || G == 32, "scores are reduced over 8, 16 or 32 lanes per row");
   static_assert(RPV == 1 || RPV == 2, "a V row is 32, 64 or 128 dwords");
-  static_assert(NREP <= NW, "one wavefront per query head does the softmax");
   static_assert(KIT <= 8 && VIT <= 32, "all rows of a chunk are requested up front: the block needs enough wavefronts");
   struct Smem {
     float sc[NREP][CHUNK_CAP];   // scores / probabilities of the chunk; in the merge, the weights of up to CHUNK_CAP chunks
@@ -179,8 +178,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
     lds_barrier();
     // Wavefront j does the whole softmax of head j by itself - maximum, exp, sum - with no barrier in between: lane i holds
     // rows i, i + 64, ... of the chunk.
-    if (wave < NREP) {
-      const int j = wave;
+    for (int j = wave; j < NREP; j += NW) {
       constexpr int PL = (CHUNK_CAP + 63) / 64;
       float sv[PL];
       float m = -INFINITY;
@@ -300,7 +298,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
     const int j0 = (2 * p0) / HD, d0 = (2 * p0) % HD;
     const float *po0 = base + (size_t)j0 * (HD + 2) + d0;
     constexpr int MSL = (CHUNK_CAP + 63) / 64;   // chunks per lane (the host keeps n_active <= CHUNK_CAP)
-    uint64_t mls[MSL];                         // wavefront j < NREP: (m, l) of this lane's chunks of head j, requested in one go
+    uint64_t mls[MSL];                         // wavefront j: (m, l) of this lane's chunks of head j, requested in one go
     if (wave < NREP) {
 #pragma unroll
       for (int i = 0; i < MSL; i++)
@@ -309,8 +307,12 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
     uint64_t part[MB];
 #pragma unroll
     for (int u = 0; u < MB; u++) part[u] = ld_pair(po0, u);
-    if (wave < NREP) {
-      const int j = wave;
+    for (int j = wave; j < NREP; j += NW) {
+      if (j != wave) {     // more query heads than wavefronts: the further heads of this wavefront, one round trip each
+#pragma unroll
+        for (int i = 0; i < MSL; i++)
+          if (i * 64 < n_active) mls[i] = ld_pair(base + (size_t)j * (HD + 2) + HD, lane + i * 64);
+      }
       float M = -INFINITY;
 #pragma unroll
       for (int i = 0; i < MSL; i++)

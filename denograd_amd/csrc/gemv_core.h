@@ -460,11 +460,11 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
   // LDS elements the staged x needs: in_f rounded up to whole batches (host side)
   static int x_elems(int in_f) { return (((in_f + STEP - 1) / STEP + UNROLL - 1) / UNROLL) * UNROLL * STEP; }
 
-  // Row groups are dealt to wavefronts block by block: wavefront w of block blk (of nblk) takes groups blk + nblk * (w + nw * i),
-  // i = 0, 1, ...  All blocks then have the same number of groups to within one, whatever the number of wavefronts per
-  // block, so they finish together (dealt wavefront by wavefront over the whole grid, the last blocks would be short of work
-  // whenever the groups do not fill every wavefront of the grid equally).
-  __device__ static __forceinline__ int first_group(int blk, int nblk) { return blk + nblk * (int)(threadIdx.x >> 6); }
+  // Row groups are dealt to the wavefronts of the grid in order: wavefront w of block blk (of nblk) takes groups
+  // (blk * nw + w) + nblk * nw * i, i = 0, 1, ...  The wavefronts of a block then stream neighbouring rows (one contiguous
+  // piece of the matrix at a time, which the memory system rewards: dealt block by block, rows nblk apart, the SwiGLU launch
+  // measured 6 % slower).
+  __device__ static __forceinline__ int first_group(int blk, int nblk) { (void)nblk; return blk * (int)(blockDim.x >> 6) + (int)(threadIdx.x >> 6); }
 
   // issue the loads of item (grp, b)
   __device__ static __forceinline__ void load_item(const GemvArgs &a, Buf &buf, int grp, int b, int pos) {
