@@ -567,6 +567,9 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; u++) {
+      // a k-step that lies wholly behind the end of the row (the last batch of a row whose length is not a multiple of the
+      // batch) has only reloaded vectors against zero padding: nothing to add.  The same for every lane: a scalar branch.
+      if ((b * UNROLL + u) * STEP >= a.in_f) continue;
       const int k = (b * UNROLL + u) * STEP + lane * VEC;   // may lie in the zero padding of xs
       XFrag<AT, VEC> xf;
       xf.load(xs + k);
