@@ -19,8 +19,12 @@ namespace jsg {
 
 // One block of 16 wavefronts per CU: an attention item is worked on by 16 wavefronts (its chain of dependent steps is what the
 // launch waits for), and the attention row is fetched by 256 blocks instead of 1024.
-constexpr int AW_THREADS = 1024;
+#ifndef JSG_AW_THREADS
+#define JSG_AW_THREADS 1024
+#endif
+constexpr int AW_THREADS = JSG_AW_THREADS;
 constexpr int AW_WAVES = AW_THREADS / 64;
+constexpr int AW_CHUNK_CAP = AW_WAVES * 16 < ATT_CHUNK_MAX ? AW_WAVES * 16 : ATT_CHUNK_MAX;   // attention_core.h: 16 rows per wavefront
 
 template <int KIND, int HD, int NREP>
 __global__ __launch_bounds__(AW_THREADS) void attn_wo_kernel(AttnArgs at, GemvArgs a, int layer) {
@@ -49,7 +53,7 @@ __global__ __launch_bounds__(AW_THREADS) void attn_wo_kernel(AttnArgs at, GemvAr
   bool has_item = false;
   if (pos >= 0 && pos < at.max_context) {
     const int T = pos + 1;
-    const int chunk = att_chunk_rows(T, at.nsplit);   // <= ATT_CHUNK_MAX, checked on the host against max_context
+    const int chunk = att_chunk_rows(T, at.nsplit, AW_CHUNK_CAP);   // the host sized nsplit for max_context and this cap
     const int n_active = (T + chunk - 1) / chunk;
     const int id = blockIdx.x;
     has_item = id < at.n_kv_heads * n_active;
@@ -72,7 +76,7 @@ __global__ __launch_bounds__(AW_THREADS) void attn_wo_kernel(AttnArgs at, GemvAr
   G::run(a, (AT *)smem, red, lut, buf, preloaded, 0, wo_blk, wo_nblk);
 }
 
-static int aw_nsplit(int max_context) { return att_max_chunks(max_context); }
+static int aw_nsplit(int max_context) { return att_max_chunks(max_context, AW_CHUNK_CAP); }
 
 // Blocks of attn_wo_kernel<KIND, HD, n_rep> the device can hold at once (occupancy x CUs).  The blocks that run attention
 // items are the first `items` of the grid; the rest, and the attention blocks themselves once their item is done, wait in
