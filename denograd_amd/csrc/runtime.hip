@@ -4,6 +4,9 @@
 #include <stdarg.h>
 #include <string.h>
 
+#include <stdlib.h>
+
+#include <unordered_map>
 #include <vector>
 
 #include "common.h"
@@ -48,6 +51,39 @@ bool prof_events(int kind, hipEvent_t *start, hipEvent_t *stop) {
   return true;
 }
 
+
+// ---- device memory: blocks that were freed wait, by size class, for the next request of that class
+// (LRUAllocator, /root/reference/jsgrad/runtime/allocator.ts:53-77).  Every launch and copy of this library is queued on one
+// in-order stream, so a block can change hands without waiting for the stream: whatever still reads the old contents
+// was queued before anything the new owner queues.  Memory goes back to the driver only where the stream is waited for
+// anyway (jsgrad_hip_sync, a failed hipMalloc, jsgrad_hip_free_cache), never from jsgrad_hip_free.
+struct MemCache {
+  std::unordered_map<void *, size_t> live;                // every block handed out -> bytes of its class
+  std::unordered_map<size_t, std::vector<void *>> idle;   // freed blocks by class, last freed on top
+  size_t live_bytes = 0, idle_bytes = 0;
+  size_t limit = 0;                                       // idle bytes beyond which the next stream wait gives them back
+  bool enabled = true;                                    // LRU=0 switches the cache off (allocator.ts:73)
+};
+static MemCache g_mem;
+
+// Classes are fine enough to waste under 2 % and coarse enough that tensors of nearly one size share blocks.
+static size_t mem_class(size_t n) {
+  const size_t step = n <= (64u << 10) ? 256 : n <= (4u << 20) ? (4u << 10) : n <= (256u << 20) ? (256u << 10) : (4u << 20);
+  return (n + step - 1) / step * step;
+}
+// The stream must have been waited for.
+static int mem_release_idle() {
+  hipError_t first = hipSuccess;
+  for (auto &kv : g_mem.idle)
+    for (void *p : kv.second) {
+      const hipError_t e = hipFree(p);
+      if (e != hipSuccess && first == hipSuccess) first = e;
+    }
+  g_mem.idle.clear();
+  g_mem.idle_bytes = 0;
+  return first == hipSuccess ? 0 : fail_hip(first, "hipFree");
+}
+
 }  // namespace jsg
 
 using jsg::state;
@@ -69,6 +105,11 @@ int jsgrad_hip_init(int device) {
   JSG_REQUIRE(strncmp(p.gcnArchName, "gfx950", 6) == 0, "jsgrad_hip_init: this library holds gfx950 code only, device is %s", p.gcnArchName);
   s.cu_count = p.multiProcessorCount;
   JSG_HIP(hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking));
+  {
+    const char *lru = getenv("LRU"), *mb = getenv("JSGRAD_HIP_CACHE_MB");
+    jsg::g_mem.enabled = !(lru && atoi(lru) == 0);
+    jsg::g_mem.limit = mb ? (size_t)strtoull(mb, nullptr, 10) << 20 : p.totalGlobalMem / 8;
+  }
   s.device = device;
   s.ready = true;
   return 0;
@@ -91,15 +132,66 @@ int jsgrad_hip_malloc(size_t nbytes, void **host_out_ptr) {
   JSG_READY();
   JSG_REQUIRE(nbytes > 0, "alloc size must be positive, getting %zu", nbytes);
   JSG_REQUIRE(!state().capturing, "jsgrad_hip_malloc during graph capture");
-  JSG_HIP(hipMalloc(host_out_ptr, nbytes));
+  jsg::MemCache &m = jsg::g_mem;
+  const size_t cls = jsg::mem_class(nbytes);
+  auto it = m.idle.find(cls);
+  void *p = nullptr;
+  if (it != m.idle.end() && !it->second.empty()) {
+    p = it->second.back();
+    it->second.pop_back();
+    m.idle_bytes -= cls;
+  } else {
+    if (m.idle_bytes > m.limit) {
+      JSG_HIP(hipStreamSynchronize(state().stream));
+      if (int r = jsg::mem_release_idle()) return r;
+    }
+    hipError_t e = hipMalloc(&p, cls);
+    if (e != hipSuccess && m.idle_bytes > 0) {
+      // out of memory with blocks lying idle: give them back and ask again (allocator.ts:60-66)
+      (void)hipGetLastError();
+      JSG_HIP(hipStreamSynchronize(state().stream));
+      if (int r = jsg::mem_release_idle()) return r;
+      e = hipMalloc(&p, cls);
+    }
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      return jsg::fail_hip(e, "hipMalloc");
+    }
+  }
+  m.live[p] = cls;
+  m.live_bytes += cls;
+  *host_out_ptr = p;
   return 0;
 }
 int jsgrad_hip_free(void *ptr) {
   JSG_READY();
   if (!ptr) return 0;
   JSG_REQUIRE(!state().capturing, "jsgrad_hip_free during graph capture");
+  jsg::MemCache &m = jsg::g_mem;
+  auto it = m.live.find(ptr);
+  JSG_REQUIRE(it != m.live.end(), "jsgrad_hip_free: %p was not handed out by jsgrad_hip_malloc (or was freed already)", ptr);
+  const size_t cls = it->second;
+  m.live.erase(it);
+  m.live_bytes -= cls;
+  if (!m.enabled) {
+    JSG_HIP(hipStreamSynchronize(state().stream));
+    JSG_HIP(hipFree(ptr));
+    return 0;
+  }
+  m.idle[cls].push_back(ptr);
+  m.idle_bytes += cls;
+  return 0;
+}
+int jsgrad_hip_free_cache(void) {
+  JSG_READY();
+  JSG_REQUIRE(!state().capturing, "jsgrad_hip_free_cache during graph capture");
   JSG_HIP(hipStreamSynchronize(state().stream));
-  JSG_HIP(hipFree(ptr));
+  return jsg::mem_release_idle();
+}
+int jsgrad_hip_mem_info(size_t *host_out_live_bytes, size_t *host_out_idle_bytes) {
+  JSG_READY();
+  if (host_out_live_bytes) *host_out_live_bytes = jsg::g_mem.live_bytes;
+  if (host_out_idle_bytes) *host_out_idle_bytes = jsg::g_mem.idle_bytes;
   return 0;
 }
 int jsgrad_hip_copyin(void *dst, const void *host_src, size_t nbytes) {
@@ -128,6 +220,7 @@ int jsgrad_hip_sync(void) {
   JSG_READY();
   JSG_REQUIRE(!state().capturing, "jsgrad_hip_sync during graph capture");
   JSG_HIP(hipStreamSynchronize(state().stream));
+  if (jsg::g_mem.idle_bytes > jsg::g_mem.limit) return jsg::mem_release_idle();
   return 0;
 }
 

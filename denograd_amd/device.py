@@ -16,7 +16,7 @@ import tempfile
 
 import numpy as np
 
-from . import ffi
+from . import diskcache, ffi
 from .ffi import HipError, check
 
 DTYPES = {"float32": (np.float32, ffi.F32), "float16": (np.float16, ffi.F16), "int8": (np.int8, None), "uint8": (np.uint8, None),
@@ -50,6 +50,17 @@ class HIPAllocator:
 
     def _free(self, opaque: int, options=None) -> None:
         check(self.lib.jsgrad_hip_free(opaque))
+
+    def free_cache(self) -> None:
+        """LRUAllocator.free_cache (allocator.ts:65-70).  The cache itself lives in the library, behind _alloc/_free: a freed
+        block waits there for the next request of its size class, and `free` (called from Buffer finalisers) never waits."""
+        check(self.lib.jsgrad_hip_free_cache())
+
+    def mem_info(self) -> tuple[int, int]:
+        """(bytes handed out, bytes lying idle in the cache)."""
+        live, idle = C.c_size_t(0), C.c_size_t(0)
+        check(self.lib.jsgrad_hip_mem_info(C.byref(live), C.byref(idle)))
+        return live.value, idle.value
 
     def _copyin(self, dest: int, src) -> None:
         mv = np.ascontiguousarray(src)
@@ -104,25 +115,40 @@ class HIPCompiler:
     """Compiler (allocator.ts:123-139) for generic (non-Llama) kernels: HIP source -> gfx950 code object.
     The CPU counterpart shells out to clang (ops_clang.ts:12-25); this one shells out to hipcc --genco."""
 
-    def __init__(self, arch: str = "gfx950", hipcc: str = "/opt/rocm/bin/hipcc"):
+    FLAGS = ["-O3", "-include", "hip/hip_runtime.h", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+    def __init__(self, arch: str = "gfx950", hipcc: str = "/opt/rocm/bin/hipcc", cachekey: str | None = "compile_hip_gfx950"):
         self.arch, self.hipcc = arch, hipcc
+        # Compiler's constructor (allocator.ts:125-127): no key, no cache
+        self.cachekey = None if os.environ.get("DISABLE_COMPILER_CACHE") else cachekey
         self.cache: dict[str, bytes] = {}
+        self.compiles = 0       # hipcc runs of this object (tests and DEBUG output)
 
     def compile(self, src: str) -> bytes:
+        self.compiles += 1
         with tempfile.TemporaryDirectory() as d:
             code, out = os.path.join(d, "k.hip"), os.path.join(d, "k.co")
             with open(code, "w") as f:
                 f.write(src)
-            r = subprocess.run([self.hipcc, "--genco", f"--offload-arch={self.arch}", "-O3", "-include", "hip/hip_runtime.h", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-                                code, "-o", out], capture_output=True, text=True)
+            r = subprocess.run([self.hipcc, "--genco", f"--offload-arch={self.arch}", *self.FLAGS, code, "-o", out], capture_output=True, text=True)
             if r.returncode != 0:
                 raise CompileError(r.stderr)
             with open(out, "rb") as f:
                 return f.read()
 
     def compile_cached(self, src: str) -> bytes:
-        if src not in self.cache:
-            self.cache[src] = self.compile(src)
+        """Compiler.compile_cached (allocator.ts:129-137): the code object comes from the disk cache when this source was
+        compiled before, by this process or an earlier one; in front of it, a dictionary for this process."""
+        if src in self.cache:
+            return self.cache[src]
+        lib = diskcache.disk_get(self.cachekey, src) if self.cachekey else None
+        if lib is None:
+            if os.environ.get("ASSERT_COMPILE"):
+                raise RuntimeError(f"tried to compile with ASSERT_COMPILE set\n{src}")
+            lib = self.compile(src)
+            if self.cachekey is not None:
+                diskcache.disk_put(self.cachekey, src, lib)
+        self.cache[src] = bytes(lib)
         return self.cache[src]
 
 

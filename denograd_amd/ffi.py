@@ -32,6 +32,8 @@ SIGNATURES: dict[str, tuple[list, object]] = {
     "jsgrad_hip_cu_count": ([C.POINTER(_i32)], _i32),
     "jsgrad_hip_malloc": ([_sz, _pp], _i32),
     "jsgrad_hip_free": ([_vp], _i32),
+    "jsgrad_hip_free_cache": ([], _i32),
+    "jsgrad_hip_mem_info": ([C.POINTER(_sz), C.POINTER(_sz)], _i32),
     "jsgrad_hip_copyin": ([_vp, _vp, _sz], _i32),
     "jsgrad_hip_copyout": ([_vp, _vp, _sz], _i32),
     "jsgrad_hip_copy": ([_vp, _vp, _sz], _i32),

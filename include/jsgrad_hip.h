@@ -43,10 +43,20 @@ int jsgrad_hip_device_name(char *host_out, size_t cap);
 /* Number of compute units (used to size grids host-side). */
 int jsgrad_hip_cu_count(int *host_out);
 
-/* Allocator._alloc / _free (allocator.ts:40-41).  size 0 is an error as in Allocator.alloc (:30-33).
- * free may be called at any time (Buffer finalisers, jsgrad/device.ts:72-74): it waits for the stream. */
+/* Allocator._alloc / _free (allocator.ts:40-41) with LRUAllocator's reuse behind them (allocator.ts:53-77).  size 0 is an
+ * error as in Allocator.alloc (:30-33).  A request is rounded up to a size class; a freed block waits for the next
+ * request of its class and changes hands without a wait (one in-order stream serves every launch and copy).  free may
+ * be called at any time (Buffer finalisers, jsgrad/device.ts:72-74) and never waits for the stream; memory returns to
+ * the driver at the next jsgrad_hip_sync once more than JSGRAD_HIP_CACHE_MB (default: an eighth of the device) lies
+ * idle, when hipMalloc runs out, or through jsgrad_hip_free_cache.  LRU=0 in the environment turns reuse off
+ * (allocator.ts:73): free then waits for the stream and calls hipFree.  A pointer that jsgrad_hip_malloc did not hand
+ * out, or a second free of one that it did, is an error. */
 int jsgrad_hip_malloc(size_t nbytes, void **host_out_ptr);
 int jsgrad_hip_free(void *ptr);
+/* LRUAllocator.free_cache (allocator.ts:65-70): wait for the stream and give every idle block back to the driver. */
+int jsgrad_hip_free_cache(void);
+/* Bytes handed out and bytes lying idle, in size classes (the library's view of GlobalCounters.mem_used, device.ts:128,135). */
+int jsgrad_hip_mem_info(size_t *host_out_live_bytes, size_t *host_out_idle_bytes);
 /* Allocator._copyin / _copyout (allocator.ts:42-43).  copyout returns after the data is in host memory. */
 int jsgrad_hip_copyin(void *dst, const void *host_src, size_t nbytes);
 int jsgrad_hip_copyout(void *host_dst, const void *src, size_t nbytes);
