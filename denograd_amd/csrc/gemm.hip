@@ -659,6 +659,270 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_gemm_kernel(GemmArgs a) 
   }
 }
 
+// ---- at most 16 rows, int8 weights: whole stretches of weight rows, turned into operand layout through LDS -----------------
+//
+// The kernel above asks for 64 bytes of each of 16 rows per load and lives for 16 rows.  Measured with loads alone, that
+// map reaches 4.0 TB/s where 512 contiguous bytes per row and wavefronts that keep streaming reach 5.0, and the kernel
+// itself stays far below its own map: a block is over before its pipeline has filled, and every block reads all of x.
+// Here a block stays on its compute unit and walks a list of units of work; a unit is COLS output columns times a K range.
+// A step of a wavefront is a tile of 16 weight rows times 512 bytes (one x chunk): eight loads of 1 KiB = two rows, held
+// in a ring of NS steps of registers (what is in flight is bounded by registers, and eight wavefronts per compute unit
+// with two to three steps each keep ~150 KiB on their way; the same ring in LDS would hold less than half).  A step that
+// has arrived is written to a 16 x 528-byte patch of LDS that belongs to the wavefront and read back in the matrix
+// instruction's operand layout (lane = row, 8 K elements = 64 bits), rows 16 bytes apart modulo the bank cycle, so the
+// 32 lanes of a read pass hit 64 different banks.  x goes through LDS as above (the fifth wavefront moves it), but one
+// chunk now serves 64 or 128 weight rows instead of 16.
+//
+// Matrices with few rows are split along K as well (wo, w2: 4096 rows): the partial accumulators go to a workspace that
+// belongs to the library, a counter per (column group, wavefront) tells the last arriver, and that wavefront adds the
+// parts in K order - the result does not depend on which block finishes last.
+constexpr int SG_THREADS = 320;
+constexpr int SG_KC = 512;                                    // K elements per x chunk = bytes of a weight row per step
+constexpr int SG_XB = 3;                                      // x chunks in LDS
+constexpr int SG_XLS = SG_KC + 8;                             // halves per LDS row of x
+#ifndef JSG_SG_NS
+#define JSG_SG_NS 3
+#endif
+constexpr int SG_NS = JSG_SG_NS;                                      // steps in a wavefront's ring
+constexpr int SG_WLS = SG_KC + 16;                            // bytes per LDS row of a weight tile
+constexpr size_t SG_LDS = (size_t)SG_XB * 16 * SG_XLS * 2 + (size_t)4 * 16 * SG_WLS;
+constexpr size_t SG_WS_BYTES = 8u << 20;
+constexpr int SG_MAX_GROUPS = 4096;
+static __device__ __align__(256) unsigned char sg_scratch[SG_WS_BYTES];
+static __device__ int sg_counters[4 * SG_MAX_GROUPS];
+
+template <int EPI, int TPW> struct SgShape {
+  static constexpr int NMAT = EPI == GEPI_SWIGLU ? 2 : 1;
+  static_assert(TPW % NMAT == 0, "w1 and w3 tiles of one column tile sit in one wavefront");
+  static constexpr int CT = TPW / NMAT;                       // column tiles per wavefront
+  static constexpr int COLS = 4 * CT * 16;                    // output columns per unit
+};
+
+struct SgArgs {
+  GemmArgs g;
+  int groups, splitk, nck;                                    // column groups, K parts, x chunks per part
+  float *ws;
+  int *counters;
+};
+
+template <int EPI, int TPW>
+__global__ __launch_bounds__(SG_THREADS, 1) void stream_gemm_kernel(SgArgs sa) {
+  typedef SgShape<EPI, TPW> S;
+  constexpr int NMAT = S::NMAT, NS = SG_NS;
+  const GemmArgs &a = sa.g;
+  extern __shared__ __align__(16) unsigned char sg_lds[];
+  _Float16 *xl = (_Float16 *)sg_lds;                          // SG_XB x [16][SG_XLS]
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l16 = lane & 15, lq = lane >> 4;
+  const int units = sa.groups * sa.splitk, nck = sa.nck;
+  const int my_units = (units - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+  const int CS = my_units * nck;                              // x chunks this block walks
+
+  if (wave == 4) {
+    // ---- the x mover: chunk cs of the block is chunk part * nck + cs % nck of x; one chunk ahead of the readers
+    auto move = [&](int cs) {
+      const int unit = blockIdx.x + (cs / nck) * gridDim.x;
+      const int kc = (unit % sa.splitk) * nck + (cs % nck + unit / sa.splitk) % nck;
+      _Float16 *dst = xl + (cs % SG_XB) * 16 * SG_XLS;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int m = r < a.M ? r : a.M - 1;                  // rows past the end are computed and never stored
+        const _Float16 *src = a.x + (size_t)m * a.K + (size_t)kc * SG_KC + lane * 8;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src, (__attribute__((address_space(3))) void *)(dst + r * SG_XLS), 16, 0, 0);
+      }
+    };
+    int issued = 0;
+    auto landed = [&](int target) {                           // the direct loads complete in order, 16 per chunk
+      const int behind = issued - target - 1;
+      if (behind >= 2) asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
+      else if (behind == 1) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    };
+    while (issued < SG_XB - 1 && issued < CS) move(issued++);
+    landed(0);
+    sk_barrier();
+    for (int cs = 0; cs < CS; cs++) {
+      if (issued < CS) move(issued++);                        // into the buffer of chunk cs - 1, whose readers are past their barrier
+      if (cs + 1 < CS) landed(cs + 1);
+      sk_barrier();
+    }
+    return;
+  }
+
+  unsigned char *stg = sg_lds + (size_t)SG_XB * 16 * SG_XLS * 2 + (size_t)wave * 16 * SG_WLS;   // this wavefront's tile
+  // load side: a load is 1 KiB = two rows of the tile; lane -> (row of the pair, 16-byte piece)
+  const int sub = lane >> 5;
+  const uint32_t wr_off = (uint32_t)(sub * SG_WLS + (lane & 31) * 16);
+  // read side: lane (l16, lq) takes 8 bytes of row l16 per matrix instruction
+  const uint32_t rd_off = (uint32_t)(l16 * SG_WLS + lq * 8);
+  const int xoff = l16 * SG_XLS + lq * 8;
+
+  // first weight row of tile tt of this wavefront in column group grp, and the matrix it belongs to
+  auto tile_of = [&](int grp, int tt, const unsigned char *&w, const _Float16 *&sc, int &row) {
+    const int n = grp * S::COLS + (wave * S::CT + tt / NMAT) * 16;
+    if constexpr (EPI == GEPI_SWIGLU) { w = (const unsigned char *)(tt % NMAT ? a.w1 : a.w0); sc = tt % NMAT ? a.s1 : a.s0; row = n; }
+    else if constexpr (EPI == GEPI_ROPE_KV) {
+      if (n < a.n0) { w = (const unsigned char *)a.w0; sc = a.s0; row = n; }
+      else if (n < a.n0 + a.n1) { w = (const unsigned char *)a.w1; sc = a.s1; row = n - a.n0; }
+      else { w = (const unsigned char *)a.w2; sc = a.s2; row = n - a.n0 - a.n1; }
+    } else { w = (const unsigned char *)a.w0; sc = a.s0; row = n; }
+  };
+
+  // Step gs of this wavefront: tile gs % TPW of x chunk gs / TPW.  The scale of the tile's row l16 travels with the step.
+  const int GS = CS * TPW;
+  u4_t ring[NS][8];
+  h2_t rscale[NS];
+  auto issue = [&](int gs, u4_t (&dst)[8], h2_t &scale) {
+    const int cs = gs / TPW, tt = gs % TPW;
+    const int unit = blockIdx.x + (cs / nck) * gridDim.x;
+    const int grp = unit / sa.splitk, part = unit % sa.splitk, c = cs % nck;
+    const unsigned char *w; const _Float16 *sc; int row;
+    tile_of(grp, tt, w, sc, row);
+    const _Float16 sv = sc[row + l16];
+    scale = h2_t{sv, sv};
+    // Column group grp starts its walk through K at chunk grp % nck and wraps around: at any moment the blocks of the
+    // launch read at different offsets inside the weight rows, which are a power of two apart in memory
+    const unsigned char *src = w + (size_t)(row + sub) * a.K + (size_t)(part * nck + (c + grp) % nck) * SG_KC + (lane & 31) * 16;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      dst[i] = ldg_stream16(src + (size_t)(2 * i) * a.K);
+      __builtin_amdgcn_sched_barrier(0);                      // issued in the order they are used: the waits count on it
+    }
+  };
+
+  // ---- epilogue of one 16x16 tile.  Accumulator r of a lane is output row 4 * (lane / 16) + r, column lane % 16.
+  auto epilogue = [&](const f4_t (&tot)[NMAT], int n_tile) {
+    const int n = n_tile + l16;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int m = lq * 4 + r;
+      if constexpr (EPI == GEPI_SWIGLU) {
+        const float g = rn16(tot[0][r]), u = rn16(tot[NMAT - 1][r]);
+        if (m < a.M) a.y[(size_t)m * a.N + n] = (_Float16)(silu_act<_Float16>(g) * u);
+      } else if constexpr (EPI == GEPI_STORE) {
+        if (m < a.M) {
+          float v = rn16(tot[0][r]);
+          if (a.residual) v = (float)a.residual[(size_t)m * a.N + n] + v;
+          a.y[(size_t)m * a.N + n] = (_Float16)v;
+        }
+      } else {
+        const int which = n < a.n0 ? 0 : (n < a.n0 + a.n1 ? 1 : 2);
+        const int nl = which == 0 ? n : (which == 1 ? n - a.n0 : n - a.n0 - a.n1);
+        const int pair = (nl % a.head_dim) >> 1;
+        const bool odd = nl & 1;
+        const float own = rn16(tot[0][r]);
+        const float other = dpp_f<0xB1>(own);                // the neighbouring column: the other half of the pair
+        if (m < a.M) {
+          const int b = m / a.seq_len, pos = a.start_pos + m % a.seq_len;
+          float v = own;
+          if (which < 2) {
+            const h2_t cs = *(const h2_t *)(a.rope_table + ((size_t)pos * (a.head_dim / 2) + pair) * 2);
+            const float cc = (float)cs.x, dd = (float)cs.y;
+            v = odd ? other * dd + own * cc : own * cc - other * dd;
+          }
+          if (which == 0) a.y[(size_t)m * a.n0 + nl] = (_Float16)v;
+          else {
+            _Float16 *cache = which == 1 ? a.cache_k : a.cache_v;
+            cache[((size_t)b * a.max_context + pos) * a.n1 + nl] = (_Float16)v;
+          }
+        }
+      }
+    }
+  };
+
+  f4_t acc[TPW];
+#pragma unroll
+  for (int tt = 0; tt < TPW; tt++) acc[tt] = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int j = 0; j < NS; j++)
+    if (j < GS) issue(j, ring[j], rscale[j]);
+  sk_barrier();                                               // x chunk 0 is in LDS
+
+  for (int gs0 = 0; gs0 < GS; gs0 += NS) {
+#pragma unroll
+    for (int j = 0; j < NS; j++) {
+      const int gs = gs0 + j;
+      if (gs < GS) {                                          // the same for every thread of the block
+        const int cs = gs / TPW, tt = gs % TPW, c = cs % nck;
+        // ---- the step's tile: registers -> LDS patch (the reads of the step before were waited for), then the slot is free
+        const h2_t sc = rscale[j];
+#pragma unroll
+        for (int i = 0; i < 8; i++) *(u4_t *)(stg + wr_off + i * 2 * SG_WLS) = ring[j][i];
+        __builtin_amdgcn_sched_barrier(0);
+        if (gs + NS < GS) issue(gs + NS, ring[j], rscale[j]);
+        __builtin_amdgcn_sched_barrier(0);
+        const _Float16 *xs = xl + (cs % SG_XB) * 16 * SG_XLS + xoff;
+        f4_t r = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int f = 0; f < SG_KC / 32; f++) {
+          const h8_t af = *(const h8_t *)&xs[f * 32];
+          const uint2 raw = *(const uint2 *)(stg + rd_off + f * 32);
+          u4_t o;
+          uint32_t lo, hi;
+          i8x4_to_h2x2(raw.x, lo, hi); o.x = pk_mul_h2(lo, sc); o.y = pk_mul_h2(hi, sc);
+          i8x4_to_h2x2(raw.y, lo, hi); o.z = pk_mul_h2(lo, sc); o.w = pk_mul_h2(hi, sc);
+          r = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, __builtin_bit_cast(h8_t, o), r, 0, 0, 0);
+        }
+#pragma unroll
+        for (int t2 = 0; t2 < TPW; t2++)
+          if (t2 == tt) acc[t2] += r;
+        if (tt == TPW - 1) {
+          if (c == nck - 1) {
+            // ---- the unit is done
+            const int unit = blockIdx.x + (cs / nck) * gridDim.x;
+            const int grp = unit / sa.splitk;
+            bool mine = true;
+            if (sa.splitk > 1) {
+              // Partial sums travel between compute units (other XCDs have their own L2): stores and loads that go to the
+              // point all of them share, and the count goes up once this wavefront's stores are acknowledged.  No fences: a
+              // fence at that scope empties the caches the other blocks are streaming x through.
+              uint64_t *part = (uint64_t *)(sa.ws + ((size_t)unit * 4 + wave) * TPW * 256) + lane * 2;
+#pragma unroll
+              for (int t2 = 0; t2 < TPW; t2++) {
+                const uint64_t lo = ((uint64_t)__float_as_uint(acc[t2][1]) << 32) | __float_as_uint(acc[t2][0]);
+                const uint64_t hi = ((uint64_t)__float_as_uint(acc[t2][3]) << 32) | __float_as_uint(acc[t2][2]);
+                __hip_atomic_store(as_global_mut<uint64_t>(part + t2 * 128), lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(as_global_mut<uint64_t>(part + t2 * 128 + 1), hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              }
+              asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+              int old = 0;
+              if (lane == 0) old = __hip_atomic_fetch_add(&sa.counters[grp * 4 + wave], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              old = __builtin_amdgcn_readfirstlane(old);
+              mine = old == sa.splitk - 1;
+              if (mine) {
+#pragma unroll
+                for (int t2 = 0; t2 < TPW; t2++) acc[t2] = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                for (int p = 0; p < sa.splitk; p++) {
+                  const uint64_t *src = (const uint64_t *)(sa.ws + ((size_t)(grp * sa.splitk + p) * 4 + wave) * TPW * 256) + lane * 2;
+#pragma unroll
+                  for (int t2 = 0; t2 < TPW; t2++) {
+                    const uint64_t lo = __hip_atomic_load(as_global<uint64_t>(src + t2 * 128), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    const uint64_t hi = __hip_atomic_load(as_global<uint64_t>(src + t2 * 128 + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    acc[t2][0] += __uint_as_float((uint32_t)lo); acc[t2][1] += __uint_as_float((uint32_t)(lo >> 32));
+                    acc[t2][2] += __uint_as_float((uint32_t)hi); acc[t2][3] += __uint_as_float((uint32_t)(hi >> 32));
+                  }
+                }
+                if (lane == 0) __hip_atomic_store(&sa.counters[grp * 4 + wave], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+              }
+            }
+            if (mine) {
+#pragma unroll
+              for (int ct = 0; ct < S::CT; ct++) {
+                f4_t tot[NMAT];
+#pragma unroll
+                for (int q = 0; q < NMAT; q++) tot[q] = acc[ct * NMAT + q];
+                epilogue(tot, grp * S::COLS + (wave * S::CT + ct) * 16);
+              }
+            }
+#pragma unroll
+            for (int t2 = 0; t2 < TPW; t2++) acc[t2] = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
+          }
+          sk_barrier();                                       // chunk cs is consumed, chunk cs + 1 is in its buffer
+        }
+      }
+    }
+  }
+}
+
 // ---- host side ---------------------------------------------------------------------------------------------------
 
 template <int KIND, int EPI, int MB, int RTW> static int launch_skinny(const GemmArgs &a, int prof_kind) {
@@ -677,6 +941,66 @@ template <int KIND, int EPI, int MB, int RTW> static int launch_skinny(const Gem
   JSG_LAUNCH(prof_kind, (skinny_gemm_kernel<KIND, EPI, MB, RTW>), dim3(a.N / S::BR), dim3(SK_THREADS), lds, a);
   return 0;
 }
+// The LDS-streamed kernel: how many K parts.  Every block should get the same number of units; more parts than needed
+// only add partial sums.
+template <int EPI, int TPW> static int launch_stream(const GemmArgs &a, int prof_kind, bool *taken) {
+  typedef SgShape<EPI, TPW> S;
+  *taken = false;
+  if (a.M > 16 || a.K % SG_KC || a.N % S::COLS) return 0;
+  const int groups = a.N / S::COLS, nchunks = a.K / SG_KC, cus = state().cu_count;
+  if (groups > SG_MAX_GROUPS) return 0;
+  int best = 0;
+  double best_score = 0.0;
+  const char *pin = getenv("JSG_SG_SPLITK");
+  for (int d = 1; d <= nchunks && d <= 16; d++) {
+    if (nchunks % d) continue;
+    const int units = groups * d;
+    if ((size_t)units * 4 * TPW * 1024 > SG_WS_BYTES) continue;
+    if (pin && atoi(pin) != d) continue;
+    const int slots = cus;                                 // one block per compute unit (LDS)
+    const int rounds = (units + slots - 1) / slots;
+    // busy share of the chip, less what the parts cost (their sums travel through memory, and the last one waits for them:
+    // on the 8B shapes 2 parts for wq|wk|wv, 4 for wo and w2 and none for w1|w3 measured best)
+    const double score = (double)units / ((double)rounds * slots) - (d > 1 ? 0.05 * d : 0.0);
+    if (score > best_score + 1e-9) { best_score = score; best = d; }
+  }
+  if (!best) return 0;
+  static float *ws = nullptr;
+  static int *counters = nullptr;
+  if (!ws) {
+    JSG_HIP(hipGetSymbolAddress((void **)&ws, HIP_SYMBOL(sg_scratch)));
+    JSG_HIP(hipGetSymbolAddress((void **)&counters, HIP_SYMBOL(sg_counters)));
+    JSG_HIP(hipFuncSetAttribute((const void *)stream_gemm_kernel<GEPI_STORE, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SG_LDS));
+    JSG_HIP(hipFuncSetAttribute((const void *)stream_gemm_kernel<GEPI_STORE, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SG_LDS));
+    JSG_HIP(hipFuncSetAttribute((const void *)stream_gemm_kernel<GEPI_ROPE_KV, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SG_LDS));
+    JSG_HIP(hipFuncSetAttribute((const void *)stream_gemm_kernel<GEPI_ROPE_KV, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SG_LDS));
+    JSG_HIP(hipFuncSetAttribute((const void *)stream_gemm_kernel<GEPI_SWIGLU, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SG_LDS));
+  }
+  SgArgs sa;
+  sa.g = a;
+  sa.groups = groups; sa.splitk = best; sa.nck = nchunks / best;
+  sa.ws = ws; sa.counters = counters;
+  const int units = groups * best;
+  *taken = true;
+  JSG_LAUNCH(prof_kind, (stream_gemm_kernel<EPI, TPW>), dim3(units < cus ? units : cus), dim3(SG_THREADS), SG_LDS, sa);
+  return 0;
+}
+// int8 weights and at most 16 rows: the LDS-streamed kernel.  One tile per wavefront and x chunk (64 columns per unit)
+// measured faster than two on every shape of the 8B model (lm_head 97 us against 105), although x is read twice as often.
+template <int EPI> static int dispatch_stream(const GemmArgs &a, int prof_kind, bool *taken) {
+  *taken = false;
+  if (getenv("JSG_GEMM_NO_STREAM")) return 0;
+  if constexpr (EPI == GEPI_SWIGLU) return launch_stream<EPI, 2>(a, prof_kind, taken);
+  else {
+    const char *pin = getenv("JSG_SG_TPW");                  // "1" or "2": tests run both
+    if (!(pin && pin[0] == '2')) {
+      const int rc = launch_stream<EPI, 1>(a, prof_kind, taken);
+      if (*taken || rc) return rc;
+    }
+    return launch_stream<EPI, 2>(a, prof_kind, taken);
+  }
+}
+
 // Few rows: the weight-streaming kernel when K is whole chunks.  Every block reads all of x; with two tiles of 16 weight
 // rows per block that is half as often.  Measured on the lm_head (8016 tiles) the two-tile shape is no faster and moves
 // more HBM bytes (1.5x the weights against 1.24x), so it is only taken when pinned.
@@ -723,6 +1047,7 @@ template <int EPI> static int dispatch_gemm(int kind, const GemmArgs &a, int pro
   const bool small = tall && (pin ? !strcmp(pin, "small") : (!piped && blocks_of(256, 128) < cus));
   bool taken = false;
   if (kind == JSGRAD_W_F16) { const int rc = dispatch_skinny<JSGRAD_W_F16, EPI>(a, prof_kind, &taken); if (taken) return rc; }
+  if (kind == JSGRAD_W_I8) { const int rc = dispatch_stream<EPI>(a, prof_kind, &taken); if (taken || rc) return rc; }
   if (kind == JSGRAD_W_I8) { const int rc = dispatch_skinny<JSGRAD_W_I8, EPI>(a, prof_kind, &taken); if (taken) return rc; }
 #define JSG_CASE(K)                                                                                                    \
   case K:                                                                                                              \

@@ -105,6 +105,7 @@ def test_few_rows_streaming_kernel_equals_tiled_kernel(hip, monkeypatch):
     """The several-row kernels compute the same products; their float sums differ in order only.  The weight-streaming
     kernel with one and with two tiles of 16 weight rows per block against the tiled kernel."""
     out_f, in_f = 256, 4096
+    monkeypatch.setenv("JSG_GEMM_NO_STREAM", "1")      # int8 with at most 16 rows would go to the LDS-streamed kernel
     for kind in ("float16", "int8"):
         for rows in (16, 29):
             w, s = make_weight(kind, out_f, in_f)
@@ -159,10 +160,62 @@ def test_tile_shapes_fused_epilogues(hip, monkeypatch, shape):
     test_gemm_qkv_rope_writes_queries_and_cache(hip, "int8", 128, 2, 50, 192)
 
 
+@pytest.mark.parametrize("tpw", ["1", "2"])
+@pytest.mark.parametrize("rows", [16, 5])
+def test_lds_streamed_kernel_against_oracle_and_the_tiled_kernel(hip, monkeypatch, tpw, rows):
+    """int8 weights, at most 16 rows: whole stretches of weight rows through LDS, K split over blocks for narrow outputs.
+    Every admissible number of K parts gives a valid result; a given number gives the same bits on every run (the parts
+    are added in K order by whoever arrives last)."""
+    monkeypatch.setenv("JSG_SG_TPW", tpw)
+    for out_f, in_f in ((256, 4096), (1024, 1536), (128, 14336)):
+        w, s = make_weight("int8", out_f, in_f)
+        x = RNG.standard_normal((rows, in_f)).astype(np.float16)
+        res = RNG.standard_normal((rows, out_f)).astype(np.float16)
+        tw, ts = dev(w, s)
+        tx, tr = Tensor(x), Tensor(res)
+        lin = orc.linear(w, s, x, out_f, in_f, True)
+        ref = (res.astype(np.float32) + lin).astype(np.float16).astype(np.float32)
+        monkeypatch.setenv("JSG_GEMM_NO_SKINNY", "1")
+        monkeypatch.setenv("JSG_GEMM_NO_STREAM", "1")
+        y = Tensor.empty((rows, out_f), "float16")
+        check(hip.jsgrad_hip_gemm(ffi.W_I8, tw.ptr, sp(ts), out_f, in_f, tx.ptr, rows, y.ptr, tr.ptr))
+        tiled = y.numpy().astype(np.float32)
+        monkeypatch.delenv("JSG_GEMM_NO_SKINNY")
+        monkeypatch.delenv("JSG_GEMM_NO_STREAM")
+        nchunks = in_f // 512
+        for parts in ["", "1", "2", "3", "4", "7", "8"]:
+            if parts and (nchunks % int(parts) or (nchunks // int(parts)) * int(tpw) < 2):
+                continue
+            monkeypatch.setenv("JSG_SG_SPLITK", parts) if parts else monkeypatch.delenv("JSG_SG_SPLITK", raising=False)
+            runs = []
+            for _ in range(2):
+                y = Tensor.full((rows, out_f), 7.0, "float16")
+                check(hip.jsgrad_hip_gemm(ffi.W_I8, tw.ptr, sp(ts), out_f, in_f, tx.ptr, rows, y.ptr, tr.ptr))
+                runs.append(y.numpy())
+            assert np.array_equal(runs[0].view(np.uint16), runs[1].view(np.uint16)), (out_f, in_f, parts)
+            got = runs[0].astype(np.float32)
+            assert_close(got, ref, True, f"{out_f}x{in_f} parts={parts or 'auto'}", ulp_at=lin)
+            assert (got == tiled).mean() > 0.97, (out_f, in_f, parts)
+        monkeypatch.delenv("JSG_SG_SPLITK", raising=False)
+
+
+@pytest.mark.parametrize("tpw", ["1", "2"])
+def test_lds_streamed_kernel_fused_epilogues(hip, monkeypatch, tpw):
+    """SwiGLU and rotary / cache epilogues of the LDS-streamed kernel, with and without K parts."""
+    monkeypatch.setenv("JSG_SG_TPW", tpw)
+    for parts in ("", "2"):
+        monkeypatch.setenv("JSG_SG_SPLITK", parts) if parts else monkeypatch.delenv("JSG_SG_SPLITK", raising=False)
+        test_gemm_ffn_gate(hip, "int8", 16, 2048, 256)
+        test_gemm_ffn_gate(hip, "int8", 3, 1024, 384)
+        test_gemm_qkv_rope_writes_queries_and_cache(hip, "int8", 128, 16, 1, 2048)
+        test_gemm_qkv_rope_writes_queries_and_cache(hip, "int8", 128, 3, 2, 1024)
+
+
 @pytest.mark.parametrize("tiles", ["1", "2"])
 def test_few_rows_fused_epilogues_with_one_and_two_tiles_per_block(hip, monkeypatch, tiles):
     """SwiGLU and rotary / cache epilogues of the weight-streaming kernel, tiles per block pinned."""
     monkeypatch.setenv("JSG_GEMM_SKINNY_TILES", tiles)
+    monkeypatch.setenv("JSG_GEMM_NO_STREAM", "1")
     test_gemm_ffn_gate(hip, "int8", 16, 2048, 256)
     test_gemm_ffn_gate(hip, "float16", 20, 1024, 128)
     test_gemm_qkv_rope_writes_queries_and_cache(hip, "int8", 128, 16, 1, 2048)
