@@ -43,15 +43,16 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct AttnStrea
     const AT *kbase = (const AT *)a.cache_k + (size_t)g * HD + (size_t)sub * EPL;
     const AT *vbase = (const AT *)a.cache_v + (size_t)g * HD + (size_t)sub * EPL;
 
-    // this lane's slice of the n_rep query rows
-    float qf[NREP][EPL];
+    // this lane's slice of the n_rep query rows (fp16: kept packed, two elements to a register, for the packed dot product)
+    constexpr int QW = sizeof(AT) == 2 ? 4 : EPL;
+    uint32_t qv[NREP][QW];
 #pragma unroll
     for (int j = 0; j < NREP; j++) {
       const AT *qp = (const AT *)a.q + (size_t)(g * NREP + j) * HD + sub * EPL;
 #pragma unroll
-      for (int e = 0; e < EPL; e++) {
-        if constexpr (COHERENT) qf[j][e] = (float)ld_coherent(qp + e);
-        else qf[j][e] = (float)qp[e];
+      for (int e = 0; e < QW; e++) {
+        if constexpr (COHERENT) qv[j][e] = __hip_atomic_load(as_global<uint32_t>(qp) + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else qv[j][e] = ((const uint32_t *)qp)[e];
       }
     }
 
@@ -69,19 +70,16 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct AttnStrea
 
     // ---- phase 1: scores of the chunk
     auto score_row = [&](u4_t raw, int t) {
-      float kf[EPL];
-      if constexpr (sizeof(AT) == 2) {
-#pragma unroll
-        for (int e = 0; e < 4; e++) { h2_t h = as_h2(raw[e]); kf[2 * e] = (float)h[0]; kf[2 * e + 1] = (float)h[1]; }
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; e++) kf[e] = __uint_as_float(raw[e]);
-      }
 #pragma unroll
       for (int j = 0; j < NREP; j++) {
         float p = 0.0f;
+        if constexpr (sizeof(AT) == 2) {     // packed dot products with float accumulation (the products are exact in float)
 #pragma unroll
-        for (int e = 0; e < EPL; e++) p = fmaf(qf[j][e], kf[e], p);
+          for (int e = 0; e < 4; e++) p = __builtin_amdgcn_fdot2(as_h2(qv[j][e]), as_h2(raw[e]), p, false);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; e++) p = fmaf(__uint_as_float(qv[j][e]), __uint_as_float(raw[e]), p);
+        }
         p = group_sum<G>(p);
         if (sub == 0) sm.sc[j][t - t0] = p * a.scale;
       }
