@@ -34,7 +34,8 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel family from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised under
 # profiles/ (average over the launches of one step).  "linear" is w2 + lm_head when attention and wo share a launch
 # (the default for fp16 activations), else wo + w2 + lm_head.
-MEASURED_TRAFFIC = {("1B", "linear", True): 62.78e6, ("8B-int8", "linear", True): 73.45e6,
+MEASURED_TRAFFIC = {("1B", "linear", True): 62.77e6, ("8B-int8", "linear", True): 73.46e6,
+                    ("1B", "ffn_gate", True): 67.31e6, ("8B-int8", "ffn_gate", True): 118.22e6,
                     ("1B", "linear", False): 36.49e6, ("8B-int8", "linear", False): 45.72e6}
 
 
