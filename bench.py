@@ -442,6 +442,55 @@ def traffic_probe(name, batch=1):
         check(lib.jsgrad_hip_sync())
 
 
+def run_rows_gemm(workload="8B-int8", rows=16, only=""):
+    """The several-row Linear launches of one decode step of `rows` sequences, one shape at a time: wq|wk|wv (as one plain
+    matrix of their combined height), wo, w1|w3 + SwiGLU, w2, lm_head.  Weights are rotated over cold copies (more than the
+    256 MB of memory-side cache between two uses of a copy); time per launch from the event pair around each dispatch.
+    `only`: comma-separated subset of the shape names (e.g. "lm_head" for a counter run on one kernel)."""
+    from denograd_amd import ffi, synthetic
+    from denograd_amd.ffi import check
+    from denograd_amd.tensor import Tensor
+    lib = ffi.load()
+    cfg = synthetic.CONFIGS[workload]
+    if cfg["quantize"] != "int8":
+        raise SystemExit("--rows-gemm-only is written for int8 workloads")
+    dim, hidden, vocab = cfg["dim"], cfg["hidden_dim"], cfg["vocab_size"]
+    hd = dim // cfg["n_heads"]
+    shapes = {"qkv": (dim + 2 * cfg["n_kv_heads"] * hd, dim), "wo": (dim, dim), "w1w3": (hidden, dim), "w2": (dim, hidden), "lm_head": (vocab, dim)}
+    out = {}
+    for name, (o, i) in shapes.items():
+        if only and name not in only.split(","):
+            continue
+        nb = o * i * (2 if name == "w1w3" else 1)
+        ncopy = max(3, min(10, (2 << 30) // nb))
+        def make():
+            w = Tensor.empty((o, i), "int8")
+            check(lib.jsgrad_hip_memset(w.ptr, 3, o * i))
+            return w
+        ws = [(make(), make() if name == "w1w3" else None) for _ in range(ncopy)]
+        sc, x = Tensor.ones((o,), "float16"), Tensor.randn((rows, i), "float16", 2, 1.0)
+        y, res = Tensor.empty((rows, o), "float16"), Tensor.randn((rows, o), "float16", 3, 1.0)
+        def launch(k):
+            a, b = ws[k % ncopy]
+            if b is not None:
+                check(lib.jsgrad_hip_gemm_ffn_gate(ffi.W_I8, a.ptr, sc.ptr, b.ptr, sc.ptr, x.ptr, rows, y.ptr, i, o))
+            else:
+                check(lib.jsgrad_hip_gemm(ffi.W_I8, a.ptr, sc.ptr, o, i, x.ptr, rows, y.ptr, res.ptr if name in ("wo", "w2") else None))
+        for k in range(ncopy):
+            launch(k)
+        check(lib.jsgrad_hip_profile(1))
+        for k in range(3 * ncopy):
+            launch(k)
+        n, tot = C.c_int(), C.c_double()
+        check(lib.jsgrad_hip_profile_read(ffi.PROF_KINDS["gemm"], C.byref(n), C.byref(tot)))
+        check(lib.jsgrad_hip_profile(0))
+        us = 1e3 * tot.value / n.value
+        out[name] = {"out_features": o * (2 if name == "w1w3" else 1), "in_features": i, "bytes": nb, "us": round(us, 2), "GBps": round(nb / us / 1e3, 1),
+                     "frac_of_hbm_peak": round(nb / us / 1e3 / HBM_PEAK_GBS, 4)}
+        del ws
+    return {"workload": workload, "rows": rows, "shapes": out}
+
+
 def run_formats(reps=5):
     """Load-time kernels of the checkpoint path, each on one lm_head-sized tensor (128256 x 2048 elements): GGML Q6_K ->
     float32, bfloat16 -> float16, and the q_proj row permutation.  HBM-bound byte work: bytes read + written per second."""
@@ -503,6 +552,9 @@ def main():
     ap.add_argument("--fused-step", action="store_true", help="run each token as one persistent kernel (jsgrad_hip_decode_step) instead of one launch per fused op")
     ap.add_argument("--stream-step", action="store_true", help="run each token as one persistent kernel with streaming wavefronts (jsgrad_hip_stream_step)")
     ap.add_argument("--formats-only", action="store_true", help="only the load-time kernels of the checkpoint path (GGML dequantisation, casts, row permutation); prints their JSON")
+    ap.add_argument("--rows-gemm-only", action="store_true", help="only the several-row Linear launches of a batched decode step (--batched workload, --batch rows), "
+                    "one shape at a time over cold weights; prints their JSON")
+    ap.add_argument("--rows-gemm-shapes", default="", help="with --rows-gemm-only: comma-separated subset of qkv,wo,w1w3,w2,lm_head")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel eagerly instead of replaying a captured HIP graph "
                     "(rocprofv3 --kernel-trace on this image crashes inside hipGraphLaunch, so profiles are taken this way)")
     args = ap.parse_args()
@@ -520,6 +572,9 @@ def main():
         return
     if args.formats_only:
         print(json.dumps({"formats": run_formats()}), flush=True)
+        return
+    if args.rows_gemm_only:
+        print(json.dumps({"rows_gemm": run_rows_gemm(args.batched or "8B-int8", args.batch, args.rows_gemm_shapes)}), flush=True)
         return
     step_mode = "stream" if args.stream_step else args.fused_step
     llm, cfg, res = run_workload(args.workload, args.prompt, args.steps, args.warmup, use_graph=not args.no_graph, fused_step=step_mode)
