@@ -93,8 +93,9 @@ static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
 constexpr int NOALLOC_MAX_DEVICES = 64;
 static void *g_scratch_ptr[NOALLOC_MAX_DEVICES];   // per device, set on the first call there
 
-// the chunk counters must start at zero whatever an earlier call left behind (a fill kernel, not a memset node: callers may
-// be capturing a graph)
+// the part of the workspace a call uses must start at zero (a zero word means `partial result not written yet`) whatever an
+// earlier call left behind, one that gave up waiting included (a fill kernel, not a memset node: callers may be capturing a
+// graph)
 __global__ void zero_words_kernel(int *p, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = 0;
@@ -147,7 +148,8 @@ int jsgrad_hip_attn_decode_static(const void *q, const void *cache_k, const void
   JSG_REQUIRE(q && cache_k && cache_v && st && out, "jsgrad_hip_attn_decode_static: null pointer argument");
   JSG_REQUIRE(n_heads > 0 && n_kv_heads > 0 && max_context > 0, "jsgrad_hip_attn_decode_static: n_heads %d / n_kv_heads %d / max_context %d", n_heads, n_kv_heads, max_context);
   JSG_REQUIRE(max_context <= 256 * ATT_CHUNK_MAX, "jsgrad_hip_attn_decode_static: max_context %d exceeds %d", max_context, 256 * ATT_CHUNK_MAX);
-  // counters [0, 256), then one partial result per (head, chunk): only the chunks this max_context can produce are needed
+  // 256 bytes of counters (used by the kernels that run many layers in one launch, not here), then one partial result per
+  // (head, chunk): only the chunks this max_context can produce are needed
   const size_t need = 256 + (size_t)n_heads * att_max_chunks(max_context) * ((size_t)head_dim + 2) * sizeof(float);
   JSG_REQUIRE(need <= NOALLOC_SCRATCH_BYTES,
               "jsgrad_hip_attn_decode_static: %d heads of %d at max_context %d need %zu bytes of workspace, the built-in one holds %zu; use jsgrad_hip_attn_decode "
@@ -161,7 +163,8 @@ int jsgrad_hip_attn_decode_static(const void *q, const void *cache_k, const void
     g_scratch_ptr[dev] = p;
   }
   void *ws = g_scratch_ptr[dev];
-  hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, state().stream, (int *)ws, 64);
+  const int words = (int)((need + 3) / 4);
+  hipLaunchKernelGGL(zero_words_kernel, dim3((words + 255) / 256), dim3(256), 0, state().stream, (int *)ws, words);
   JSG_LAUNCHED();
   return jsgrad_hip_attn_decode(q, cache_k, cache_v, st, out, ws, n_heads, n_kv_heads, head_dim, max_context, act);
 }

@@ -17,6 +17,13 @@ namespace jsg {
 
 constexpr int ATT_CHUNK_MAX = 256;  // positions per item held in LDS; also the most chunks the merge can index
 
+// A partial result as a workspace word that says by itself whether it has been written: the complement of the float's bits,
+// so that zero means `not yet`.  Only the NaN with all bits set would come out as zero; it is stored as another NaN.
+__device__ __forceinline__ uint32_t att_word(float v) {
+  const uint32_t b = __float_as_uint(v);
+  return ~(b == 0xFFFFFFFFu ? 0x7FC00000u : b);
+}
+
 // Rows per chunk for T visible positions.  A launch is a chain of round trips (rows, partial results, merge), and the merge
 // fetches one partial result per chunk, so chunks are few and long rather than many and short: 64 rows up to 512 positions,
 // 128 up to 2048, 256 beyond (at most 8 / 16 / T/256 chunks per kv head).
@@ -252,48 +259,75 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
     }
     lds_barrier();
     constexpr int SLOTS = NW;
+    // ---- hand-over of the chunk's partial result.
+    // WORDS (kernels whose launch is the whole life of the workspace contents, COHERENT false): every 32-bit word says by
+    // itself whether it has been written.  The workspace holds zeros; a value is stored as the complement of its bits
+    // (att_word), so no block waits for its stores or counts itself in: the block of chunk 0 asks for the words of all chunks
+    // until none is zero, and puts the zeros back for the next launch.  The chain store - acknowledge - count - see the count
+    // - fetch becomes store - fetch.
+    // Otherwise (kernels that run many layers in one launch, where a cleared word could meet the next layer's store) the
+    // blocks count themselves in after their stores were acknowledged, and the block of chunk 0 waits for the count.
+    constexpr bool WORDS = !COHERENT;
+    auto enc = [](float v) { return WORDS ? __uint_as_float(att_word(v)) : v; };
+    auto dec = [](uint32_t w) { return __uint_as_float(WORDS ? ~w : w); };
     float *mine = a.partial + ((size_t)g * a.nsplit + split) * NREP * (HD + 2);
     for (int i = tid; i < NREP * HD; i += nthreads) {
       const int j = i / HD, d = i % HD;
       float v = 0.0f;
 #pragma unroll
       for (int w = 0; w < SLOTS; w++) v += sm.o_part[w][j][d];
-      st_coherent(&mine[j * (HD + 2) + d], v);
+      st_coherent(&mine[j * (HD + 2) + d], enc(v));
     }
     if (tid < NREP) {
-      st_coherent(&mine[tid * (HD + 2) + HD], sm.m_sh[tid]);
-      st_coherent(&mine[tid * (HD + 2) + HD + 1], sm.l_sh[tid]);
+      st_coherent(&mine[tid * (HD + 2) + HD], enc(sm.m_sh[tid]));
+      st_coherent(&mine[tid * (HD + 2) + HD + 1], enc(sm.l_sh[tid]));
     }
-
-    // ---- publish.  The block of chunk 0 merges the chunks of its kv head; the others count themselves in and are done.
-    __syncthreads();  // every coherent store of the block has been acknowledged
-    if (split != 0) {
-      if (tid == 0) __hip_atomic_fetch_add(&a.counters[g], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // nobody waits for the answer
-      then();
-      return;
-    }
-    if (n_active > 1) {
-      if (tid == 0) {
-        // The other chunks' blocks never wait for anything before they count themselves in, and the launch keeps them all on the
-        // device, so this wait ends; it is bounded all the same and reports through the error word where one is given.
-        int it = 0;
-        while (ld_coherent(&a.counters[g]) != n_active - 1) {
-          if (++it > (1 << 20)) { if (a.err != nullptr) st_coherent(a.err, 1); break; }
-          __builtin_amdgcn_s_sleep(2);
-        }
-        __hip_atomic_store(&a.counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // zero again for the next launch
+    if constexpr (WORDS) {
+      if (split != 0) {
+        then();
+        return;
       }
-      __syncthreads();
+      lds_barrier();   // m_sh / l_sh / sc are written again below
+    } else {
+      __syncthreads();  // every coherent store of the block has been acknowledged
+      if (split != 0) {
+        if (tid == 0) __hip_atomic_fetch_add(&a.counters[g], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // nobody waits for the answer
+        then();
+        return;
+      }
+      if (n_active > 1) {
+        if (tid == 0) {
+          // The other chunks' blocks never wait for anything before they count themselves in, and the launch keeps them all on the
+          // device, so this wait ends; it is bounded all the same and reports through the error word where one is given.
+          int it = 0;
+          while (ld_coherent(&a.counters[g]) != n_active - 1) {
+            if (++it > (1 << 20)) { if (a.err != nullptr) st_coherent(a.err, 1); break; }
+            __builtin_amdgcn_s_sleep(2);
+          }
+          __hip_atomic_store(&a.counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // zero again for the next launch
+        }
+        __syncthreads();
+      }
     }
     // merge.  Every thread owns two neighbouring output elements and requests their partial sums of the first MB chunks
     // right away; while those travel, one wavefront per query head fetches the per-chunk (m, l), turns them into weights
     // exp(m_s - M) and 1/L in LDS; then the sums are folded in chunk order.  One round trip for up to MB chunks.
+    // WORDS: a request is repeated while one of its words is still zero.  The other chunks' blocks never wait for anything
+    // before they store, and the launch keeps them all on the device, so this ends; it is bounded all the same, reports
+    // through the error word where one is given, and the result is then NaN.
     const float *base = a.partial + (size_t)g * a.nsplit * NREP * (HD + 2);
     constexpr int MB = 16;                       // chunks per batch of requests
     constexpr int NPAIR = NREP * HD / 2;         // element pairs of this kv head's query heads
+    constexpr int POLL_LIMIT = 1 << 18;
+    auto pair_at = [&](const float *po, int s_) { return po + (size_t)(s_ < n_active ? s_ : n_active - 1) * NREP * (HD + 2); };
     auto ld_pair = [&](const float *po, int s_) -> uint64_t {   // two floats of chunk s_ (8-byte aligned: HD + 2 is even)
-      return __hip_atomic_load(as_global<uint64_t>(po + (size_t)(s_ < n_active ? s_ : n_active - 1) * NREP * (HD + 2)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return __hip_atomic_load(as_global<uint64_t>(pair_at(po, s_)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     };
+    auto clear_pair = [&](const float *po, int s_) {
+      __hip_atomic_store(as_global_mut<uint64_t>(const_cast<float *>(pair_at(po, s_))), 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    };
+    auto written = [](uint64_t w) { return (uint32_t)w != 0u && (uint32_t)(w >> 32) != 0u; };
+    auto gave_up = [&]() { if (a.err != nullptr) st_coherent(a.err, 1); };
     const int p0 = tid < NPAIR ? tid : 0;        // threads beyond the pairs request pair 0 again (their result is not stored)
     const int j0 = (2 * p0) / HD, d0 = (2 * p0) % HD;
     const float *po0 = base + (size_t)j0 * (HD + 2) + d0;
@@ -308,27 +342,47 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
 #pragma unroll
     for (int u = 0; u < MB; u++) part[u] = ld_pair(po0, u);
     for (int j = wave; j < NREP; j += NW) {
-      if (j != wave) {     // more query heads than wavefronts: the further heads of this wavefront, one round trip each
+      const float *pml = base + (size_t)j * (HD + 2) + HD;
+      bool lost = false;
+      // the first head of this wavefront was requested above; further heads (more query heads than wavefronts) and repeated
+      // requests cost a round trip each
+      for (int it = 0;; it++) {
+        if (j != wave || it > 0) {
+#pragma unroll
+          for (int i = 0; i < MSL; i++)
+            if (i * 64 < n_active) mls[i] = ld_pair(pml, lane + i * 64);
+        }
+        if constexpr (!WORDS) break;
+        bool ok = true;
 #pragma unroll
         for (int i = 0; i < MSL; i++)
-          if (i * 64 < n_active) mls[i] = ld_pair(base + (size_t)j * (HD + 2) + HD, lane + i * 64);
+          if (lane + i * 64 < n_active && !written(mls[i])) ok = false;
+        if (ok) break;
+        if (it >= POLL_LIMIT) { lost = true; gave_up(); break; }
+        __builtin_amdgcn_s_sleep(1);
+      }
+      if constexpr (WORDS) {
+#pragma unroll
+        for (int i = 0; i < MSL; i++)
+          if (lane + i * 64 < n_active) clear_pair(pml, lane + i * 64);
       }
       float M = -INFINITY;
 #pragma unroll
       for (int i = 0; i < MSL; i++)
-        if (lane + i * 64 < n_active) M = fmaxf(M, __uint_as_float((uint32_t)mls[i]));
+        if (lane + i * 64 < n_active) M = fmaxf(M, dec((uint32_t)mls[i]));
       M = wave_max(M);
       float L = 0.0f;
 #pragma unroll
       for (int i = 0; i < MSL; i++) {
         const int s_ = lane + i * 64;
         if (s_ < n_active) {
-          const float w = exp_f32(__uint_as_float((uint32_t)mls[i]) - M);
+          const float w = exp_f32(dec((uint32_t)mls[i]) - M);
           sm.sc[j][s_] = w;  // n_active <= nsplit <= CHUNK_CAP
-          L = fmaf(__uint_as_float((uint32_t)(mls[i] >> 32)), w, L);
+          L = fmaf(dec((uint32_t)(mls[i] >> 32)), w, L);
         }
       }
       L = wave_sum(L);
+      if (__builtin_amdgcn_ballot_w64(lost) != 0) L = __builtin_nanf("");
       if (lane == 0) sm.l_sh[j] = 1.0f / L;  // softmax normalisation is e * (1/sum) (tensor.ts:2211-2214)
     }
     lds_barrier();
@@ -345,16 +399,31 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       const float *po = base + (size_t)j * (HD + 2) + d;
       float Oa = 0.0f, Ob = 0.0f;
       for (int s0 = 0; s0 < n_active; s0 += MB) {
-        if (s0 > 0 || p != tid) {                 // the first batch of the first pair is already here
+        for (int it = 0;; it++) {
+          if (s0 > 0 || p != tid || it > 0) {     // the first batch of the first pair is already here
 #pragma unroll
-          for (int u = 0; u < MB; u++) part[u] = ld_pair(po, s0 + u);
+            for (int u = 0; u < MB; u++) part[u] = ld_pair(po, s0 + u);
+          }
+          if constexpr (!WORDS) break;
+          bool ok = true;
+#pragma unroll
+          for (int u = 0; u < MB; u++)
+            if (s0 + u < n_active && !written(part[u])) ok = false;
+          if (ok) break;
+          if (it >= POLL_LIMIT) { Oa = Ob = __builtin_nanf(""); gave_up(); break; }
+          __builtin_amdgcn_s_sleep(1);
+        }
+        if constexpr (WORDS) {
+#pragma unroll
+          for (int u = 0; u < MB; u++)
+            if (s0 + u < n_active) clear_pair(po, s0 + u);
         }
 #pragma unroll
         for (int u = 0; u < MB; u++)
           if (s0 + u < n_active) {
             const float w = sm.sc[j][s0 + u];
-            Oa = fmaf(__uint_as_float((uint32_t)part[u]), w, Oa);
-            Ob = fmaf(__uint_as_float((uint32_t)(part[u] >> 32)), w, Ob);
+            Oa = fmaf(dec((uint32_t)part[u]), w, Oa);
+            Ob = fmaf(dec((uint32_t)(part[u] >> 32)), w, Ob);
           }
       }
       finish(2 * p, Oa);

@@ -142,14 +142,15 @@ int jsgrad_hip_qkv_rope(int kind, const void *wq, const void *sq, const void *wk
 
 /* repeat_kv + scaled_dot_product_attention over cache rows [0, state[1]] (models/llama.ts:89-95,
  * tensor.ts:3920-3934), grouped-query: query head h reads kv head h / (n_heads/n_kv_heads).
- * workspace: jsgrad_hip_attn_workspace_bytes() bytes, zero-filled once before first use. */
+ * workspace: jsgrad_hip_attn_workspace_bytes() bytes, zero-filled once before first use: a zero word means `partial result not
+ * written yet`, and every launch leaves the workspace zero again. */
 size_t jsgrad_hip_attn_workspace_bytes(int n_heads, int n_kv_heads, int head_dim);
 int jsgrad_hip_attn_decode(const void *q, const void *cache_k, const void *cache_v, const int32_t *state, void *out, void *workspace,
                            int n_heads, int n_kv_heads, int head_dim, int max_context, int act);
 
 /* jsgrad_hip_attn_decode without the workspace argument, for callers that cannot allocate device memory (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The partial
- * results and chunk counters live in an array built into the library: jsgrad_hip_attn_decode_static_max_bytes() bytes
+ * results live in an array built into the library: jsgrad_hip_attn_decode_static_max_bytes() bytes
  * (8 MiB) on every GPU the library runs on, held until the process ends.  The call allocates and frees nothing; shapes whose
  * workspace (256 + n_heads * chunks(max_context) * (head_dim + 2) * 4 bytes, chunks <= 256) does not fit are refused with an
  * error.  All calls on one GPU share the array: they are ordered by the library's stream; calls that overlap on one GPU
