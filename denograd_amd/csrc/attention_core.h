@@ -24,13 +24,18 @@ __device__ __forceinline__ uint32_t att_word(float v) {
   return ~(b == 0xFFFFFFFFu ? 0x7FC00000u : b);
 }
 
-// Rows per chunk for T visible positions.  A launch is a chain of round trips (rows, partial results, merge), and the merge
-// fetches one partial result per chunk, so chunks are few and long rather than many and short: 64 rows up to 512 positions,
-// 128 up to 2048, 256 beyond (at most 8 / 16 / T/256 chunks per kv head).
+// Rows per chunk for T visible positions.  A launch is a chain of round trips (rows, partial results, merge); the rows of a
+// chunk are fetched by one block, and the merge fetches one partial result per chunk.  About ten chunks per kv head is
+// where the two meet (measured on the 8B shape: 584 positions in 10 chunks 14.0 us per attention + wo launch, in 5 chunks
+// 15.3, in 19 chunks 16.0; 1064 positions in 9 chunks 13.5 us, in 17 chunks 14.5; 8, 10, 12 and 16 as the target measure
+// alike): a tenth of T, in whole 16s, at least 64 rows; 128-row chunks at 4100 positions are slower than 256 (18.6 / 15.8 us).
 // `nsplit` chunks is what the workspace and the grid provide: the chunk grows if T would need more.
-// `cap`: the longest chunk the block shape can take (16 rows per wavefront, at most ATT_CHUNK_MAX).
+// `cap`: the longest chunk the block shape can take (16 rows per wavefront, at most ATT_CHUNK_MAX; never below 64).
+constexpr int ATT_TARGET_CHUNKS = 10, ATT_CHUNK_MIN = 64, ATT_CHUNK_POLICY_MAX = ATT_CHUNK_MAX;
 __host__ __device__ __forceinline__ int att_policy_rows(int T, int cap) {
-  const int c = T <= 512 ? 64 : (T <= 2048 ? 128 : 256);
+  int c = ((T + ATT_TARGET_CHUNKS - 1) / ATT_TARGET_CHUNKS + 15) & ~15;
+  c = c < ATT_CHUNK_MIN ? ATT_CHUNK_MIN : c;
+  c = c < ATT_CHUNK_POLICY_MAX ? c : ATT_CHUNK_POLICY_MAX;
   return c < cap ? c : cap;
 }
 __host__ __device__ __forceinline__ int att_chunk_rows(int T, int nsplit, int cap = ATT_CHUNK_MAX) {
@@ -38,13 +43,14 @@ __host__ __device__ __forceinline__ int att_chunk_rows(int T, int nsplit, int ca
   const int need = (T + nsplit - 1) / nsplit;
   return c < need ? need : c;
 }
-// chunks a launch must provide for every T up to max_context (the count is not monotonic in T across the policy's steps)
+// chunks a launch must provide for every T up to max_context: up to ATT_TARGET_CHUNKS * ATT_CHUNK_MIN positions the count
+// grows with T, then it stays at or below the target until the chunks reach their longest
 __host__ __device__ __forceinline__ int att_max_chunks(int max_context, int cap = ATT_CHUNK_MAX) {
-  auto n = [cap](int T) { const int c = att_policy_rows(T, cap); return (T + c - 1) / c; };
-  int m = n(max_context < 512 ? max_context : 512);
-  if (max_context > 512) { const int v = n(max_context < 2048 ? max_context : 2048); m = v > m ? v : m; }
-  if (max_context > 2048) { const int v = n(max_context); m = v > m ? v : m; }
-  return m;
+  const int longest = cap < ATT_CHUNK_POLICY_MAX ? cap : ATT_CHUNK_POLICY_MAX;
+  const int knee = ATT_TARGET_CHUNKS * ATT_CHUNK_MIN;
+  const int low = ((max_context < knee ? max_context : knee) + ATT_CHUNK_MIN - 1) / ATT_CHUNK_MIN;
+  const int high = (max_context + longest - 1) / longest;
+  return low > high ? low : high;
 }
 
 struct AttnArgs {

@@ -70,9 +70,17 @@ def test_attention_wo_launch_capacity_rule():
     against a given capacity here (on a GPU the library asks the occupancy calculator)."""
     from denograd_amd.llama import attn_wo_fits
     lib = ffi.load()
-    # chunks of the context: 64 rows up to 512 positions, 128 up to 2048, 256 beyond; the most any T <= max_context asks for
-    assert lib.jsgrad_hip_attn_wo_items(8, 841) == 8 * 8        # T = 512 -> 8 chunks of 64 (841 itself: 7 of 128)
-    assert lib.jsgrad_hip_attn_wo_items(8, 2304) == 8 * 16      # T = 2048 -> 16 chunks of 128
+    # chunks of the context: a tenth of T in whole 16s, at least 64 and at most 256 rows; the library provides the most
+    # chunks any T <= max_context asks for.  Checked against the rule itself, every T tried.
+    def rows(T):
+        return min(256, max(64, (-(-T // 10) + 15) // 16 * 16))
+    most, m = {}, 0
+    for T in range(1, 16385):
+        m = max(m, -(-T // rows(T)))
+        most[T] = m
+    for ctx in (1, 63, 64, 65, 512, 640, 641, 841, 952, 1400, 2304, 2560, 2561, 4340, 8192, 16384):
+        assert lib.jsgrad_hip_attn_wo_items(8, ctx) == 8 * most[ctx], ctx
+    assert lib.jsgrad_hip_attn_wo_items(8, 841) == 8 * 10       # 10 chunks of 64 at T = 640 (841 itself: 9 of 96)
     assert lib.jsgrad_hip_attn_wo_items(2, 64) == 2 * 1
     assert lib.jsgrad_hip_attn_wo_items(8, 16384) == 8 * 64     # 64 chunks of 256
     cap = 4 * 256      # four blocks of 256 threads per compute unit
