@@ -5,17 +5,22 @@
 
 namespace jsg {
 
-// One sequence (or few): blocks of 16 wavefronts, an item's rows requested up front (attention_core.h).
-constexpr int ATT_NW = 16;
-template <typename AT, int HD, int NREP>
-__global__ __launch_bounds__(ATT_NW * 64) void attn_decode_kernel(AttnArgs a) {
-  typedef Attn<AT, HD, NREP, ATT_NW, false> A;
+// One sequence (or few): an item's rows are requested up front by a block of NW wavefronts (attention_core.h), 16 rows per
+// wavefront at most.  Blocks of 8 wavefronts measured faster than 16 at every context tried (8B shape at 4100 positions:
+// 12.4 us against 15.8); their chunks hold 128 rows, and the merge can index 128 chunks, so contexts beyond 16384 positions
+// take the 16-wavefront shape (256-row chunks, 256 chunks).  jsgrad_hip_attn_wo runs the same item with 8 wavefronts, so
+// the two agree bit for bit wherever both apply.
+constexpr int ATT_NW = 8, ATT_NW_LONG = 16;
+constexpr int ATT_SHORT_CONTEXT = (ATT_NW * 16) * (ATT_NW * 16);
+template <typename AT, int HD, int NREP, int NW>
+__global__ __launch_bounds__(NW * 64) void attn_decode_kernel(AttnArgs a) {
+  typedef Attn<AT, HD, NREP, NW, false> A;
   __shared__ typename A::Smem sm;
   const int g = blockIdx.x, split = blockIdx.y;
   const int pos = a.st[1];
   if (pos < 0 || pos >= a.max_context) return;
   const int T = pos + 1;
-  const int chunk = att_chunk_rows(T, a.nsplit);  // <= ATT_CHUNK_MAX, checked on the host against max_context
+  const int chunk = att_chunk_rows(T, a.nsplit, A::CHUNK_CAP);  // the host sized nsplit for max_context and this cap
   const int n_active = (T + chunk - 1) / chunk;
   if (split >= n_active) return;
   A::item(a, sm, g, split, T, chunk, n_active);
@@ -57,11 +62,11 @@ static int stream_nsplit(int max_context, int heads_x_batch) {
   return by_lds > wanted ? by_lds : wanted;
 }
 
-template <typename AT, int HD> static int launch_attn(const AttnArgs &a, int n_rep) {
-  dim3 grid(a.n_kv_heads, a.nsplit, 1), block(ATT_NW * 64);
+template <typename AT, int HD, int NW> static int launch_attn(const AttnArgs &a, int n_rep) {
+  dim3 grid(a.n_kv_heads, a.nsplit, 1), block(NW * 64);
 #define JSG_REP(N)                                                                                   \
   case N:                                                                                            \
-    JSG_LAUNCH(PROF_ATTN, (attn_decode_kernel<AT, HD, N>), grid, block, 0, a);                         \
+    JSG_LAUNCH(PROF_ATTN, (attn_decode_kernel<AT, HD, N, NW>), grid, block, 0, a);                     \
     break;
   switch (n_rep) {
     JSG_REP(1) JSG_REP(2) JSG_REP(3) JSG_REP(4) JSG_REP(8)
@@ -150,7 +155,8 @@ int jsgrad_hip_attn_decode_static(const void *q, const void *cache_k, const void
   JSG_REQUIRE(max_context <= 256 * ATT_CHUNK_MAX, "jsgrad_hip_attn_decode_static: max_context %d exceeds %d", max_context, 256 * ATT_CHUNK_MAX);
   // 256 bytes of counters (used by the kernels that run many layers in one launch, not here), then one partial result per
   // (head, chunk): only the chunks this max_context can produce are needed
-  const size_t need = 256 + (size_t)n_heads * att_max_chunks(max_context) * ((size_t)head_dim + 2) * sizeof(float);
+  const int cap = max_context <= ATT_SHORT_CONTEXT ? ATT_NW * 16 : ATT_CHUNK_MAX;
+  const size_t need = 256 + (size_t)n_heads * att_max_chunks(max_context, cap) * ((size_t)head_dim + 2) * sizeof(float);
   JSG_REQUIRE(need <= NOALLOC_SCRATCH_BYTES,
               "jsgrad_hip_attn_decode_static: %d heads of %d at max_context %d need %zu bytes of workspace, the built-in one holds %zu; use jsgrad_hip_attn_decode "
               "with a workspace of its own", n_heads, head_dim, max_context, need, (size_t)NOALLOC_SCRATCH_BYTES);
@@ -181,11 +187,16 @@ int jsgrad_hip_attn_decode(const void *q, const void *cache_k, const void *cache
   a.q = q; a.cache_k = cache_k; a.cache_v = cache_v; a.st = st; a.out = out;
   a.counters = (int *)workspace;
   a.partial = (float *)((char *)workspace + 256);
-  a.n_kv_heads = n_kv_heads; a.nsplit = att_max_chunks(max_context); a.max_context = max_context;
+  const bool short_ctx = max_context <= ATT_SHORT_CONTEXT;
+  a.n_kv_heads = n_kv_heads; a.nsplit = att_max_chunks(max_context, short_ctx ? ATT_NW * 16 : ATT_CHUNK_MAX); a.max_context = max_context;
   a.scale = (float)(1.0 / sqrt((double)head_dim));
   const int n_rep = n_heads / n_kv_heads;
-  if (act == JSGRAD_F16) return head_dim == 64 ? launch_attn<_Float16, 64>(a, n_rep) : launch_attn<_Float16, 128>(a, n_rep);
-  return head_dim == 64 ? launch_attn<float, 64>(a, n_rep) : launch_attn<float, 128>(a, n_rep);
+  if (short_ctx) {
+    if (act == JSGRAD_F16) return head_dim == 64 ? launch_attn<_Float16, 64, ATT_NW>(a, n_rep) : launch_attn<_Float16, 128, ATT_NW>(a, n_rep);
+    return head_dim == 64 ? launch_attn<float, 64, ATT_NW>(a, n_rep) : launch_attn<float, 128, ATT_NW>(a, n_rep);
+  }
+  if (act == JSGRAD_F16) return head_dim == 64 ? launch_attn<_Float16, 64, ATT_NW_LONG>(a, n_rep) : launch_attn<_Float16, 128, ATT_NW_LONG>(a, n_rep);
+  return head_dim == 64 ? launch_attn<float, 64, ATT_NW_LONG>(a, n_rep) : launch_attn<float, 128, ATT_NW_LONG>(a, n_rep);
 }
 
 }  // extern "C"

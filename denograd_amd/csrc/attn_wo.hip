@@ -17,10 +17,12 @@
 
 namespace jsg {
 
-// One block of 16 wavefronts per CU: an attention item is worked on by 16 wavefronts (its chain of dependent steps is what the
-// launch waits for), and the attention row is fetched by 256 blocks instead of 1024.
+// Two blocks of 8 wavefronts per CU: an attention item is worked on by 8 wavefronts, as in jsgrad_hip_attn_decode for
+// contexts of up to 16384 positions (the two agree bit for bit), and the attention row is fetched by 512 blocks.  Measured
+// against blocks of 16 wavefronts: 1B 1394 -> 1448 tok/s, 3B int8 813 -> 831, 8B int8 515 -> 524 (at 4100 positions
+// 448 -> 446); blocks of 4 wavefronts are slower than both.
 #ifndef JSG_AW_THREADS
-#define JSG_AW_THREADS 1024
+#define JSG_AW_THREADS 512
 #endif
 constexpr int AW_THREADS = JSG_AW_THREADS;
 constexpr int AW_WAVES = AW_THREADS / 64;
@@ -150,7 +152,7 @@ static int attn_wo_impl(const void *q, const void *cache_k, const void *cache_v,
   JSG_REQUIRE(kind == JSGRAD_W_F16 || so || query_capacity, "jsgrad_hip_attn_wo: quantised weight needs a scale");
   JSG_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_kv_heads <= 64 && n_heads % n_kv_heads == 0, "jsgrad_hip_attn_wo: n_heads %d / n_kv_heads %d", n_heads, n_kv_heads);
   JSG_REQUIRE(head_dim == 64 || head_dim == 128, "jsgrad_hip_attn_wo: head_dim %d (64 and 128 are built)", head_dim);
-  JSG_REQUIRE(max_context > 0 && max_context <= 64 * ATT_CHUNK_MAX, "jsgrad_hip_attn_wo: max_context %d exceeds %d", max_context, 64 * ATT_CHUNK_MAX);
+  JSG_REQUIRE(max_context > 0 && max_context <= 64 * AW_CHUNK_CAP, "jsgrad_hip_attn_wo: max_context %d exceeds %d", max_context, 64 * AW_CHUNK_CAP);
   JSG_REQUIRE(layer >= 0 && layer < 128, "jsgrad_hip_attn_wo: layer index %d", layer);
   const int qdim = n_heads * head_dim;
   JSG_REQUIRE(dim > 0 && dim % 2 == 0 && qdim % 16 == 0 && (size_t)qdim * 2 <= 64 * 1024, "jsgrad_hip_attn_wo: dim %d / n_heads*head_dim %d", dim, qdim);

@@ -70,22 +70,22 @@ def test_attention_wo_launch_capacity_rule():
     against a given capacity here (on a GPU the library asks the occupancy calculator)."""
     from denograd_amd.llama import attn_wo_fits
     lib = ffi.load()
-    # chunks of the context: a tenth of T in whole 16s, at least 64 and at most 256 rows; the library provides the most
-    # chunks any T <= max_context asks for.  Checked against the rule itself, every T tried.
+    # chunks of the context: a tenth of T in whole 16s, at least 64 and at most 128 rows (blocks of 8 wavefronts, 16 rows
+    # each); the library provides the most chunks any T <= max_context asks for.  Checked against the rule itself, every T tried.
     def rows(T):
-        return min(256, max(64, (-(-T // 10) + 15) // 16 * 16))
+        return min(128, max(64, (-(-T // 10) + 15) // 16 * 16))
     most, m = {}, 0
     for T in range(1, 16385):
         m = max(m, -(-T // rows(T)))
         most[T] = m
-    for ctx in (1, 63, 64, 65, 512, 640, 641, 841, 952, 1400, 2304, 2560, 2561, 4340, 8192, 16384):
+    for ctx in (1, 63, 64, 65, 512, 640, 641, 841, 952, 1280, 1281, 1400, 2304, 2560, 2561, 4340, 8192):
         assert lib.jsgrad_hip_attn_wo_items(8, ctx) == 8 * most[ctx], ctx
     assert lib.jsgrad_hip_attn_wo_items(8, 841) == 8 * 10       # 10 chunks of 64 at T = 640 (841 itself: 9 of 96)
     assert lib.jsgrad_hip_attn_wo_items(2, 64) == 2 * 1
-    assert lib.jsgrad_hip_attn_wo_items(8, 16384) == 8 * 64     # 64 chunks of 256
-    cap = 4 * 256      # four blocks of 256 threads per compute unit
-    assert attn_wo_fits(32, 8, 128, 8192, ffi.W_I8, 4096, capacity=cap)            # the 8B shape: 256 items
+    assert lib.jsgrad_hip_attn_wo_items(8, 8192) == 8 * 64      # 64 chunks of 128
+    cap = 2 * 256      # two blocks of 512 threads per compute unit
+    assert attn_wo_fits(32, 8, 128, 8192, ffi.W_I8, 4096, capacity=cap)            # the 8B shape: 8 x 64 = 512 items just fit
     assert attn_wo_fits(32, 32, 64, 2048, ffi.W_F16, 2048, capacity=cap)           # 32 kv heads x 16 chunks = 512 items
-    assert not attn_wo_fits(32, 32, 64, 16384, ffi.W_F16, 2048, capacity=cap)      # 32 x 64 = 2048 items
-    assert attn_wo_fits(32, 32, 64, 8192, ffi.W_F16, 2048, capacity=cap)           # 32 x 32 = 1024 items just fit
-    assert not attn_wo_fits(64, 64, 64, 8192, ffi.W_F16, 4096, capacity=cap)
+    assert not attn_wo_fits(32, 32, 64, 4096, ffi.W_F16, 2048, capacity=cap)       # 32 x 32 = 1024 items
+    assert attn_wo_fits(64, 64, 64, 512, ffi.W_F16, 4096, capacity=cap)            # 64 x 8 = 512 items
+    assert not attn_wo_fits(64, 64, 64, 1280, ffi.W_F16, 4096, capacity=cap)       # 64 x 10 = 640 items

@@ -303,7 +303,8 @@ def attn_oracle(q, K, V, H, KV, hd, T, act16, round_p=True):
 
 @pytest.mark.parametrize("dt,H,KV,hd,ctx", [("float32", 4, 2, 64, 64), ("float16", 32, 8, 64, 1024), ("float16", 24, 8, 128, 600), ("float16", 8, 8, 128, 300),
                                              ("float16", 8, 1, 64, 2100), ("float32", 6, 2, 128, 96),
-                                             ("float16", 8, 2, 128, 4096)])   # 64-row chunks: more iterations than the rows requested up front
+                                             ("float16", 8, 2, 128, 4096),
+                                             ("float16", 4, 2, 64, 17000)])   # beyond 16384 positions: the 16-wavefront blocks with 256-row chunks
 def test_attention_decode(hip, dt, H, KV, hd, ctx):
     """GQA decode attention over the cache for several T, including T=1, chunk boundaries and the full cache;
     repeated launches share one workspace (the merging block must leave the counters at zero)."""

@@ -127,11 +127,11 @@ def test_prompt_prefix_reuse_and_cache_overrun():
 
 
 def test_many_kv_heads_fall_back_to_two_launches_and_still_match():
-    """32 kv heads at 16384 positions of context would need 2048 attention blocks in the fused attention + wo launch, more than
+    """32 kv heads at 8192 positions of context would need 2048 attention blocks in the fused attention + wo launch, more than
     the device holds at once: the library refuses that launch and the model runs attention and wo as two launches."""
     from denograd_amd import ffi
     from denograd_amd.tensor import Tensor
-    cfg = dict(dim=2048, hidden_dim=512, n_heads=32, n_kv_heads=32, n_layers=2, vocab_size=1024, norm_eps=1e-5, rope_theta=500000.0, max_context=16384,
+    cfg = dict(dim=2048, hidden_dim=512, n_heads=32, n_kv_heads=32, n_layers=2, vocab_size=1024, norm_eps=1e-5, rope_theta=500000.0, max_context=8192,
                act_dtype="float16", quantize="float16", tied=False, name="mha32")
     sd = synthetic.random_state_dict(cfg, seed=1)
     gpu = Llama3.from_config(cfg).load_weights(sd, quantized=True)
@@ -142,7 +142,7 @@ def test_many_kv_heads_fall_back_to_two_launches_and_still_match():
     lib = ffi.load()
     t = Tensor.zeros((2048 * 64,), "float16")
     ws = Tensor.zeros((lib.jsgrad_hip_attn_wo_workspace_bytes(32, 32, 64),), "uint8")
-    rc = lib.jsgrad_hip_attn_wo(t.ptr, t.ptr, t.ptr, gpu.model.state.ptr, ws.ptr, 32, 32, 64, 16384, ffi.W_F16, t.ptr, None, 2048, None, t.ptr, 0)
+    rc = lib.jsgrad_hip_attn_wo(t.ptr, t.ptr, t.ptr, gpu.model.state.ptr, ws.ptr, 32, 32, 64, 8192, ffi.W_F16, t.ptr, None, 2048, None, t.ptr, 0)
     assert rc != 0 and b"attention items" in lib.jsgrad_hip_last_error()
     # the same heads with a context of 512 positions (256 items) share the launch when the device says they fit
     import ctypes as C
