@@ -24,18 +24,25 @@ __device__ __forceinline__ uint32_t att_word(float v) {
   return ~(b == 0xFFFFFFFFu ? 0x7FC00000u : b);
 }
 
-// Rows per chunk for T visible positions.  A launch is a chain of round trips (rows, partial results, merge); the rows of a
-// chunk are fetched by one block, and the merge fetches one partial result per chunk.  About ten chunks per kv head is
-// where the two meet (measured on the 8B shape: 584 positions in 10 chunks 14.0 us per attention + wo launch, in 5 chunks
-// 15.3, in 19 chunks 16.0; 1064 positions in 9 chunks 13.5 us, in 17 chunks 14.5; 8, 10, 12 and 16 as the target measure
-// alike): a tenth of T, in whole 16s, at least 64 rows; 128-row chunks at 4100 positions are slower than 256 (18.6 / 15.8 us).
+// Rows per chunk for T visible positions.  A launch is a chain of round trips (rows, partial results, merge): the rows of a
+// chunk are fetched by one block, which takes time in proportion to the rows, and the merge fetches one partial result per
+// chunk, which takes time in proportion to T / rows; the sum is least where rows grows like the square root of T.
+// Measured with blocks of 8 wavefronts (tok/s of the whole decode step, chunks of 48 / 64 / 80 / 96 / 128 rows): 1B at 600
+// positions 1452 / 1455 / 1438 / 1440 / -; 8B int8 at 584 positions 526 / 526 / 516 / 504 / -; 3B int8 at 1064 positions
+// 820 / 815 / 841 / 835 / -; 8B int8 at 2100 positions 467 / 471 / 483 / 481 / 474 (112 rows); at 4100 positions
+// 423 / 434 / 437 / 443 / 449.  rows = 2 sqrt(T) in whole 16s, at least ATT_CHUNK_MIN, at most what the block shape takes.
 // `nsplit` chunks is what the workspace and the grid provide: the chunk grows if T would need more.
 // `cap`: the longest chunk the block shape can take (16 rows per wavefront, at most ATT_CHUNK_MAX; never below 64).
-constexpr int ATT_TARGET_CHUNKS = 10, ATT_CHUNK_MIN = 64, ATT_CHUNK_POLICY_MAX = ATT_CHUNK_MAX;
+constexpr int ATT_ROWS_SQ_PER_T = 4, ATT_CHUNK_MIN = 48;   // rows^2 = 4 T; ATT_CHUNK_MIN is a multiple of 16
+__host__ __device__ __forceinline__ int att_isqrt(int x) {   // floor(sqrt(x)), the same on the host and on the device
+  int r = (int)__builtin_sqrtf((float)x);
+  while (r * r > x) r--;
+  while ((r + 1) * (r + 1) <= x) r++;
+  return r;
+}
 __host__ __device__ __forceinline__ int att_policy_rows(int T, int cap) {
-  int c = ((T + ATT_TARGET_CHUNKS - 1) / ATT_TARGET_CHUNKS + 15) & ~15;
+  int c = (att_isqrt(ATT_ROWS_SQ_PER_T * T) + 15) & ~15;
   c = c < ATT_CHUNK_MIN ? ATT_CHUNK_MIN : c;
-  c = c < ATT_CHUNK_POLICY_MAX ? c : ATT_CHUNK_POLICY_MAX;
   return c < cap ? c : cap;
 }
 __host__ __device__ __forceinline__ int att_chunk_rows(int T, int nsplit, int cap = ATT_CHUNK_MAX) {
@@ -43,14 +50,20 @@ __host__ __device__ __forceinline__ int att_chunk_rows(int T, int nsplit, int ca
   const int need = (T + nsplit - 1) / nsplit;
   return c < need ? need : c;
 }
-// chunks a launch must provide for every T up to max_context: up to ATT_TARGET_CHUNKS * ATT_CHUNK_MIN positions the count
-// grows with T, then it stays at or below the target until the chunks reach their longest
+// chunks a launch must provide for every T up to max_context.  The rows per chunk never shrink as T grows, so for each
+// chunk length r the most chunks are asked for at the largest T that still gets r rows: sqrt(K T) <= r, i.e.
+// T <= ((r + 1)^2 - 1) / K (any T for the shortest and up to max_context for the longest).
 __host__ __device__ __forceinline__ int att_max_chunks(int max_context, int cap = ATT_CHUNK_MAX) {
-  const int longest = cap < ATT_CHUNK_POLICY_MAX ? cap : ATT_CHUNK_POLICY_MAX;
-  const int knee = ATT_TARGET_CHUNKS * ATT_CHUNK_MIN;
-  const int low = ((max_context < knee ? max_context : knee) + ATT_CHUNK_MIN - 1) / ATT_CHUNK_MIN;
-  const int high = (max_context + longest - 1) / longest;
-  return low > high ? low : high;
+  int most = 1;
+  for (int r = ATT_CHUNK_MIN; ; r += 16) {
+    if (r > cap) r = cap;
+    int t_last = ((r + 1) * (r + 1) - 1) / ATT_ROWS_SQ_PER_T;
+    if (r == cap || t_last > max_context) t_last = max_context;
+    const int n = (t_last + r - 1) / r;
+    most = n > most ? n : most;
+    if (r == cap || t_last == max_context) break;
+  }
+  return most;
 }
 
 struct AttnArgs {

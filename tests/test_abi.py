@@ -70,22 +70,23 @@ def test_attention_wo_launch_capacity_rule():
     against a given capacity here (on a GPU the library asks the occupancy calculator)."""
     from denograd_amd.llama import attn_wo_fits
     lib = ffi.load()
-    # chunks of the context: a tenth of T in whole 16s, at least 64 and at most 128 rows (blocks of 8 wavefronts, 16 rows
-    # each); the library provides the most chunks any T <= max_context asks for.  Checked against the rule itself, every T tried.
+    # chunks of the context: 2 sqrt(T) rows in whole 16s, at least 48 and at most 128 (blocks of 8 wavefronts, 16 rows each);
+    # the library provides the most chunks any T <= max_context asks for.  Checked against the rule itself, every T tried.
+    import math
     def rows(T):
-        return min(128, max(64, (-(-T // 10) + 15) // 16 * 16))
+        return min(128, max(48, (math.isqrt(4 * T) + 15) // 16 * 16))
     most, m = {}, 0
-    for T in range(1, 16385):
+    for T in range(1, 8193):
         m = max(m, -(-T // rows(T)))
         most[T] = m
-    for ctx in (1, 63, 64, 65, 512, 640, 641, 841, 952, 1280, 1281, 1400, 2304, 2560, 2561, 4340, 8192):
+    for ctx in (1, 47, 48, 49, 512, 600, 601, 841, 952, 1056, 1057, 1400, 2304, 2560, 4096, 4097, 4340, 8192):
         assert lib.jsgrad_hip_attn_wo_items(8, ctx) == 8 * most[ctx], ctx
-    assert lib.jsgrad_hip_attn_wo_items(8, 841) == 8 * 10       # 10 chunks of 64 at T = 640 (841 itself: 9 of 96)
-    assert lib.jsgrad_hip_attn_wo_items(2, 64) == 2 * 1
+    assert lib.jsgrad_hip_attn_wo_items(8, 600) == 8 * 13       # 13 chunks of 48 rows
+    assert lib.jsgrad_hip_attn_wo_items(2, 48) == 2 * 1
     assert lib.jsgrad_hip_attn_wo_items(8, 8192) == 8 * 64      # 64 chunks of 128
     cap = 2 * 256      # two blocks of 512 threads per compute unit
     assert attn_wo_fits(32, 8, 128, 8192, ffi.W_I8, 4096, capacity=cap)            # the 8B shape: 8 x 64 = 512 items just fit
-    assert attn_wo_fits(32, 32, 64, 2048, ffi.W_F16, 2048, capacity=cap)           # 32 kv heads x 16 chunks = 512 items
+    assert attn_wo_fits(32, 32, 64, 768, ffi.W_F16, 2048, capacity=cap)            # 32 kv heads x 13 chunks = 416 items
     assert not attn_wo_fits(32, 32, 64, 4096, ffi.W_F16, 2048, capacity=cap)       # 32 x 32 = 1024 items
-    assert attn_wo_fits(64, 64, 64, 512, ffi.W_F16, 4096, capacity=cap)            # 64 x 8 = 512 items
-    assert not attn_wo_fits(64, 64, 64, 1280, ffi.W_F16, 4096, capacity=cap)       # 64 x 10 = 640 items
+    assert attn_wo_fits(64, 64, 64, 384, ffi.W_F16, 4096, capacity=cap)            # 64 x 8 = 512 items
+    assert not attn_wo_fits(64, 64, 64, 600, ffi.W_F16, 4096, capacity=cap)        # 64 x 13 = 832 items
