@@ -20,8 +20,8 @@ __global__ __launch_bounds__(NW * 64) void attn_decode_kernel(AttnArgs a) {
   const int pos = a.st[1];
   if (pos < 0 || pos >= a.max_context) return;
   const int T = pos + 1;
-  const int chunk = att_chunk_rows(T, a.nsplit, A::CHUNK_CAP);  // the host sized nsplit for max_context and this cap
-  const int n_active = (T + chunk - 1) / chunk;
+  const int chunk = att_policy_rows(T, A::CHUNK_CAP);            // the host sized nsplit for max_context and this cap
+  const int n_active = att_chunk_count(T, chunk);
   if (split >= n_active) return;
   A::item(a, sm, g, split, T, chunk, n_active);
 }

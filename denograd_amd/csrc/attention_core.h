@@ -31,25 +31,29 @@ __device__ __forceinline__ uint32_t att_word(float v) {
 // positions 1452 / 1455 / 1438 / 1440 / -; 8B int8 at 584 positions 526 / 526 / 516 / 504 / -; 3B int8 at 1064 positions
 // 820 / 815 / 841 / 835 / -; 8B int8 at 2100 positions 467 / 471 / 483 / 481 / 474 (112 rows); at 4100 positions
 // 423 / 434 / 437 / 443 / 449.  rows = 2 sqrt(T) in whole 16s, at least ATT_CHUNK_MIN, at most what the block shape takes.
-// `nsplit` chunks is what the workspace and the grid provide: the chunk grows if T would need more.
 // `cap`: the longest chunk the block shape can take (16 rows per wavefront, at most ATT_CHUNK_MAX; never below 64).
 constexpr int ATT_ROWS_SQ_PER_T = 4, ATT_CHUNK_MIN = 48;   // rows^2 = 4 T; ATT_CHUNK_MIN is a multiple of 16
-__host__ __device__ __forceinline__ int att_isqrt(int x) {   // floor(sqrt(x)), the same on the host and on the device
-  int r = (int)__builtin_sqrtf((float)x);
+__host__ __device__ __forceinline__ int att_isqrt(int x) {   // floor(sqrt(x)), the same on the host and on the device:
+  int r = (int)__builtin_sqrtf((float)x);                    // any estimate, made exact by the two loops
   while (r * r > x) r--;
   while ((r + 1) * (r + 1) <= x) r++;
   return r;
+}
+// ceil(T / chunk) without an integer division (dozens of dependent instructions on the device, at the head of a launch
+// that is a chain of latencies): an estimate from a reciprocal, made exact by the two loops
+__host__ __device__ __forceinline__ int att_chunk_count(int T, int chunk) {
+  int n = (int)((float)T * (1.0f / (float)chunk)) + 1;
+  while ((n - 1) * chunk >= T) n--;
+  while (n * chunk < T) n++;
+  return n;
 }
 __host__ __device__ __forceinline__ int att_policy_rows(int T, int cap) {
   int c = (att_isqrt(ATT_ROWS_SQ_PER_T * T) + 15) & ~15;
   c = c < ATT_CHUNK_MIN ? ATT_CHUNK_MIN : c;
   return c < cap ? c : cap;
 }
-__host__ __device__ __forceinline__ int att_chunk_rows(int T, int nsplit, int cap = ATT_CHUNK_MAX) {
-  const int c = att_policy_rows(T, cap);
-  const int need = (T + nsplit - 1) / nsplit;
-  return c < need ? need : c;
-}
+// (A launch provides att_max_chunks(max_context, cap) chunks, the most this rule asks for at any T <= max_context, so the
+// kernels take the rule as it is.)
 // chunks a launch must provide for every T up to max_context.  The rows per chunk never shrink as T grows, so for each
 // chunk length r the most chunks are asked for at the largest T that still gets r rows: sqrt(K T) <= r, i.e.
 // T <= ((r + 1)^2 - 1) / K (any T for the shortest and up to max_context for the longest).
@@ -74,6 +78,7 @@ struct AttnArgs {
   int *err = nullptr;   // optional: set to 1 when the merging block's bounded wait for the other chunks ran out
   float *partial;  // [n_kv_heads][nsplit][n_rep][HD + 2]
   int n_kv_heads, nsplit, max_context;
+  int kv_magic = 0;   // ceil(65536 / n_kv_heads): block id / n_kv_heads = (id * kv_magic) >> 16 for id * n_kv_heads < 65536 (attn_wo.hip)
   float scale;     // float(1 / sqrt(head_dim)) (tensor.ts:3923 `.div(Math.sqrt(d))` = mul by the folded reciprocal)
   // several sequences at the same position (grid z): distance between consecutive sequences, in bytes (q, out, caches)
   // and in elements (counters, partial); zero for a single sequence
@@ -357,9 +362,11 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       for (int i = 0; i < MSL; i++)
         if (i * 64 < n_active) mls[i] = ld_pair(base + (size_t)wave * (HD + 2) + HD, lane + i * 64);   // same test for the whole wavefront
     }
+    // The partial sums of this thread's first pair are asked for as soon as its wavefront has seen every chunk's (m, l)
+    // (the owners of pairs are threads of those wavefronts: NREP * HD / 128 <= NREP of them): asked for before that, the
+    // words of a chunk that is still computing come back empty and the request has to be repeated a round trip later.
     uint64_t part[MB];
-#pragma unroll
-    for (int u = 0; u < MB; u++) part[u] = ld_pair(po0, u);
+    bool asked = false;
     for (int j = wave; j < NREP; j += NW) {
       const float *pml = base + (size_t)j * (HD + 2) + HD;
       bool lost = false;
@@ -380,6 +387,11 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
         if (it >= POLL_LIMIT) { lost = true; gave_up(); break; }
         __builtin_amdgcn_s_sleep(1);
       }
+      if (!asked && tid < NPAIR) {
+#pragma unroll
+        for (int u = 0; u < MB; u++) part[u] = ld_pair(po0, u);
+      }
+      asked = true;
       if constexpr (WORDS) {
 #pragma unroll
         for (int i = 0; i < MSL; i++)
@@ -404,6 +416,10 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       if (__builtin_amdgcn_ballot_w64(lost) != 0) L = __builtin_nanf("");
       if (lane == 0) sm.l_sh[j] = 1.0f / L;  // softmax normalisation is e * (1/sum) (tensor.ts:2211-2214)
     }
+    if (!asked && tid < NPAIR) {        // a wavefront without a query head of its own (no built shape has one that owns pairs)
+#pragma unroll
+      for (int u = 0; u < MB; u++) part[u] = ld_pair(po0, u);
+    }
     lds_barrier();
     auto finish = [&](int i, float O) {
       const int j = i / HD, d = i % HD;
@@ -424,26 +440,29 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
             for (int u = 0; u < MB; u++) part[u] = ld_pair(po, s0 + u);
           }
           if constexpr (!WORDS) break;
+          // no branches from here to the sums: a chunk index past the end stands for the last chunk (ld_pair, clear_pair),
+          // whose words are checked and cleared again and enter the sum with weight zero
           bool ok = true;
 #pragma unroll
-          for (int u = 0; u < MB; u++)
-            if (s0 + u < n_active && !written(part[u])) ok = false;
+          for (int u = 0; u < MB; u++) ok = ok & written(part[u]);
           if (ok) break;
           if (it >= POLL_LIMIT) { Oa = Ob = __builtin_nanf(""); gave_up(); break; }
           __builtin_amdgcn_s_sleep(1);
         }
         if constexpr (WORDS) {
 #pragma unroll
-          for (int u = 0; u < MB; u++)
-            if (s0 + u < n_active) clear_pair(po, s0 + u);
+          for (int u = 0; u < MB; u++) clear_pair(po, s0 + u);
         }
+        float wgt[MB];
 #pragma unroll
-        for (int u = 0; u < MB; u++)
-          if (s0 + u < n_active) {
-            const float w = sm.sc[j][s0 + u];
-            Oa = fmaf(dec((uint32_t)part[u]), w, Oa);
-            Ob = fmaf(dec((uint32_t)(part[u] >> 32)), w, Ob);
-          }
+        for (int u = 0; u < MB; u++) wgt[u] = sm.sc[j][s0 + u < n_active ? s0 + u : n_active - 1];
+#pragma unroll
+        for (int u = 0; u < MB; u++) {
+          const bool in = s0 + u < n_active;
+          const float w = in ? wgt[u] : 0.0f;
+          Oa = fmaf(in ? dec((uint32_t)part[u]) : 0.0f, w, Oa);
+          Ob = fmaf(in ? dec((uint32_t)(part[u] >> 32)) : 0.0f, w, Ob);
+        }
       }
       finish(2 * p, Oa);
       finish(2 * p + 1, Ob);

@@ -55,15 +55,17 @@ __global__ __launch_bounds__(AW_THREADS) void attn_wo_kernel(AttnArgs at, GemvAr
   bool has_item = false;
   if (pos >= 0 && pos < at.max_context) {
     const int T = pos + 1;
-    const int chunk = att_chunk_rows(T, at.nsplit, AW_CHUNK_CAP);   // the host sized nsplit for max_context and this cap
-    const int n_active = (T + chunk - 1) / chunk;
+    const int chunk = att_policy_rows(T, AW_CHUNK_CAP);              // the host sized nsplit for max_context and this cap
+    const int n_active = att_chunk_count(T, chunk);
     const int id = blockIdx.x;
     has_item = id < at.n_kv_heads * n_active;
     // This wavefront's first wo item is requested as soon as the attention item lets it (attention_core.h: loads return in
     // order and the item's barriers wait for every outstanding one, so weights requested earlier would sit in front of the
     // rows and partial results the item waits for): when the block has published its chunk, or, in the block that merges,
     // behind the merge's requests, so that the weights travel while the merge computes.
-    if (has_item) A::item(at, sm, id % at.n_kv_heads, id / at.n_kv_heads, T, chunk, n_active, [&]() { if (preloaded) G::load_item(a, buf, grp, 0, 0); });
+    // (kv head, chunk) of block id without an integer division: the host passes ceil(65536 / n_kv_heads)
+    const int split = (int)(((uint32_t)id * (uint32_t)at.kv_magic) >> 16), g = id - split * at.n_kv_heads;
+    if (has_item) A::item(at, sm, g, split, T, chunk, n_active, [&]() { if (preloaded) G::load_item(a, buf, grp, 0, 0); });
   } else if (blockIdx.x == 0 && threadIdx.x == 0) {
     st_coherent(a.err, 1);   // no attention row will come for such a position
   }
@@ -162,6 +164,7 @@ static int attn_wo_impl(const void *q, const void *cache_k, const void *cache_v,
   at.counters = (int *)ws;
   at.partial = (float *)(ws + 512);
   at.n_kv_heads = n_kv_heads; at.nsplit = aw_nsplit(max_context); at.max_context = max_context;
+  at.kv_magic = (65536 + n_kv_heads - 1) / n_kv_heads;   // exact for block ids below 65536 / n_kv_heads >= 1024 (the grid has at most two blocks per CU)
   at.scale = (float)(1.0 / sqrt((double)head_dim));
   at.out_tagged = (uint32_t *)(ws + 512 + (size_t)n_heads * 256 * (head_dim + 2) * sizeof(float));
   at.err = (int *)(ws + 256);
