@@ -224,23 +224,39 @@ template <typename AT, bool COHERENT> __device__ __forceinline__ void stage_x(co
       // all chunks of a thread are asked for together, again and again until every one carries the tag: one round trip
       // when the row is there, instead of one per chunk
       constexpr int NCH = 2;
-      for (int c0 = tid; c0 < nchunks; c0 += NCH * nt) {
-        u4_t v[NCH];
-        for (int it = 0;; it++) {
-          bool ok = true;
+      if (nchunks <= nt) {
+        // one chunk per thread at most (every block of the launch fetches the whole row at the same moment: nothing is
+        // requested twice)
+        if (tid < nchunks) {
+          u4_t v;
+          for (int it = 0;; it++) {
+            bool ok = true;
+            v = tw_load8(a.x_tagged + (size_t)tid * 8, a.x_tag, ok);
+            if (ok) break;
+            if (it > (1 << 18)) { st_coherent(a.err, 1); break; }
+            __builtin_amdgcn_s_sleep(4);   // not there yet: leave the memory system to those who are producing it
+          }
+          xl[tid] = v;
+        }
+      } else {
+        for (int c0 = tid; c0 < nchunks; c0 += NCH * nt) {
+          u4_t v[NCH];
+          for (int it = 0;; it++) {
+            bool ok = true;
+#pragma unroll
+            for (int i = 0; i < NCH; i++) {
+              const int c = c0 + i * nt;
+              v[i] = tw_load8(a.x_tagged + (size_t)(c < nchunks ? c : c0) * 8, a.x_tag, ok);   // past the end: its own first chunk again
+            }
+            if (ok) break;
+            if (it > (1 << 18)) { st_coherent(a.err, 1); break; }
+            __builtin_amdgcn_s_sleep(4);   // not there yet: leave the memory system to those who are producing it
+          }
 #pragma unroll
           for (int i = 0; i < NCH; i++) {
             const int c = c0 + i * nt;
-            v[i] = tw_load8(a.x_tagged + (size_t)(c < nchunks ? c : c0) * 8, a.x_tag, ok);   // past the end: its own first chunk again
+            if (c < nchunks) xl[c] = v[i];
           }
-          if (ok) break;
-          if (it > (1 << 18)) { st_coherent(a.err, 1); break; }
-          __builtin_amdgcn_s_sleep(4);   // not there yet: leave the memory system to those who are producing it
-        }
-#pragma unroll
-        for (int i = 0; i < NCH; i++) {
-          const int c = c0 + i * nt;
-          if (c < nchunks) xl[c] = v[i];
         }
       }
     } else {
