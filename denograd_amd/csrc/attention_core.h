@@ -33,12 +33,6 @@ __device__ __forceinline__ uint32_t att_word(float v) {
 // 423 / 434 / 437 / 443 / 449.  rows = 2 sqrt(T) in whole 16s, at least ATT_CHUNK_MIN, at most what the block shape takes.
 // `cap`: the longest chunk the block shape can take (16 rows per wavefront, at most ATT_CHUNK_MAX; never below 64).
 constexpr int ATT_ROWS_SQ_PER_T = 4, ATT_CHUNK_MIN = 48;   // rows^2 = 4 T; ATT_CHUNK_MIN is a multiple of 16
-__host__ __device__ __forceinline__ int att_isqrt(int x) {   // floor(sqrt(x)), the same on the host and on the device:
-  int r = (int)__builtin_sqrtf((float)x);                    // any estimate, made exact by the two loops
-  while (r * r > x) r--;
-  while ((r + 1) * (r + 1) <= x) r++;
-  return r;
-}
 // ceil(T / chunk) without an integer division (dozens of dependent instructions on the device, at the head of a launch
 // that is a chain of latencies): an estimate from a reciprocal, made exact by the two loops
 __host__ __device__ __forceinline__ int att_chunk_count(int T, int chunk) {
@@ -47,10 +41,11 @@ __host__ __device__ __forceinline__ int att_chunk_count(int T, int chunk) {
   while (n * chunk < T) n++;
   return n;
 }
+// floor(sqrt(K T)) rounded up to a whole 16 is the smallest r = 16 i with K T < (r + 1)^2: a few compares, no square root
 __host__ __device__ __forceinline__ int att_policy_rows(int T, int cap) {
-  int c = (att_isqrt(ATT_ROWS_SQ_PER_T * T) + 15) & ~15;
-  c = c < ATT_CHUNK_MIN ? ATT_CHUNK_MIN : c;
-  return c < cap ? c : cap;
+  int r = ATT_CHUNK_MIN;
+  while (r < cap && ATT_ROWS_SQ_PER_T * T >= (r + 1) * (r + 1)) r += 16;
+  return r < cap ? r : cap;
 }
 // (A launch provides att_max_chunks(max_context, cap) chunks, the most this rule asks for at any T <= max_context, so the
 // kernels take the rule as it is.)
