@@ -340,8 +340,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct AttnStrea
       if (lane == 0) sm.l_sh[j] = 1.0f / L;  // softmax normalisation is e * (1/sum) (tensor.ts:2211-2214)
     }
     __syncthreads();
-    // ... then every thread sums its output elements over the chunks in chunk order.  Two elements at a time: the first 32
-    // chunks of both are requested together (one round trip where there would be two; few chunks is the usual case)
+    // ... then every thread sums its output elements over the chunks in chunk order, two elements at a time
     auto finish = [&](int i, float O) {
       const int j = i / HD, d = i % HD;
       AT *dst = (AT *)a.out + (size_t)(g * NREP + j) * HD + d;
@@ -357,35 +356,35 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct AttnStrea
       const bool two = PAIRS && i1 < NREP * HD;
       const int ja = i0 / HD, jb = (two ? i1 : i0) / HD;
       const float *pa = base + (size_t)ja * (HD + 2) + i0 % HD, *pb = base + (size_t)jb * (HD + 2) + (two ? i1 : i0) % HD;
-      float parta[32], partb[32];
-#pragma unroll
-      for (int u = 0; u < 32; u++) parta[u] = ld_part(pa, u);
-      if constexpr (PAIRS) {
-#pragma unroll
-        for (int u = 0; u < 32; u++) partb[u] = ld_part(pb, u);
-      }
+      // 16 chunks of both elements per round of requests (the usual number of chunks fits one round), summed in chunk order
+      // without a branch per chunk (a branch each would make every weight an LDS read with a wait of its own): the weights
+      // of 8 chunks are read together; an index past the last chunk stands for the last chunk (ld_part) with weight zero.
+      constexpr int MBS = 16;
       float Oa = 0.0f, Ob = 0.0f;
+      auto add = [&](const float (&part)[MBS], int j, int s0, float O) {
 #pragma unroll
-      for (int u = 0; u < 32; u++)
-        if (u < n_active) Oa = fmaf(parta[u], sm.sc[ja][u], Oa);
-      if constexpr (PAIRS) {
+        for (int u0 = 0; u0 < MBS; u0 += 8) {
+          float w[8];
 #pragma unroll
-        for (int u = 0; u < 32; u++)
-          if (u < n_active) Ob = fmaf(partb[u], sm.sc[jb][u], Ob);
-      }
-      for (int s0 = 32; s0 < n_active; s0 += 32) {           // more than 32 chunks: the rest in batches, element by element
+          for (int u = 0; u < 8; u++) w[u] = sm.sc[j][s0 + u0 + u < n_active ? s0 + u0 + u : n_active - 1];
 #pragma unroll
-        for (int u = 0; u < 32; u++) parta[u] = ld_part(pa, s0 + u);
+          for (int u = 0; u < 8; u++) {
+            const bool in = s0 + u0 + u < n_active;
+            O = fmaf(in ? part[u0 + u] : 0.0f, in ? w[u] : 0.0f, O);
+          }
+        }
+        return O;
+      };
+      for (int s0 = 0; s0 < n_active; s0 += MBS) {
+        float parta[MBS], partb[MBS];
 #pragma unroll
-        for (int u = 0; u < 32; u++)
-          if (s0 + u < n_active) Oa = fmaf(parta[u], sm.sc[ja][s0 + u], Oa);
+        for (int u = 0; u < MBS; u++) parta[u] = ld_part(pa, s0 + u);
         if constexpr (PAIRS) {
 #pragma unroll
-          for (int u = 0; u < 32; u++) partb[u] = ld_part(pb, s0 + u);
-#pragma unroll
-          for (int u = 0; u < 32; u++)
-            if (s0 + u < n_active) Ob = fmaf(partb[u], sm.sc[jb][s0 + u], Ob);
+          for (int u = 0; u < MBS; u++) partb[u] = ld_part(pb, s0 + u);
         }
+        Oa = add(parta, ja, s0, Oa);
+        if constexpr (PAIRS) Ob = add(partb, jb, s0, Ob);
       }
       finish(i0, Oa);
       if (two) finish(i1, Ob);
