@@ -239,21 +239,37 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       for (int c = 0; c < IPR; c++)
 #pragma unroll
         for (int e = 0; e < EP; e++) of[j][c][e] = 0.0f;
+    // The probabilities of PB row steps are read from LDS together, then multiplied: read one step at a time behind the
+    // test that skips the steps a short chunk does not have, every step would wait out an LDS round trip of its own.
+    constexpr int PB = (NREP * HD >= 512 ? 2 : 4) * IPR;   // loads per batch: 4 row steps, 2 where the sums already fill the registers
 #pragma unroll
-    for (int i = 0; i < VIT; i++) {
-      const int ri = i / IPR, part = i % IPR;
-      if (ri * RPV < VR) {
-        const int r = ri * RPV + vsel;
-        const int t = t0 + wave * VR + r;
-        const bool ok = r < VR && t < t1;
-        float vf[EP];
-        if constexpr (sizeof(AT) == 2) { const h2_t h = as_h2(vreg[i]); vf[0] = (float)h[0]; vf[1] = (float)h[1]; }
-        else vf[0] = __uint_as_float(vreg[i]);
+    for (int i0 = 0; i0 < VIT; i0 += PB) {
+      if ((i0 / IPR) * RPV < VR) {             // the same for the whole block
+        float pr[PB / IPR][NREP];
+        bool okr[PB / IPR];
 #pragma unroll
-        for (int j = 0; j < NREP; j++) {
-          const float p = ok ? sm.sc[j][ok ? t - t0 : 0] : 0.0f;   // rows past the chunk: an existing row times zero
+        for (int q = 0; q < PB / IPR; q++) {
+          const int r = (i0 / IPR + q) * RPV + vsel;
+          const int t = t0 + wave * VR + r;
+          okr[q] = r < VR && t < t1;
 #pragma unroll
-          for (int e = 0; e < EP; e++) of[j][part][e] = fmaf(p, vf[e], of[j][part][e]);
+          for (int j = 0; j < NREP; j++) pr[q][j] = sm.sc[j][okr[q] ? t - t0 : 0];
+        }
+#pragma unroll
+        for (int ii = 0; ii < PB; ii++) {
+          const int i = i0 + ii;
+          if (i < VIT && (i / IPR) * RPV < VR) {   // a step past the wavefront's rows has no value loaded
+            const int q = ii / IPR, part = i % IPR;
+            float vf[EP];
+            if constexpr (sizeof(AT) == 2) { const h2_t h = as_h2(vreg[i]); vf[0] = (float)h[0]; vf[1] = (float)h[1]; }
+            else vf[0] = __uint_as_float(vreg[i]);
+#pragma unroll
+            for (int j = 0; j < NREP; j++) {
+              const float p = okr[q] ? pr[q][j] : 0.0f;   // rows past the chunk: an existing row times zero
+#pragma unroll
+              for (int e = 0; e < EP; e++) of[j][part][e] = fmaf(p, vf[e], of[j][part][e]);
+            }
+          }
         }
       }
     }
