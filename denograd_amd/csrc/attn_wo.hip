@@ -52,26 +52,30 @@ __global__ __launch_bounds__(AW_THREADS) void attn_wo_kernel(AttnArgs at, GemvAr
   const int wo_blk = (int)blockIdx.x - at.n_kv_heads, wo_nblk = (int)gridDim.x - at.n_kv_heads;
   const int grp = G::first_group(wo_blk, wo_nblk);
   const bool preloaded = wo_blk >= 0 && grp < G::ngroups(a);
-  bool has_item = false;
+  // A block either runs an attention item or, without one, asks for its first wo item right away.  The two are the
+  // branches of one if / else on purpose: written as two tests in a row, the compiler's wait-count pass saw the requests of
+  // the second reach the first, and made every K and V request of the item wait for the one before it.
+  int T = 1, chunk = ATT_CHUNK_MIN, n_active = 0;
   if (pos >= 0 && pos < at.max_context) {
-    const int T = pos + 1;
-    const int chunk = att_policy_rows(T, AW_CHUNK_CAP);              // the host sized nsplit for max_context and this cap
-    const int n_active = att_chunk_count(T, chunk);
-    const int id = blockIdx.x;
-    has_item = id < at.n_kv_heads * n_active;
+    T = pos + 1;
+    chunk = att_policy_rows(T, AW_CHUNK_CAP);                        // the host sized nsplit for max_context and this cap
+    n_active = att_chunk_count(T, chunk);
+  } else if (blockIdx.x == 0 && threadIdx.x == 0) {
+    st_coherent(a.err, 1);   // no attention row will come for such a position
+  }
+  const int id = blockIdx.x;
+  if (id < at.n_kv_heads * n_active) {
     // This wavefront's first wo item is requested as soon as the attention item lets it (attention_core.h: loads return in
     // order and the item's barriers wait for every outstanding one, so weights requested earlier would sit in front of the
     // rows and partial results the item waits for): when the block has published its chunk, or, in the block that merges,
     // behind the merge's requests, so that the weights travel while the merge computes.
     // (kv head, chunk) of block id without an integer division: the host passes ceil(65536 / n_kv_heads)
     const int split = (int)(((uint32_t)id * (uint32_t)at.kv_magic) >> 16), g = id - split * at.n_kv_heads;
-    if (has_item) A::item(at, sm, g, split, T, chunk, n_active, [&]() { if (preloaded) G::load_item(a, buf, grp, 0, 0); });
-  } else if (blockIdx.x == 0 && threadIdx.x == 0) {
-    st_coherent(a.err, 1);   // no attention row will come for such a position
-  }
-  // The other blocks give the items' small requests a head start before they flood the memory system with theirs; either
-  // way the weights are there before the attention row is.
-  if (!has_item) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+    A::item(at, sm, g, split, T, chunk, n_active, [&]() { if (preloaded) G::load_item(a, buf, grp, 0, 0); });
+  } else {
+    // The other blocks give the items' small requests a head start before they flood the memory system with theirs; either
+    // way the weights are there before the attention row is.
     __builtin_amdgcn_s_sleep(64);
     if (preloaded) G::load_item(a, buf, grp, 0, 0);
   }
