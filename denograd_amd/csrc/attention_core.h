@@ -317,20 +317,17 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       st_coherent(&mine[tid * (HD + 2) + HD], enc(sm.m_sh[tid]));
       st_coherent(&mine[tid * (HD + 2) + HD + 1], enc(sm.l_sh[tid]));
     }
+    // One way through for every block: the block of chunk 0 merges, then every block calls `then`.  (With an early exit
+    // for the others, the compiler placed their `then` in front of the merge and made the merging block wait for its own
+    // stores, as if they were `then`'s requests, before it could ask for anybody's results.)
+    const bool merges = split == 0;
     if constexpr (WORDS) {
-      if (split != 0) {
-        then();
-        return;
-      }
-      lds_barrier();   // m_sh / l_sh / sc are written again below
+      if (merges) lds_barrier();   // m_sh / l_sh / sc are written again below
     } else {
       __syncthreads();  // every coherent store of the block has been acknowledged
-      if (split != 0) {
+      if (!merges) {
         if (tid == 0) __hip_atomic_fetch_add(&a.counters[g], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // nobody waits for the answer
-        then();
-        return;
-      }
-      if (n_active > 1) {
+      } else if (n_active > 1) {
         if (tid == 0) {
           // The other chunks' blocks never wait for anything before they count themselves in, and the launch keeps them all on the
           // device, so this wait ends; it is bounded all the same and reports through the error word where one is given.
@@ -344,139 +341,141 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
         __syncthreads();
       }
     }
-    // merge.  Every thread owns two neighbouring output elements and requests their partial sums of the first MB chunks
-    // right away; while those travel, one wavefront per query head fetches the per-chunk (m, l), turns them into weights
-    // exp(m_s - M) and 1/L in LDS; then the sums are folded in chunk order.  One round trip for up to MB chunks.
-    // WORDS: a request is repeated while one of its words is still zero.  The other chunks' blocks never wait for anything
-    // before they store, and the launch keeps them all on the device, so this ends; it is bounded all the same, reports
-    // through the error word where one is given, and the result is then NaN.
-    const float *base = a.partial + (size_t)g * a.nsplit * NREP * (HD + 2);
-    constexpr int MB = 16;                       // chunks per batch of requests
-    constexpr int NPAIR = NREP * HD / 2;         // element pairs of this kv head's query heads
-    constexpr int POLL_LIMIT = 1 << 18;
-    auto pair_at = [&](const float *po, int s_) { return po + (size_t)(s_ < n_active ? s_ : n_active - 1) * NREP * (HD + 2); };
-    auto ld_pair = [&](const float *po, int s_) -> uint64_t {   // two floats of chunk s_ (8-byte aligned: HD + 2 is even)
-      return __hip_atomic_load(as_global<uint64_t>(pair_at(po, s_)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    };
-    auto clear_pair = [&](const float *po, int s_) {
-      __hip_atomic_store(as_global_mut<uint64_t>(const_cast<float *>(pair_at(po, s_))), 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    };
-    auto written = [](uint64_t w) { return (uint32_t)w != 0u && (uint32_t)(w >> 32) != 0u; };
-    auto gave_up = [&]() { if (a.err != nullptr) st_coherent(a.err, 1); };
-    const int p0 = tid < NPAIR ? tid : 0;        // threads beyond the pairs request pair 0 again (their result is not stored)
-    const int j0 = (2 * p0) / HD, d0 = (2 * p0) % HD;
-    const float *po0 = base + (size_t)j0 * (HD + 2) + d0;
-    constexpr int MSL = (CHUNK_CAP + 63) / 64;   // chunks per lane (the host keeps n_active <= CHUNK_CAP)
-    uint64_t mls[MSL];                         // wavefront j: (m, l) of this lane's chunks of head j, requested in one go
-    if (wave < NREP) {
-#pragma unroll
-      for (int i = 0; i < MSL; i++)
-        if (i * 64 < n_active) mls[i] = ld_pair(base + (size_t)wave * (HD + 2) + HD, lane + i * 64);   // same test for the whole wavefront
-    }
-    // The partial sums of this thread's first pair are asked for as soon as its wavefront has seen every chunk's (m, l)
-    // (the owners of pairs are threads of those wavefronts: NREP * HD / 128 <= NREP of them): asked for before that, the
-    // words of a chunk that is still computing come back empty and the request has to be repeated a round trip later.
-    uint64_t part[MB];
-    bool asked = false;
-    for (int j = wave; j < NREP; j += NW) {
-      const float *pml = base + (size_t)j * (HD + 2) + HD;
-      bool lost = false;
-      // the first head of this wavefront was requested above; further heads (more query heads than wavefronts) and repeated
-      // requests cost a round trip each
-      for (int it = 0;; it++) {
-        if (j != wave || it > 0) {
-#pragma unroll
-          for (int i = 0; i < MSL; i++)
-            if (i * 64 < n_active) mls[i] = ld_pair(pml, lane + i * 64);
-        }
-        if constexpr (!WORDS) break;
-        bool ok = true;
-#pragma unroll
+    if (merges) {
+      // merge.  Every thread owns two neighbouring output elements and requests their partial sums of the first MB chunks
+      // right away; while those travel, one wavefront per query head fetches the per-chunk (m, l), turns them into weights
+      // exp(m_s - M) and 1/L in LDS; then the sums are folded in chunk order.  One round trip for up to MB chunks.
+      // WORDS: a request is repeated while one of its words is still zero.  The other chunks' blocks never wait for anything
+      // before they store, and the launch keeps them all on the device, so this ends; it is bounded all the same, reports
+      // through the error word where one is given, and the result is then NaN.
+      const float *base = a.partial + (size_t)g * a.nsplit * NREP * (HD + 2);
+      constexpr int MB = 16;                       // chunks per batch of requests
+      constexpr int NPAIR = NREP * HD / 2;         // element pairs of this kv head's query heads
+      constexpr int POLL_LIMIT = 1 << 18;
+      auto pair_at = [&](const float *po, int s_) { return po + (size_t)(s_ < n_active ? s_ : n_active - 1) * NREP * (HD + 2); };
+      auto ld_pair = [&](const float *po, int s_) -> uint64_t {   // two floats of chunk s_ (8-byte aligned: HD + 2 is even)
+        return __hip_atomic_load(as_global<uint64_t>(pair_at(po, s_)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      };
+      auto clear_pair = [&](const float *po, int s_) {
+        __hip_atomic_store(as_global_mut<uint64_t>(const_cast<float *>(pair_at(po, s_))), 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      };
+      auto written = [](uint64_t w) { return (uint32_t)w != 0u && (uint32_t)(w >> 32) != 0u; };
+      auto gave_up = [&]() { if (a.err != nullptr) st_coherent(a.err, 1); };
+      const int p0 = tid < NPAIR ? tid : 0;        // threads beyond the pairs request pair 0 again (their result is not stored)
+      const int j0 = (2 * p0) / HD, d0 = (2 * p0) % HD;
+      const float *po0 = base + (size_t)j0 * (HD + 2) + d0;
+      constexpr int MSL = (CHUNK_CAP + 63) / 64;   // chunks per lane (the host keeps n_active <= CHUNK_CAP)
+      uint64_t mls[MSL];                         // wavefront j: (m, l) of this lane's chunks of head j, requested in one go
+      if (wave < NREP) {
+  #pragma unroll
         for (int i = 0; i < MSL; i++)
-          if (lane + i * 64 < n_active && !written(mls[i])) ok = false;
-        if (ok) break;
-        if (it >= POLL_LIMIT) { lost = true; gave_up(); break; }
-        __builtin_amdgcn_s_sleep(1);
+          if (i * 64 < n_active) mls[i] = ld_pair(base + (size_t)wave * (HD + 2) + HD, lane + i * 64);   // same test for the whole wavefront
       }
-      if (!asked && tid < NPAIR) {
-#pragma unroll
-        for (int u = 0; u < MB; u++) part[u] = ld_pair(po0, u);
-      }
-      asked = true;
-      if constexpr (WORDS) {
-#pragma unroll
-        for (int i = 0; i < MSL; i++)
-          if (lane + i * 64 < n_active) clear_pair(pml, lane + i * 64);
-      }
-      float M = -INFINITY;
-#pragma unroll
-      for (int i = 0; i < MSL; i++)
-        if (lane + i * 64 < n_active) M = fmaxf(M, dec((uint32_t)mls[i]));
-      M = wave_max(M);
-      float L = 0.0f;
-#pragma unroll
-      for (int i = 0; i < MSL; i++) {
-        const int s_ = lane + i * 64;
-        if (s_ < n_active) {
-          const float w = exp_f32(dec((uint32_t)mls[i]) - M);
-          sm.sc[j][s_] = w;  // n_active <= nsplit <= CHUNK_CAP
-          L = fmaf(dec((uint32_t)(mls[i] >> 32)), w, L);
-        }
-      }
-      L = wave_sum(L);
-      if (__builtin_amdgcn_ballot_w64(lost) != 0) L = __builtin_nanf("");
-      if (lane == 0) sm.l_sh[j] = 1.0f / L;  // softmax normalisation is e * (1/sum) (tensor.ts:2211-2214)
-    }
-    if (!asked && tid < NPAIR) {        // a wavefront without a query head of its own (no built shape has one that owns pairs)
-#pragma unroll
-      for (int u = 0; u < MB; u++) part[u] = ld_pair(po0, u);
-    }
-    lds_barrier();
-    auto finish = [&](int i, float O) {
-      const int j = i / HD, d = i % HD;
-      AT *dst = (AT *)a.out + (size_t)(g * NREP + j) * HD + d;
-      const float r = Act<AT>::rn(O * sm.l_sh[j]);  // the cast of the P.V result
-      if (a.out_tagged != nullptr) tw_store(a.out_tagged + (size_t)(g * NREP + j) * HD + d, a.out_tag, r);
-      else if constexpr (COHERENT) st_coherent(dst, (AT)r);
-      else *dst = (AT)r;
-    };
-    for (int p = tid; p < NPAIR; p += nthreads) {
-      const int j = (2 * p) / HD, d = (2 * p) % HD;
-      const float *po = base + (size_t)j * (HD + 2) + d;
-      float Oa = 0.0f, Ob = 0.0f;
-      for (int s0 = 0; s0 < n_active; s0 += MB) {
+      // The partial sums of this thread's first pair are asked for as soon as its wavefront has seen every chunk's (m, l)
+      // (the owners of pairs are threads of those wavefronts: NREP * HD / 128 <= NREP of them): asked for before that, the
+      // words of a chunk that is still computing come back empty and the request has to be repeated a round trip later.
+      uint64_t part[MB];
+      bool asked = false;
+      for (int j = wave; j < NREP; j += NW) {
+        const float *pml = base + (size_t)j * (HD + 2) + HD;
+        bool lost = false;
+        // the first head of this wavefront was requested above; further heads (more query heads than wavefronts) and repeated
+        // requests cost a round trip each
         for (int it = 0;; it++) {
-          if (s0 > 0 || p != tid || it > 0) {     // the first batch of the first pair is already here
-#pragma unroll
-            for (int u = 0; u < MB; u++) part[u] = ld_pair(po, s0 + u);
+          if (j != wave || it > 0) {
+  #pragma unroll
+            for (int i = 0; i < MSL; i++)
+              if (i * 64 < n_active) mls[i] = ld_pair(pml, lane + i * 64);
           }
           if constexpr (!WORDS) break;
-          // no branches from here to the sums: a chunk index past the end stands for the last chunk (ld_pair, clear_pair),
-          // whose words are checked and cleared again and enter the sum with weight zero
           bool ok = true;
-#pragma unroll
-          for (int u = 0; u < MB; u++) ok = ok & written(part[u]);
+  #pragma unroll
+          for (int i = 0; i < MSL; i++)
+            if (lane + i * 64 < n_active && !written(mls[i])) ok = false;
           if (ok) break;
-          if (it >= POLL_LIMIT) { Oa = Ob = __builtin_nanf(""); gave_up(); break; }
+          if (it >= POLL_LIMIT) { lost = true; gave_up(); break; }
           __builtin_amdgcn_s_sleep(1);
         }
+        if (!asked && tid < NPAIR) {
+  #pragma unroll
+          for (int u = 0; u < MB; u++) part[u] = ld_pair(po0, u);
+        }
+        asked = true;
         if constexpr (WORDS) {
-#pragma unroll
-          for (int u = 0; u < MB; u++) clear_pair(po, s0 + u);
+  #pragma unroll
+          for (int i = 0; i < MSL; i++)
+            if (lane + i * 64 < n_active) clear_pair(pml, lane + i * 64);
         }
-        float wgt[MB];
-#pragma unroll
-        for (int u = 0; u < MB; u++) wgt[u] = sm.sc[j][s0 + u < n_active ? s0 + u : n_active - 1];
-#pragma unroll
-        for (int u = 0; u < MB; u++) {
-          const bool in = s0 + u < n_active;
-          const float w = in ? wgt[u] : 0.0f;
-          Oa = fmaf(in ? dec((uint32_t)part[u]) : 0.0f, w, Oa);
-          Ob = fmaf(in ? dec((uint32_t)(part[u] >> 32)) : 0.0f, w, Ob);
+        float M = -INFINITY;
+  #pragma unroll
+        for (int i = 0; i < MSL; i++)
+          if (lane + i * 64 < n_active) M = fmaxf(M, dec((uint32_t)mls[i]));
+        M = wave_max(M);
+        float L = 0.0f;
+  #pragma unroll
+        for (int i = 0; i < MSL; i++) {
+          const int s_ = lane + i * 64;
+          if (s_ < n_active) {
+            const float w = exp_f32(dec((uint32_t)mls[i]) - M);
+            sm.sc[j][s_] = w;  // n_active <= nsplit <= CHUNK_CAP
+            L = fmaf(dec((uint32_t)(mls[i] >> 32)), w, L);
+          }
         }
+        L = wave_sum(L);
+        if (__builtin_amdgcn_ballot_w64(lost) != 0) L = __builtin_nanf("");
+        if (lane == 0) sm.l_sh[j] = 1.0f / L;  // softmax normalisation is e * (1/sum) (tensor.ts:2211-2214)
       }
-      finish(2 * p, Oa);
-      finish(2 * p + 1, Ob);
+      if (!asked && tid < NPAIR) {        // a wavefront without a query head of its own (no built shape has one that owns pairs)
+  #pragma unroll
+        for (int u = 0; u < MB; u++) part[u] = ld_pair(po0, u);
+      }
+      lds_barrier();
+      auto finish = [&](int i, float O) {
+        const int j = i / HD, d = i % HD;
+        AT *dst = (AT *)a.out + (size_t)(g * NREP + j) * HD + d;
+        const float r = Act<AT>::rn(O * sm.l_sh[j]);  // the cast of the P.V result
+        if (a.out_tagged != nullptr) tw_store(a.out_tagged + (size_t)(g * NREP + j) * HD + d, a.out_tag, r);
+        else if constexpr (COHERENT) st_coherent(dst, (AT)r);
+        else *dst = (AT)r;
+      };
+      for (int p = tid; p < NPAIR; p += nthreads) {
+        const int j = (2 * p) / HD, d = (2 * p) % HD;
+        const float *po = base + (size_t)j * (HD + 2) + d;
+        float Oa = 0.0f, Ob = 0.0f;
+        for (int s0 = 0; s0 < n_active; s0 += MB) {
+          for (int it = 0;; it++) {
+            if (s0 > 0 || p != tid || it > 0) {     // the first batch of the first pair is already here
+  #pragma unroll
+              for (int u = 0; u < MB; u++) part[u] = ld_pair(po, s0 + u);
+            }
+            if constexpr (!WORDS) break;
+            // no branches from here to the sums: a chunk index past the end stands for the last chunk (ld_pair, clear_pair),
+            // whose words are checked and cleared again and enter the sum with weight zero
+            bool ok = true;
+  #pragma unroll
+            for (int u = 0; u < MB; u++) ok = ok & written(part[u]);
+            if (ok) break;
+            if (it >= POLL_LIMIT) { Oa = Ob = __builtin_nanf(""); gave_up(); break; }
+            __builtin_amdgcn_s_sleep(1);
+          }
+          if constexpr (WORDS) {
+  #pragma unroll
+            for (int u = 0; u < MB; u++) clear_pair(po, s0 + u);
+          }
+          float wgt[MB];
+  #pragma unroll
+          for (int u = 0; u < MB; u++) wgt[u] = sm.sc[j][s0 + u < n_active ? s0 + u : n_active - 1];
+  #pragma unroll
+          for (int u = 0; u < MB; u++) {
+            const bool in = s0 + u < n_active;
+            const float w = in ? wgt[u] : 0.0f;
+            Oa = fmaf(in ? dec((uint32_t)part[u]) : 0.0f, w, Oa);
+            Ob = fmaf(in ? dec((uint32_t)(part[u] >> 32)) : 0.0f, w, Ob);
+          }
+        }
+        finish(2 * p, Oa);
+        finish(2 * p + 1, Ob);
+      }
     }
     then();
   }
