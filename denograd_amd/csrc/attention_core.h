@@ -186,18 +186,25 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
     for (int i = 0; i < KIT; i++) {
       if (i * NW * RPI < CH) {
         const int t = t0 + (wave + i * NW) * RPI + grp;
+        // all heads' dot products, then their sums over the lane group step by step for all heads together, then one test
+        // for the lanes that store: head by head with a test in each, every head waits out its own chain of instructions
+        float p[NREP];
 #pragma unroll
         for (int j = 0; j < NREP; j++) {
-          float p = 0.0f;
+          p[j] = 0.0f;
           if constexpr (sizeof(AT) == 2) {     // packed dot products with float accumulation (the products are exact in float)
 #pragma unroll
-            for (int e = 0; e < 4; e++) p = __builtin_amdgcn_fdot2(as_h2(qv[j][e]), as_h2(kreg[i][e]), p, false);
+            for (int e = 0; e < 4; e++) p[j] = __builtin_amdgcn_fdot2(as_h2(qv[j][e]), as_h2(kreg[i][e]), p[j], false);
           } else {
 #pragma unroll
-            for (int e = 0; e < 4; e++) p = fmaf(__uint_as_float(qv[j][e]), __uint_as_float(kreg[i][e]), p);
+            for (int e = 0; e < 4; e++) p[j] = fmaf(__uint_as_float(qv[j][e]), __uint_as_float(kreg[i][e]), p[j]);
           }
-          p = group_sum<G>(p);
-          if (sub == 0 && t < t1) sm.sc[j][t - t0] = p * a.scale;
+        }
+#pragma unroll
+        for (int j = 0; j < NREP; j++) p[j] = group_sum<G>(p[j]);
+        if (sub == 0 && t < t1) {
+#pragma unroll
+          for (int j = 0; j < NREP; j++) sm.sc[j][t - t0] = p[j] * a.scale;
         }
       }
     }
