@@ -72,12 +72,12 @@ __global__ __launch_bounds__(AW_THREADS) void attn_wo_kernel(AttnArgs at, GemvAr
     // (kv head, chunk) of block id without an integer division: the host passes ceil(65536 / n_kv_heads)
     const int split = (int)(((uint32_t)id * (uint32_t)at.kv_magic) >> 16), g = id - split * at.n_kv_heads;
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
-    A::item(at, sm, g, split, T, chunk, n_active, [&]() { if (preloaded) G::load_item(a, buf, grp, 0, 0); });
+    A::item(at, sm, g, split, T, chunk, n_active, [&]() { G::load_item(a, buf, grp, 0, 0, preloaded); });
   } else {
     // The other blocks give the items' small requests a head start before they flood the memory system with theirs; either
     // way the weights are there before the attention row is.
     __builtin_amdgcn_s_sleep(64);
-    if (preloaded) G::load_item(a, buf, grp, 0, 0);
+    G::load_item(a, buf, grp, 0, 0, preloaded);
   }
   if (wo_blk < 0) return;
   __syncthreads();   // the LDS of the attention item is done with

@@ -99,6 +99,18 @@ template <typename T> __device__ __forceinline__ const JSG_GLOBAL T *as_global(c
 template <typename T> __device__ __forceinline__ JSG_GLOBAL T *as_global_mut(void *p) { return (JSG_GLOBAL T *)(uintptr_t)p; }
 // 16 bytes that are read once: streamed past the caches
 __device__ __forceinline__ u4_t ldg_stream16(const void *p) { return __builtin_nontemporal_load(as_global<u4_t>(p)); }
+// Streaming 16-byte loads through a buffer descriptor: base + 32-bit byte offset, and an offset of BUF_END asks for
+// nothing (the load returns zeros without a memory request, and still takes its place among the outstanding loads).  A caller
+// can thus issue "the load of an item that may not exist" as straight-line code instead of a branch around it.
+constexpr uint32_t BUF_END = 0xFFFFFF00u;
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t wave_buffer(const void *p) {   // p: the same for every lane of the wavefront
+  const uint64_t v = (uint64_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return __builtin_amdgcn_make_buffer_rsrc((void *)(((uint64_t)hi << 32) | lo), 0, (int)BUF_END, 0x00020000);
+}
+__device__ __forceinline__ u4_t buf_stream16(__amdgpu_buffer_rsrc_t rs, uint32_t off) {
+  return __builtin_bit_cast(u4_t, __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, 0, 2));   // 2: nontemporal
+}
 template <typename T> __device__ __forceinline__ T ldg(const T *p) { return *as_global<T>(p); }
 
 __device__ __forceinline__ void st_coherent(float *p, float v) { __hip_atomic_store(as_global_mut<float>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }

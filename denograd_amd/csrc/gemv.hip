@@ -6,12 +6,13 @@
 namespace jsg {
 
 // fp16 activations: four blocks per CU (128 registers per lane), which the grid is sized for
-template <int KIND, typename AT, int EPI, int ROWS, int UNROLL>
+// EXACT: see Gemv::load_item; the host picks it for launches whose wavefronts walk three items or more
+template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool EXACT>
 __global__ __launch_bounds__(256, sizeof(AT) == 2 ? 4 : 1) void gemv_kernel(GemvArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   __shared__ float red[8];
   __shared__ float lut[KIND == JSGRAD_W_NF4 ? NF4_LUT_WORDS : 16];
-  typedef Gemv<KIND, AT, EPI, ROWS, UNROLL, false> G;
+  typedef Gemv<KIND, AT, EPI, ROWS, UNROLL, false, EXACT> G;
   // read the position now, not in the epilogue: the load then overlaps the weight stream instead of ending the kernel
   const int pos = EPI == EPI_ROPE_KV ? a.st[1] : 0;
   GemvBuf buf;
@@ -28,8 +29,13 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL> static int launc
   static const int per_cu = getenv("JSG_GEMV_BLOCKS_PER_CU") ? atoi(getenv("JSG_GEMV_BLOCKS_PER_CU")) : 4;
   const int cap = state().cu_count * per_cu;      // 16 resident wavefronts per CU; more rows than that are walked grid-stride
   dim3 grid(need < cap ? need : cap), block(NW * 64);
-  size_t lds = (size_t)Gemv<KIND, AT, EPI, ROWS, UNROLL, false>::x_elems(a.in_f) * sizeof(AT);
-  JSG_LAUNCH(kind, (gemv_kernel<KIND, AT, EPI, ROWS, UNROLL>), grid, block, lds, a);
+  typedef Gemv<KIND, AT, EPI, ROWS, UNROLL, false> G;
+  size_t lds = (size_t)G::x_elems(a.in_f) * sizeof(AT);
+  // items a wavefront walks: its row groups (dealt grid-stride) x the batches of a row
+  const int waves = (int)grid.x * NW;
+  const int items = ((ngroups + waves - 1) / waves) * (G::x_elems(a.in_f) / (UNROLL * G::STEP));
+  if (items >= 3) JSG_LAUNCH(kind, (gemv_kernel<KIND, AT, EPI, ROWS, UNROLL, true>), grid, block, lds, a);
+  else JSG_LAUNCH(kind, (gemv_kernel<KIND, AT, EPI, ROWS, UNROLL, false>), grid, block, lds, a);
   return 0;
 }
 // Two register buffers of UNROLL x NM x ROWS 16-byte loads each: (2 rows, 4 steps) for one matrix, (2 rows, 2 steps)

@@ -440,7 +440,7 @@ __device__ __forceinline__ void set_extra(GemvBuf &b, int r, _Float16 v) { b.ext
 // consumed, and the first item is requested before x is staged (or, with `preloaded`, before the caller even waited
 // for the previous phase), so a wavefront always has a batch of 128-bit loads in flight.
 // COHERENT: x, residual and outputs cross between blocks of the same launch.
-template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> struct Gemv {
+template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT, bool EXACT = false> struct Gemv {
   static constexpr int VEC = WFmt<KIND>::VEC;
   static constexpr int BITS = KIND == JSGRAD_W_F32 ? 32 : KIND == JSGRAD_W_F16 ? 16 : KIND == JSGRAD_W_I8 ? 8 : 4;
   static constexpr int STEP = 64 * VEC;                 // elements one wavefront covers per k-step
@@ -482,10 +482,26 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
   // measured 6 % slower).
   __device__ static __forceinline__ int first_group(int blk, int nblk) { (void)nblk; return blk * (int)(blockDim.x >> 6) + (int)(threadIdx.x >> 6); }
 
-  // issue the loads of item (grp, b)
-  __device__ static __forceinline__ void load_item(const GemvArgs &a, Buf &buf, int grp, int b, int pos) {
+  // Issue the loads of item (grp, b), if it exists.
+  // EXACT false: an item that does not exist is a branch around this function.  Where a path with requests and a path
+  // without them meet, the compiler's wait counts have to hold for both, i.e. they are those of the path WITHOUT the
+  // requests: a buffer is then waited for as if nothing had been requested after it, a wait that takes in most of the
+  // requests that were (the other buffer, just sent).  With one or two items per wavefront that costs nothing.
+  // EXACT true (launches whose wavefronts walk three items or more): straight-line code.  An item that does not exist asks
+  // for nothing through the buffer descriptor (no memory request, but its place among the outstanding loads) and reads its
+  // few scalars from a clamped, valid row; the row's scale, residual element or rotary pair are asked for with every item,
+  // not only with the last batch of a row.  Every wait is then the exact count, and two items stay in flight per
+  // wavefront; the price is the address arithmetic of up to two items that do not exist at the end of each wavefront's
+  // sequence.
+  __device__ static __forceinline__ void load_item(const GemvArgs &a, Buf &buf, int grp, int b, int pos, bool exists = true) {
+    if constexpr (!EXACT) {
+      if (!exists) return;
+    }
     const int lane = threadIdx.x & 63, in_f = a.in_f;
     const Where w = locate(a, grp);
+    __amdgpu_buffer_rsrc_t rs[NM];
+#pragma unroll
+    for (int j = 0; j < NM; j++) rs[j] = wave_buffer(wbase(a, w.m, j));
 #pragma unroll
     for (int u = 0; u < UNROLL; u++) {
       // Lanes past the end of the row reload its last vector instead of branching around the load (their x is zero,
@@ -497,12 +513,14 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
 #pragma unroll
         for (int r = 0; r < ROWS; r++) {
           const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;  // tail rows reload the last row, never stored
-          const char *p = (const char *)wbase(a, w.m, j) + (((size_t)row * in_f + (size_t)k) * BITS) / 8;
-          buf.w[wi(u, j, r)] = ldg_stream16(p);
-          if constexpr (KIND == JSGRAD_W_NF4) buf.nscale[wi(u, j, r)] = ldg((const _Float16 *)sbase(a, w.m, j) + (((size_t)row * in_f + (size_t)k) >> 6));
+          const size_t el = (size_t)row * in_f + (size_t)k;
+          buf.w[wi(u, j, r)] = buf_stream16(rs[j], (EXACT && !exists) ? BUF_END : (uint32_t)((el * BITS) / 8));
+          if constexpr (KIND == JSGRAD_W_NF4) buf.nscale[wi(u, j, r)] = ldg((const _Float16 *)sbase(a, w.m, j) + (el >> 6));
         }
     }
-    if (b != nbatch(a) - 1) return;
+    if constexpr (!EXACT) {
+      if (b != nbatch(a) - 1) return;
+    }
 #pragma unroll
     for (int r = 0; r < ROWS; r++) {
       const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;
@@ -529,7 +547,7 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
   // the first item of this wavefront, requested ahead of run()
   __device__ static __forceinline__ void prefetch(const GemvArgs &a, Buf &buf, int pos) {
     const int grp = first_group(blockIdx.x, gridDim.x);
-    if (grp < ngroups(a)) load_item(a, buf, grp, 0, pos);
+    load_item(a, buf, grp, 0, pos, grp < ngroups(a));
   }
 
   // Ask for one dword of every 128-byte line of items [first, first + DEPTH) of this wavefront's sequence without
@@ -674,7 +692,7 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
     if constexpr (EARLY_X) stage_x_issue<AT>(a, xst);
     fill_lut(lut);
     int grp = first_group(blk, nblk), b = 0;
-    if (!preloaded && grp < ng) load_item(a, bufA, grp, 0, pos);
+    if (!preloaded) load_item(a, bufA, grp, 0, pos, grp < ng);
     auto advance = [&](int &g, int &bb) {
       if (++bb == nb) { bb = 0; g += gstride; }
     };
@@ -687,9 +705,9 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
     if constexpr (EARLY_X) {
       // x is back after one round trip; its registers are free again before the second item's are needed
       stage_x_finish<AT>(a, xst, xs, red, nb * UNROLL * STEP);
-      if (gB < ng) load_item(a, bufB, gB, bB, pos);
+      load_item(a, bufB, gB, bB, pos, gB < ng);
     } else {
-      if (gB < ng) load_item(a, bufB, gB, bB, pos);
+      load_item(a, bufB, gB, bB, pos, gB < ng);
       stage_x<AT, COHERENT>(a, xs, red, nb * UNROLL * STEP);
     }
 
@@ -699,11 +717,11 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT> s
       if (gB >= ng) break;
       grp = gB; b = bB;
       advance(grp, b);                                   // the item after B goes into A
-      if (grp < ng) load_item(a, bufA, grp, b, pos);
+      load_item(a, bufA, grp, b, pos, grp < ng);
       use_item(a, bufB, gB, bB, acc, xs, lut, pos);
       gB = grp; bB = b;
       advance(gB, bB);                                   // and the one after that into B
-      if (grp < ng && gB < ng) load_item(a, bufB, gB, bB, pos);
+      load_item(a, bufB, gB, bB, pos, grp < ng && gB < ng);
     }
   }
 };
