@@ -493,8 +493,9 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT, b
   // not only with the last batch of a row.  Every wait is then the exact count, and two items stay in flight per
   // wavefront; the price is the address arithmetic of up to two items that do not exist at the end of each wavefront's
   // sequence.
-  __device__ static __forceinline__ void load_item(const GemvArgs &a, Buf &buf, int grp, int b, int pos, bool exists = true) {
-    if constexpr (!EXACT) {
+  __device__ static __forceinline__ void load_item(const GemvArgs &a, Buf &buf, int grp, int b, int pos, bool exists = true) { load_item_as<EXACT>(a, buf, grp, b, pos, exists); }
+  template <bool STRAIGHT> __device__ static __forceinline__ void load_item_as(const GemvArgs &a, Buf &buf, int grp, int b, int pos, bool exists) {
+    if constexpr (!STRAIGHT) {
       if (!exists) return;
     }
     const int lane = threadIdx.x & 63, in_f = a.in_f;
@@ -514,11 +515,11 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT, b
         for (int r = 0; r < ROWS; r++) {
           const int row = w.r0 + r < w.mrows ? w.r0 + r : w.mrows - 1;  // tail rows reload the last row, never stored
           const size_t el = (size_t)row * in_f + (size_t)k;
-          buf.w[wi(u, j, r)] = buf_stream16(rs[j], (EXACT && !exists) ? BUF_END : (uint32_t)((el * BITS) / 8));
+          buf.w[wi(u, j, r)] = buf_stream16(rs[j], (STRAIGHT && !exists) ? BUF_END : (uint32_t)((el * BITS) / 8));
           if constexpr (KIND == JSGRAD_W_NF4) buf.nscale[wi(u, j, r)] = ldg((const _Float16 *)sbase(a, w.m, j) + (el >> 6));
         }
     }
-    if constexpr (!EXACT) {
+    if constexpr (!STRAIGHT) {
       if (b != nbatch(a) - 1) return;
     }
 #pragma unroll
@@ -692,7 +693,8 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT, b
     if constexpr (EARLY_X) stage_x_issue<AT>(a, xst);
     fill_lut(lut);
     int grp = first_group(blk, nblk), b = 0;
-    if (!preloaded) load_item(a, bufA, grp, 0, pos, grp < ng);
+    // the first item is straight-line code in every launch (the staging of x below then waits for x and not for it)
+    if (!preloaded) load_item_as<true>(a, bufA, grp, 0, pos, grp < ng);
     auto advance = [&](int &g, int &bb) {
       if (++bb == nb) { bb = 0; g += gstride; }
     };
