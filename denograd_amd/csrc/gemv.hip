@@ -6,8 +6,8 @@
 namespace jsg {
 
 // fp16 activations: four blocks per CU (128 registers per lane), which the grid is sized for
-// EXACT: see Gemv::load_item; the host picks it for launches whose wavefronts walk three items or more
-template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool EXACT>
+// EXACT: see Gemv::load_item; the host picks it from the items a wavefront of the launch walks
+template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, int EXACT>
 __global__ __launch_bounds__(256, sizeof(AT) == 2 ? 4 : 1) void gemv_kernel(GemvArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   __shared__ float red[8];
@@ -33,9 +33,11 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL> static int launc
   size_t lds = (size_t)G::x_elems(a.in_f) * sizeof(AT);
   // items a wavefront walks: its row groups (dealt grid-stride) x the batches of a row
   const int waves = (int)grid.x * NW;
-  const int items = ((ngroups + waves - 1) / waves) * (G::x_elems(a.in_f) / (UNROLL * G::STEP));
-  if (items >= 3) JSG_LAUNCH(kind, (gemv_kernel<KIND, AT, EPI, ROWS, UNROLL, true>), grid, block, lds, a);
-  else JSG_LAUNCH(kind, (gemv_kernel<KIND, AT, EPI, ROWS, UNROLL, false>), grid, block, lds, a);
+  const int nbatch = G::x_elems(a.in_f) / (UNROLL * G::STEP);
+  const int items = ((ngroups + waves - 1) / waves) * nbatch;
+  if (items >= 3) JSG_LAUNCH(kind, (gemv_kernel<KIND, AT, EPI, ROWS, UNROLL, 2>), grid, block, lds, a);
+  else if (nbatch >= 2) JSG_LAUNCH(kind, (gemv_kernel<KIND, AT, EPI, ROWS, UNROLL, 1>), grid, block, lds, a);
+  else JSG_LAUNCH(kind, (gemv_kernel<KIND, AT, EPI, ROWS, UNROLL, 0>), grid, block, lds, a);
   return 0;
 }
 // Two register buffers of UNROLL x NM x ROWS 16-byte loads each: (2 rows, 4 steps) for one matrix, (2 rows, 2 steps)

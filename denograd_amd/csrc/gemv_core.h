@@ -440,7 +440,7 @@ __device__ __forceinline__ void set_extra(GemvBuf &b, int r, _Float16 v) { b.ext
 // consumed, and the first item is requested before x is staged (or, with `preloaded`, before the caller even waited
 // for the previous phase), so a wavefront always has a batch of 128-bit loads in flight.
 // COHERENT: x, residual and outputs cross between blocks of the same launch.
-template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT, bool EXACT = false> struct Gemv {
+template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT, int EXACT = 0> struct Gemv {
   static constexpr int VEC = WFmt<KIND>::VEC;
   static constexpr int BITS = KIND == JSGRAD_W_F32 ? 32 : KIND == JSGRAD_W_F16 ? 16 : KIND == JSGRAD_W_I8 ? 8 : 4;
   static constexpr int STEP = 64 * VEC;                 // elements one wavefront covers per k-step
@@ -483,17 +483,18 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT, b
   __device__ static __forceinline__ int first_group(int blk, int nblk) { (void)nblk; return blk * (int)(blockDim.x >> 6) + (int)(threadIdx.x >> 6); }
 
   // Issue the loads of item (grp, b), if it exists.
-  // EXACT false: an item that does not exist is a branch around this function.  Where a path with requests and a path
+  // Not STRAIGHT: an item that does not exist is a branch around this function.  Where a path with requests and a path
   // without them meet, the compiler's wait counts have to hold for both, i.e. they are those of the path WITHOUT the
   // requests: a buffer is then waited for as if nothing had been requested after it, a wait that takes in most of the
-  // requests that were (the other buffer, just sent).  With one or two items per wavefront that costs nothing.
-  // EXACT true (launches whose wavefronts walk three items or more): straight-line code.  An item that does not exist asks
-  // for nothing through the buffer descriptor (no memory request, but its place among the outstanding loads) and reads its
-  // few scalars from a clamped, valid row; the row's scale, residual element or rotary pair are asked for with every item,
-  // not only with the last batch of a row.  Every wait is then the exact count, and two items stay in flight per
-  // wavefront; the price is the address arithmetic of up to two items that do not exist at the end of each wavefront's
-  // sequence.
-  __device__ static __forceinline__ void load_item(const GemvArgs &a, Buf &buf, int grp, int b, int pos, bool exists = true) { load_item_as<EXACT>(a, buf, grp, b, pos, exists); }
+  // requests that were (the other buffer, just sent).
+  // STRAIGHT: straight-line code.  An item that does not exist asks for nothing through the buffer descriptor (no memory
+  // request, but its place among the outstanding loads) and reads its few scalars from a clamped, valid row; the row's
+  // scale, residual element or rotary pair are asked for with every item, not only with the last batch of a row.  Every
+  // wait after it is then the exact count; the price is the address arithmetic of an item that does not exist.
+  // Which requests are straight-line (EXACT, chosen by the host from the items a wavefront of the launch walks): the first
+  // item always; the second when every wavefront has two (EXACT >= 1); those inside the loop when it has three or more
+  // (EXACT >= 2).
+  __device__ static __forceinline__ void load_item(const GemvArgs &a, Buf &buf, int grp, int b, int pos, bool exists = true) { load_item_as<(EXACT >= 2)>(a, buf, grp, b, pos, exists); }
   template <bool STRAIGHT> __device__ static __forceinline__ void load_item_as(const GemvArgs &a, Buf &buf, int grp, int b, int pos, bool exists) {
     if constexpr (!STRAIGHT) {
       if (!exists) return;
@@ -707,9 +708,9 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT, b
     if constexpr (EARLY_X) {
       // x is back after one round trip; its registers are free again before the second item's are needed
       stage_x_finish<AT>(a, xst, xs, red, nb * UNROLL * STEP);
-      load_item(a, bufB, gB, bB, pos, gB < ng);
+      load_item_as<(EXACT >= 1)>(a, bufB, gB, bB, pos, gB < ng);
     } else {
-      load_item(a, bufB, gB, bB, pos, gB < ng);
+      load_item_as<(EXACT >= 1)>(a, bufB, gB, bB, pos, gB < ng);
       stage_x<AT, COHERENT>(a, xs, red, nb * UNROLL * STEP);
     }
 
