@@ -145,7 +145,10 @@ def make_weight(kind, out_f, in_f, dt):
 
 LINEAR_CASES = [("f32", "float32", 40, 256), ("f32", "float32", 1024, 768), ("f16", "float16", 72, 512), ("f16", "float16", 2048, 2048), ("f16", "float32", 64, 512),
                 ("i8", "float16", 100, 1024), ("i8", "float16", 4096, 4096), ("i8", "float16", 96, 14336), ("i8", "float32", 64, 256),
-                ("nf4", "float16", 64, 2048), ("nf4", "float16", 130, 4096), ("nf4", "float16", 48, 64)]
+                ("nf4", "float16", 64, 2048), ("nf4", "float16", 130, 4096), ("nf4", "float16", 48, 64),
+                # the three ways a launch requests its items (by the items a wavefront walks): two batches of one row pair,
+                # three row pairs per wavefront of a full grid with a ragged end, and (above: 96 x 14336) four batches
+                ("f16", "float16", 256, 4096), ("f16", "float16", 20000, 512)]
 
 
 @pytest.mark.parametrize("kind,dt,out_f,in_f", LINEAR_CASES)
