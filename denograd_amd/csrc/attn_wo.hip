@@ -162,6 +162,7 @@ static int attn_wo_impl(const void *q, const void *cache_k, const void *cache_v,
   JSG_REQUIRE(layer >= 0 && layer < 128, "jsgrad_hip_attn_wo: layer index %d", layer);
   const int qdim = n_heads * head_dim;
   JSG_REQUIRE(dim > 0 && dim % 2 == 0 && qdim % 16 == 0 && (size_t)qdim * 2 <= 64 * 1024, "jsgrad_hip_attn_wo: dim %d / n_heads*head_dim %d", dim, qdim);
+  JSG_REQUIRE(fits_buffer_offsets((size_t)dim, (size_t)qdim, 16), "jsgrad_hip_attn_wo: wo of %d x %d elements reaches 4 GiB (32-bit byte offsets)", dim, qdim);
   char *ws = (char *)workspace;
   AttnArgs at;
   at.q = q; at.cache_k = cache_k; at.cache_v = cache_v; at.st = st; at.out = nullptr;

@@ -103,6 +103,8 @@ __device__ __forceinline__ u4_t ldg_stream16(const void *p) { return __builtin_n
 // nothing (the load returns zeros without a memory request, and still takes its place among the outstanding loads).  A caller
 // can thus issue "the load of an item that may not exist" as straight-line code instead of a branch around it.
 constexpr uint32_t BUF_END = 0xFFFFFF00u;
+// host side: a matrix read this way must end below BUF_END
+inline bool fits_buffer_offsets(size_t rows, size_t row_elems, int bits) { return rows * row_elems * (size_t)bits / 8 < (size_t)BUF_END; }
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t wave_buffer(const void *p) {   // p: the same for every lane of the wavefront
   const uint64_t v = (uint64_t)p;
   const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));

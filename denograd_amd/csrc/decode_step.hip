@@ -311,6 +311,8 @@ int jsgrad_hip_decode_step(const jsgrad_hip_step_t *d) {
   JSG_REQUIRE(d->dim % vec == 0 && d->hidden % vec == 0 && (d->n_heads * d->head_dim) % vec == 0, "jsgrad_hip_decode_step: feature sizes must be multiples of %d", vec);
   JSG_REQUIRE(d->dim <= 4 * STEP_THREADS * 8, "jsgrad_hip_decode_step: dim %d exceeds the fused RMSNorm limit", d->dim);
   JSG_REQUIRE(d->kind == JSGRAD_W_F16 || d->out_s, "jsgrad_hip_decode_step: quantised lm_head needs a scale");
+  JSG_REQUIRE(fits_buffer_offsets((size_t)d->vocab, (size_t)d->dim, 16) && fits_buffer_offsets((size_t)d->hidden, (size_t)d->dim, 16),
+              "jsgrad_hip_decode_step: a weight matrix reaches 4 GiB (32-bit byte offsets)");
   const int nsplit = 64;
   JSG_REQUIRE(d->max_context <= nsplit * ATT_CHUNK_MAX, "jsgrad_hip_decode_step: max_context %d exceeds %d", d->max_context, nsplit * ATT_CHUNK_MAX);
   const int feat = d->hidden > d->dim ? d->hidden : d->dim;

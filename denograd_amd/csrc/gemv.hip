@@ -30,6 +30,8 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL> static int launc
   const int cap = state().cu_count * per_cu;      // 16 resident wavefronts per CU; more rows than that are walked grid-stride
   dim3 grid(need < cap ? need : cap), block(NW * 64);
   typedef Gemv<KIND, AT, EPI, ROWS, UNROLL, false> G;
+  const int most_rows = a.rows0 > a.rows1 ? (a.rows0 > a.rows2 ? a.rows0 : a.rows2) : (a.rows1 > a.rows2 ? a.rows1 : a.rows2);
+  JSG_REQUIRE(fits_buffer_offsets((size_t)most_rows, (size_t)a.in_f, G::BITS), "one-row Linear: a weight matrix of %d x %d elements reaches 4 GiB (32-bit byte offsets)", most_rows, a.in_f);
   size_t lds = (size_t)G::x_elems(a.in_f) * sizeof(AT);
   // items a wavefront walks: its row groups (dealt grid-stride) x the batches of a row
   const int waves = (int)grid.x * NW;

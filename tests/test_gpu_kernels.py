@@ -187,6 +187,9 @@ def test_linear_rejects_bad_shapes(hip):
         check(hip.jsgrad_hip_linear(ffi.W_I8, w.ptr, y.ptr, 8, 100, x.ptr, y.ptr, None, 0.0, None, ffi.F16))
     with pytest.raises(ffi.HipError, match="needs a scale"):
         check(hip.jsgrad_hip_linear(ffi.W_I8, w.ptr, None, 8, 96, x.ptr, y.ptr, None, 0.0, None, ffi.F16))
+    # the weights are read through 32-bit byte offsets: a matrix of 4 GiB or more is refused before anything is launched
+    with pytest.raises(ffi.HipError, match="4 GiB"):
+        check(hip.jsgrad_hip_linear(ffi.W_F32, w.ptr, None, 70000, 16384, x.ptr, y.ptr, None, 0.0, None, ffi.F32))
 
 
 @pytest.mark.parametrize("dt", ["float32", "float16"])
