@@ -129,7 +129,9 @@ int jsgrad_hip_rmsnorm(const void *x, const void *weight, void *y, int dim, floa
 /* Linear.call / Int8Linear.call / NF4Linear.call on one row (nn/index.ts:411, llama3.ts:35,91-97):
  * y[out_f] = x[in_f] . W^T, float accumulation, result in the activation dtype.
  * norm_weight != NULL fuses RMSNorm(x) in front (TransformerBlock.call, models/llama.ts:125-126);
- * residual != NULL adds it after the cast: y = residual + linear (the `x.add(...)` of llama.ts:125-126). */
+ * residual != NULL adds it after the cast: y = residual + linear (the `x.add(...)` of llama.ts:125-126).
+ * The one-row launches (this one, _qkv_rope, _ffn_gate, _attn_wo, _decode_step) address a weight matrix with 32-bit byte
+ * offsets: a matrix of 4 GiB or more is refused. */
 int jsgrad_hip_linear(int kind, const void *w, const void *scale, int out_f, int in_f, const void *x, void *y,
                       const void *norm_weight, float eps, const void *residual, int act);
 
