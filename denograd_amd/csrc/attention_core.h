@@ -140,6 +140,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
     const size_t row_stride = (size_t)a.n_kv_heads * HD;
     const AT *kbase = (const AT *)a.cache_k + (size_t)g * HD + (size_t)sub * EPL;
     const AT *vbase = (const AT *)a.cache_v + (size_t)g * HD;
+    JSG_LSTAMP(10);
 
     // ---- every request of the item goes out now: the query rows (once per block, 16-byte pieces), then this lane's K rows,
     // then its V dwords.  They come back in that order.
@@ -179,6 +180,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
     // ---- phase 1: scores of the chunk.  The query rows are here first: publish them, take this lane's slice.
     if (tid < QCH) ((u4_t *)sm.qs)[tid] = qpiece;
     lds_barrier();
+    JSG_LSTAMP(11);
     u4_t qv[NREP];
 #pragma unroll
     for (int j = 0; j < NREP; j++) qv[j] = ((const u4_t *)sm.qs)[j * G + sub];
@@ -209,6 +211,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       }
     }
     lds_barrier();
+    JSG_LSTAMP(12);
     // Wavefront j does the whole softmax of head j by itself - maximum, exp, sum - with no barrier in between: lane i holds
     // rows i, i + 64, ... of the chunk.
     for (int j = wave; j < NREP; j += NW) {
@@ -236,6 +239,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       if (lane == 0) { sm.m_sh[j] = m; sm.l_sh[j] = l; }
     }
     lds_barrier();
+    JSG_LSTAMP(13);
 
     // ---- phase 2: o[j][d] = sum_t p[j][t] * V[t][d] over the rows of this wavefront; this lane's elements are
     // d = (vcol + LPR * part) * EP + e
@@ -300,6 +304,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
           for (int e = 0; e < EP; e++) sm.o_part[wave][j][(vcol + LPR * c) * EP + e] = of[j][c][e];
     }
     lds_barrier();
+    JSG_LSTAMP(14);
     constexpr int SLOTS = NW;
     // ---- hand-over of the chunk's partial result.
     // WORDS (kernels whose launch is the whole life of the workspace contents, COHERENT false): every 32-bit word says by
@@ -324,6 +329,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       st_coherent(&mine[tid * (HD + 2) + HD], enc(sm.m_sh[tid]));
       st_coherent(&mine[tid * (HD + 2) + HD + 1], enc(sm.l_sh[tid]));
     }
+    JSG_LSTAMP(15);
     // One way through for every block: the block of chunk 0 merges, then every block calls `then`.  (With an early exit
     // for the others, the compiler placed their `then` in front of the merge and made the merging block wait for its own
     // stores, as if they were `then`'s requests, before it could ask for anybody's results.)
@@ -408,6 +414,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
           for (int u = 0; u < MB; u++) part[u] = ld_pair(po0, u);
         }
         asked = true;
+        JSG_LSTAMP(16);
         if constexpr (WORDS) {
   #pragma unroll
           for (int i = 0; i < MSL; i++)
@@ -437,6 +444,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
         for (int u = 0; u < MB; u++) part[u] = ld_pair(po0, u);
       }
       lds_barrier();
+      JSG_LSTAMP(17);
       auto finish = [&](int i, float O) {
         const int j = i / HD, d = i % HD;
         AT *dst = (AT *)a.out + (size_t)(g * NREP + j) * HD + d;
@@ -483,6 +491,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
         finish(2 * p, Oa);
         finish(2 * p + 1, Ob);
       }
+      JSG_LSTAMP(18);
     }
     then();
   }

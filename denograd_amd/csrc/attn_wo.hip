@@ -41,7 +41,9 @@ __global__ __launch_bounds__(AW_THREADS) void attn_wo_kernel(AttnArgs at, GemvAr
   // The position first, and nothing else until it is here: a small request issued into an idle memory system is back in a
   // fraction of a microsecond, behind the bursts of weight requests of all blocks it takes several times as long, and every
   // later step of the attention items hangs on it.
+  JSG_LCLEAR();
   const int pos = at.st[1];
+  JSG_LSTAMP(0);
   const uint32_t tag = tw_tag(pos * 128 + layer);   // the version of this launch: no other launch that writes the same tagged
   at.out_tag = tag;                                 // row has it (another layer, or another position of the same layer)
   a.x_tag = tag;
@@ -79,10 +81,15 @@ __global__ __launch_bounds__(AW_THREADS) void attn_wo_kernel(AttnArgs at, GemvAr
     __builtin_amdgcn_s_sleep(64);
     G::load_item(a, buf, grp, 0, 0, preloaded);
   }
-  if (wo_blk < 0) return;
-  __syncthreads();   // the LDS of the attention item is done with
-  G::run(a, (AT *)smem, red, lut, buf, preloaded, 0, wo_blk, wo_nblk);
+  JSG_LSTAMP(1);
+  if (wo_blk >= 0) {
+    __syncthreads();   // the LDS of the attention item is done with
+    G::run(a, (AT *)smem, red, lut, buf, preloaded, 0, wo_blk, wo_nblk);
+    JSG_LSTAMP(21);
+  }
+  JSG_LFLUSH(blockIdx.x == 0 ? 0 : (blockIdx.x == (unsigned)at.n_kv_heads ? 1 : (blockIdx.x == gridDim.x - 1 ? 2 : -1)));
 }
+JSG_TRACE_ENTRY(jsgrad_hip_attn_wo_trace)
 
 static int aw_nsplit(int max_context) { return att_max_chunks(max_context, AW_CHUNK_CAP); }
 

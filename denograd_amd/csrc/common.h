@@ -196,6 +196,12 @@ __device__ __forceinline__ void trace_stamp(int row, int slot) {
 }
 #define JSG_STAMP(slot) jsg::trace_stamp(jsg::trace_row(), slot)
 #define JSG_STAMP_ROW(row, slot) jsg::trace_stamp(row, slot)
+// The same stamps kept in LDS and copied out when the block ends: a stamp written to memory is a store, and the next wait for
+// a load waits for it too, which stretches whatever follows it.  JSG_LCLEAR() first, JSG_LFLUSH(row) last (both block-wide).
+static __shared__ unsigned long long jsg_tl[32];
+#define JSG_LSTAMP(slot) do { if (threadIdx.x == 0) jsg::jsg_tl[slot] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#define JSG_LCLEAR() do { if (threadIdx.x < 32) jsg::jsg_tl[threadIdx.x] = 0; __syncthreads(); } while (0)
+#define JSG_LFLUSH(row) do { __syncthreads(); const int row_ = (row); if (row_ >= 0 && threadIdx.x < 32) jsg::g_trace[row_][threadIdx.x] = jsg::jsg_tl[threadIdx.x]; } while (0)
 #define JSG_TRACE_ENTRY(name)                                                                              \
   extern "C" int name(unsigned long long *host_out) {                                                      \
     JSG_HIP(hipStreamSynchronize(jsg::state().stream));                                                    \
@@ -207,6 +213,9 @@ __device__ __forceinline__ void trace_stamp(int row, int slot) {
 #else
 #define JSG_STAMP(slot) ((void)0)
 #define JSG_STAMP_ROW(row, slot) ((void)0)
+#define JSG_LSTAMP(slot) ((void)0)
+#define JSG_LCLEAR() ((void)0)
+#define JSG_LFLUSH(row) ((void)0)
 #define JSG_TRACE_ENTRY(name)
 #endif
 

@@ -218,9 +218,9 @@ template <typename AT, bool COHERENT> __device__ __forceinline__ void stage_x(co
           __builtin_amdgcn_s_sleep(8);
         }
       }
-      JSG_STAMP(2);
+      JSG_LSTAMP(2);
       lds_barrier();   // only "the probe is through": requests of this wavefront that are in flight stay in flight
-      JSG_STAMP(3);
+      JSG_LSTAMP(3);
       // all chunks of a thread are asked for together, again and again until every one carries the tag: one round trip
       // when the row is there, instead of one per chunk
       constexpr int NCH = 2;
@@ -263,7 +263,7 @@ template <typename AT, bool COHERENT> __device__ __forceinline__ void stage_x(co
       for (int c = tid; c < nchunks; c += nt) xl[c] = ldx(c);
     }
     __syncthreads();
-    JSG_STAMP(4);
+    JSG_LSTAMP(4);
     return;
   }
   const u4_t *wg = (const u4_t *)a.norm_w;

@@ -387,6 +387,15 @@ static int g_threads = 1;
 /* Threads for the loops over independent outputs (rows of a Linear, heads of the attention).  1 = the reference's way. */
 void or_set_threads(int n) { g_threads = n < 1 ? 1 : n; }
 
+/* The order in which a one-row Linear adds its products is not fixed by anything this file can check (see "parity
+ * unpinned" at the top).  0 (the default) is the restatement's reading of the reference: one accumulator, sequential over
+ * the reduce axis.  1 is another legitimate order of the SAME products: eight interleaved accumulators (element k goes to
+ * accumulator k % 8) added pairwise at the end, the shape a vectorised loop has.  It exists so that tests can measure how
+ * far two float summation orders drift apart through a deep model, and hold the HIP path (whose order is a third one:
+ * lanes, then a tree) to that yardstick; it is never the reference arithmetic. */
+static int g_sum_order = 0;
+void or_set_sum_order(int mode) { g_sum_order = mode ? 1 : 0; }
+
 /* one weight row as the floats the products use: W[o][k] as stored, code*scale, or RN16(code*scale) */
 static void weight_row(const or_linear_t *L, int o, int materialised, const float *code, float *wrow) {
   const int in_f = L->in_f;
@@ -418,6 +427,21 @@ void or_linear_ex(const or_linear_t *L, const float *x, float *y, int act16, int
   const int in_f = L->in_f;
   float code[16];
   or_nf4_code(code);
+  if (g_sum_order == 1) {
+#pragma omp parallel num_threads(g_threads) if (g_threads > 1)
+    {
+      float *wrow = (float *)malloc(sizeof(float) * (size_t)in_f);
+#pragma omp for schedule(static)
+      for (int o = 0; o < L->out_f; o++) {
+        weight_row(L, o, materialised, code, wrow);
+        float a[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        for (int k = 0; k < in_f; k++) a[k & 7] = a[k & 7] + x[k] * wrow[k];
+        y[o] = rn_act(((a[0] + a[1]) + (a[2] + a[3])) + ((a[4] + a[5]) + (a[6] + a[7])), act16);
+      }
+      free(wrow);
+    }
+    return;
+  }
 #pragma omp parallel for schedule(static) num_threads(g_threads) if (g_threads > 1)
   for (int o = 0; o < L->out_f; o++) {
     float acc = 0.0f;

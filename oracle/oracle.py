@@ -53,6 +53,7 @@ def lib() -> C.CDLL:
             "or_linear_call": ([i32, i32, i32, vp, vp, vp, i32, vp, i32], None),
             "or_linear_call_rowwise": ([i32, i32, i32, vp, vp, vp, i32, vp, i32], None),
             "or_set_threads": ([i32], None),
+            "or_set_sum_order": ([i32], None),
             "or_rmsnorm": ([vp, vp, i32, f32, i32, vp], None),
             "or_rope": ([vp, i32, i32, vp, i32], None),
             "or_argmax": ([vp, i32], i32),
@@ -171,6 +172,13 @@ def set_threads(n: int) -> None:
     """Threads for loops over independent outputs (1 = single-threaded like the reference's CLANG device, the default).
     Results do not depend on it."""
     lib().or_set_threads(int(n))
+
+
+def set_sum_order(mode: int) -> None:
+    """0: the restatement's order of a one-row Linear's sum (one accumulator, sequential); 1: the same products in
+    eight interleaved accumulators added pairwise.  A yardstick for tests (how far two float summation orders drift
+    apart through a deep model), never the reference arithmetic."""
+    lib().or_set_sum_order(int(mode))
 
 
 def linear(w, scale, x, out_f: int, in_f: int, act16: bool, rowwise: bool = False) -> np.ndarray:

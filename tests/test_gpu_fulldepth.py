@@ -1,0 +1,86 @@
+"""Greedy decoding at FULL depth: the Llama-3.1-8B-shaped int8 model with all 32 layers and the Llama-3.2-1B-shaped fp16
+model with all 16 layers (shapes: /root/reference/jsgrad/models/llama3.ts:119-132), random-init weights made and quantised on
+the device and copied to the host for the CPU oracle, so both sides hold the same codes and scales.
+
+An 8-token prompt, then 32 greedy steps (/root/reference/jsgrad/models/llama.ts:210-212 with temperature 0).  Every step feeds
+both sides the oracle's previous token, so one differing pick cannot hide what comes after it.
+
+What can hold at this depth, and what is asserted.  Two correct fp16 implementations whose float sums associate differently
+do not stay within a last-bit of each other through 16 or 32 layers: a last-bit difference in one activation moves every
+output of the next Linear a little, which flips further roundings, and the difference grows like a random walk with depth
+(tests/test_oracle_model.py shows it on the oracle alone, orc.set_sum_order).  At 32 layers the r.m.s. of that difference is
+0.5-0.7 % of the logits' r.m.s., which is the size of the rtol/atol 1e-2 allowance itself for the many logits near zero: the
+first entries pass it from about 8 layers on, several per cent of them at 32.  So the bars here are:
+  * the device is no further from the oracle than the oracle's own second summation order is (r.m.s. over all logits, with a
+    factor of 2 for the spread between positions): the deviation is summation noise, not an error;
+  * r.m.s. deviation below 1e-2 of the logits' r.m.s., no entry further out than 6x the rtol/atol 1e-2 allowance (the share
+    of entries outside the allowance is printed; it is what a deviation of that r.m.s. implies);
+  * the device's token is the oracle's, or the oracle's own logits of the two tokens lie closer than twice the largest
+    deviation measured at that position (a pick the noise can decide); such positions are counted and printed.
+The 2-layer models at the same widths (tests/test_gpu_fullshape.py) and the five small models (tests/test_gpu_model.py) hold
+the strict bars: every logit within rtol/atol 1e-2, tokens identical or inside a 2-ulp tie."""
+import os
+import time
+
+import numpy as np
+import pytest
+
+import oracle as orc
+from denograd_amd import synthetic
+from denograd_amd.llama3 import Llama3
+from denograd_amd.state import get_state_dict
+
+pytestmark = pytest.mark.gpu
+THREADS = min(16, os.cpu_count() or 1)
+N_PROMPT, N_STEPS, N_YARD = 8, 32, 10
+
+
+@pytest.mark.parametrize("name,layers", [("8B-int8", 32), ("1B", 16)])
+def test_greedy_tokens_at_full_depth(name, layers):
+    cfg = synthetic.config(name, max_context=N_PROMPT + N_STEPS + 8)
+    assert cfg["n_layers"] == layers
+    t0 = time.perf_counter()
+    gpu = Llama3.from_config(cfg).random_init(seed=11, tied=cfg["tied"])
+    sd = {k: v.numpy() for k, v in get_state_dict(gpu.model).items()}
+    cpu, yard = orc.OracleModel(cfg, sd), orc.OracleModel(cfg, sd)
+    orc.set_threads(THREADS)     # independent outputs split among threads; results do not depend on the count
+    try:
+        prompt = [int(t) for t in synthetic.random_prompt(cfg, N_PROMPT, seed=21)]
+        t_build = time.perf_counter() - t0
+        tok, picks, outside, worst = None, [], 0, 0.0
+        dev2 = yard2 = ref2 = 0.0          # sums of squares over the positions the yardstick also ran
+        dev2_all = ref2_all = 0.0
+        for pos in range(N_PROMPT + N_STEPS - 1):
+            t = prompt[pos] if pos < N_PROMPT else tok
+            tok_c, lg_c = cpu.forward([t], pos)
+            tok_g = gpu._call(t); gpu.start_pos += 1        # eager at position 0, captured at 1, replayed from 2 on
+            lg_g = gpu.model.logits.numpy().astype(np.float32)
+            d = np.abs(lg_g - lg_c)
+            ratio = d / (1e-2 + 1e-2 * np.abs(lg_c))
+            worst = max(worst, float(ratio.max()))
+            outside += int(np.sum(ratio > 1.0))
+            dev2_all += float(np.sum(d * d)); ref2_all += float(np.sum(lg_c * lg_c))
+            if pos < N_YARD:       # the oracle's second summation order on the same inputs
+                orc.set_sum_order(1)
+                _, lg_y = yard.forward([t], pos)
+                orc.set_sum_order(0)
+                dev2 += float(np.sum(d * d)); yard2 += float(np.sum((lg_y - lg_c) ** 2)); ref2 += float(np.sum(lg_c * lg_c))
+            if pos >= N_PROMPT - 1:      # a generated position
+                gap = float(lg_c[tok_c] - lg_c[tok_g])
+                assert tok_g == tok_c or 0 <= gap <= 2 * float(d.max()), \
+                    f"{name} position {pos}: token {tok_g} != {tok_c}, oracle gap {gap:.4f} against a largest deviation of {d.max():.4f}"
+                picks.append(tok_g == tok_c)
+            tok = tok_c
+        n_logits = (N_PROMPT + N_STEPS - 1) * cfg["vocab_size"]
+        rel, rel_dev, rel_yard = np.sqrt(dev2_all / ref2_all), np.sqrt(dev2 / ref2), np.sqrt(yard2 / ref2)
+        print(f"{name}, {layers} layers: {sum(picks)} of {len(picks)} greedy picks identical"
+              f"{' (the free-running sequences are the same)' if all(picks) else ', the others decided inside the deviation'}; "
+              f"r.m.s. deviation {rel:.2e} of the logits' r.m.s. (first {N_YARD} positions: device {rel_dev:.2e}, the oracle's second summation order {rel_yard:.2e}); "
+              f"{100.0 * outside / n_logits:.2f} % of {n_logits} logits outside rtol/atol 1e-2, the worst by {worst:.2f}x; build {t_build:.1f}s, total {time.perf_counter() - t0:.1f}s")
+        assert gpu.model.attn_wo_error() == 0
+        assert rel_dev <= 2.0 * rel_yard, f"{name}: device {rel_dev:.2e} from the oracle, the oracle's second summation order only {rel_yard:.2e}"
+        assert rel <= 1e-2 and worst <= 6.0 and outside <= 0.2 * n_logits
+        assert sum(picks) >= len(picks) - 6
+    finally:
+        orc.set_sum_order(0)
+        orc.set_threads(1)

@@ -152,6 +152,38 @@ def test_8b_int8_one_pass_over_512_positions_of_two_sequences():
     cpu.set_batched(False)
 
 
+def test_8b_int8_one_pass_at_config_5_size():
+    """BASELINE config 5's prefill at its real size: tokens [16, 2048] from position 0 in ONE pass (32768 rows through the tiled
+    MFMA GEMMs at K = 4096 / 14336, causal attention over 2048 keys of 16 sequences).  The oracle's several-row forward is run
+    for the first and the last sequence (the two ends of the row space): last-position logits within rtol/atol 1e-2, the token
+    rule of check_token, and the new cache rows of both layers on a sample of positions that includes both ends."""
+    name = "8B-int8"
+    cfg, gpu, cpu, _ = build(name)
+    B, S = 16, 2048
+    assert cfg["max_context"] >= S
+    cpu.set_batched(True)
+    for layer in gpu.model.layers:
+        layer.attention._ensure_cache("float16", gpu.device, B)
+    prompts = np.stack([synthetic.random_prompt(cfg, S, seed=300 + b) for b in range(B)]).astype(np.int32)
+    tok = gpu.model.forward_rows(prompts, 0).numpy()
+    lg = gpu.model.rows_logits().numpy().astype(np.float32)
+    sample = np.unique(np.concatenate([np.arange(4), np.arange(S - 4, S), np.random.default_rng(5).integers(0, S, 56)]))
+    worst = 0.0
+    for b in (0, B - 1):
+        rows = [layer.attention.cache_kv.numpy()[:, b, :S].astype(np.float32) for layer in gpu.model.layers]     # [2, S, KV, hd] per layer
+        cpu.reset()
+        tok_c, lg_c = cpu.forward(prompts[b], 0)
+        r = ratio(lg[b], lg_c)
+        worst = max(worst, r)
+        assert r <= 1.0, f"sequence {b}: prefill logits {r:.3f} of the 1e-2 budget"
+        check_token(int(tok[b]), tok_c, lg_c, f"sequence {b}")
+        for l in range(cfg["n_layers"]):
+            assert np.allclose(rows[l][0][sample], cpu.cache_k[l, :S][sample], rtol=1e-2, atol=1e-2), (b, l)
+            assert np.allclose(rows[l][1][sample], cpu.cache_v[l, :S][sample], rtol=1e-2, atol=1e-2), (b, l)
+    cpu.set_batched(False)
+    print(f"one pass of 16 x 2048: worst logit ratio {worst:.3f} of the 1e-2 budget")
+
+
 def test_8b_int8_batched_decode_step_of_16_sequences():
     """BASELINE config 5's decode shape: one position for each of 16 sequences at 2112 visible positions (the few-row
     weight-streaming GEMM, batched decode attention), against the oracle run per sequence with `batched` set."""

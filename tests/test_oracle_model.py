@@ -89,3 +89,32 @@ def test_embedding_is_row_gather():
     cfg2 = small_cfg("float32", None)
     sd2 = make(cfg2)
     assert np.array_equal(orc.OracleModel(cfg2, sd2).embed(5), sd2["tok_embeddings.weight"][5])
+
+
+def test_summation_order_alone_moves_deep_models_by_more_than_an_ulp():
+    """What the order of a float sum is worth at depth.  The same fp16 model, the same products, two orders of adding them in
+    the one-row Linear (orc.set_sum_order): after two layers the logits differ in the last fp16 bits, and the difference
+    grows with depth like a random walk, because a last-bit change of one activation moves every output of the next Linear
+    a little, which flips further roundings.  Any implementation whose sums associate differently from the reference's
+    (every parallel one) sits at this distance from it: the yardstick for the full-depth comparison of the HIP path."""
+    rms = {}
+    for L in (2, 8, 32):
+        cfg = small_cfg("float16", "float16", dim=256, hidden_dim=768, n_layers=L, vocab_size=1024, max_context=16)
+        sd = synthetic.random_state_dict(cfg, seed=4, std=0.02)
+        toks = synthetic.random_prompt(cfg, 8, seed=6)
+        a, b = orc.OracleModel(cfg, sd), orc.OracleModel(cfg, sd)
+        d2, n = 0.0, 0
+        try:
+            for i, t in enumerate(toks):
+                orc.set_sum_order(0)
+                _, lg0 = a.forward([t], i)
+                orc.set_sum_order(1)
+                _, lg1 = b.forward([t], i)
+                d2 += float(np.sum((lg1 - lg0) ** 2)); n += lg0.size
+                scale = float(np.sqrt(np.mean(lg0 ** 2)))
+        finally:
+            orc.set_sum_order(0)
+        rms[L] = np.sqrt(d2 / n) / scale
+    assert 0 < rms[2] < rms[8] < rms[32], rms
+    assert rms[2] < 2e-3 and rms[32] < 2e-2, rms            # still small against the 1e-2 budget, but not last-bit any more
+    assert 1.5 < rms[32] / rms[2] < 16, rms                 # grows with depth, roughly like its square root (x4 for x16 layers)
