@@ -28,15 +28,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the `linear` kernel family (average over wo, w2 and the lm_head of one step), from two
-# `rocprofv3 --pmc` runs of `bench.py --traffic-probe` (FETCH_SIZE, then WRITE_SIZE), each scaled by what the counter
-# reads for the 512 MiB copy in the same run (factors 2.000 and 1.000).  Counters cannot be read from inside this process.
-# HBM bytes per launch of the dominant kernel family from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised under
-# profiles/ (average over the launches of one step).  "linear" is w2 + lm_head when attention and wo share a launch
-# (the default for fp16 activations), else wo + w2 + lm_head.
-MEASURED_TRAFFIC = {("1B", "linear", True): 62.77e6, ("8B-int8", "linear", True): 73.46e6,
-                    ("1B", "ffn_gate", True): 67.31e6, ("8B-int8", "ffn_gate", True): 118.22e6,
-                    ("1B", "linear", False): 36.49e6, ("8B-int8", "linear", False): 45.72e6}
+# `roofline.traffic` (HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counters) cannot be read from inside this process:
+# it is null here, and the counter runs of `bench.py --traffic-probe` under rocprofv3 are summarised under profiles/.
 
 
 def log(*a):
@@ -276,7 +269,7 @@ def run_workload(name, prompt_len, steps, warmup, profile_steps=8, use_graph=Tru
                 "attn_wo": "attn_wo_kernel (decode attention + wo + residual)", "attn_decode": "attn_decode_kernel"}[dom]
         achieved = fam[dom]["GBps"]
         roof = {"bound": "hbm", "kernel": kern, "family": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get((name, dom, "attn_wo" in fam)),
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                 "bytes_per_launch": int(kb[dom] / fam[dom]["launches_per_step"]), "avg_us_per_launch": round(fam[dom]["avg_us_per_launch"], 2),
                 "ms_per_step": round(fam[dom]["ms_per_step"], 4),
                 # the same launches as read-only kernels of the same sizes: the rate a launch of this size can reach at all

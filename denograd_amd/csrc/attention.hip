@@ -98,11 +98,23 @@ template <int HD> static int launch_attn_stream(const AttnArgs &a, int n_rep, in
 constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)8 << 20;
 static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
 constexpr int NOALLOC_MAX_DEVICES = 64;
-static void *g_scratch_ptr[NOALLOC_MAX_DEVICES];   // per device, set on the first call there
+static void *g_scratch_ptr[NOALLOC_MAX_DEVICES];   // per device, set by jsgrad_hip_init there (attn_static_init)
 
-// the part of the workspace a call uses must start at zero (a zero word means `partial result not written yet`) whatever an
+// The device address of the built-in workspace on the current device; called by jsgrad_hip_init with that device current, so
+// that no later call (one under graph capture, say) has to resolve a symbol.
+int attn_static_init(int dev) {
+  JSG_REQUIRE(dev >= 0 && dev < NOALLOC_MAX_DEVICES, "jsgrad_hip_init: device %d beyond the %d the built-in attention workspace is kept for", dev, NOALLOC_MAX_DEVICES);
+  if (g_scratch_ptr[dev] != nullptr) return 0;
+  void *p = nullptr;
+  JSG_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+  JSG_REQUIRE(p != nullptr, "jsgrad_hip_init: no device address for the built-in attention workspace");
+  g_scratch_ptr[dev] = p;
+  return 0;
+}
+
+// the partial results a call uses must start at zero (a zero word means `partial result not written yet`) whatever an
 // earlier call left behind, one that gave up waiting included (a fill kernel, not a memset node: callers may be capturing a
-// graph)
+// graph).  The first 256 bytes are not touched: the error word there stays set until it is read.
 __global__ void zero_words_kernel(int *p, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = 0;
@@ -149,30 +161,72 @@ int jsgrad_hip_attn_decode_batch(const void *q, const void *cache_k, const void 
 
 size_t jsgrad_hip_attn_decode_static_max_bytes(void) { return NOALLOC_SCRATCH_BYTES; }
 
+static int attn_decode_check(const char *who, int n_heads, int n_kv_heads, int head_dim, int max_context, int act) {
+  JSG_REQUIRE(act == JSGRAD_F16 || act == JSGRAD_F32, "%s: unknown activation dtype %d", who, act);
+  JSG_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_kv_heads <= 64 && n_heads % n_kv_heads == 0, "%s: n_heads %d / n_kv_heads %d", who, n_heads, n_kv_heads);
+  JSG_REQUIRE(head_dim == 64 || head_dim == 128, "%s: head_dim %d (64 and 128 are built)", who, head_dim);
+  JSG_REQUIRE(max_context > 0 && max_context <= 256 * ATT_CHUNK_MAX, "%s: max_context %d exceeds %d", who, max_context, 256 * ATT_CHUNK_MAX);
+  const int n_rep = n_heads / n_kv_heads;
+  JSG_REQUIRE(n_rep <= 4 || n_rep == 8, "%s: n_heads/n_kv_heads = %d is not one of 1,2,3,4,8", who, n_rep);
+  // The blocks of chunk 0 (the first n_kv_heads of the grid) wait on the device for the other chunks' partial results.
+  // Those other blocks wait for nobody, so the launch finishes as long as the waiting blocks leave room on the device for
+  // at least one of them; the device is required to have more compute units than there are waiting blocks.
+  JSG_REQUIRE(n_kv_heads < state().cu_count, "%s: %d kv heads but only %d compute units", who, n_kv_heads, state().cu_count);
+  return 0;
+}
+
+static int read_error_word(const char *who, void *word, int *host_out_error) {
+  JSG_READY();
+  JSG_REQUIRE(word && host_out_error, "%s: null pointer", who);
+  JSG_REQUIRE(!state().capturing, "%s during graph capture", who);
+  JSG_HIP(hipMemcpyAsync(host_out_error, word, sizeof(int), hipMemcpyDeviceToHost, state().stream));
+  JSG_HIP(hipStreamSynchronize(state().stream));
+  return 0;
+}
+
+int jsgrad_hip_attn_decode_status(void *workspace, int n_heads, int n_kv_heads, int head_dim, int *host_out_error) {
+  if (int e = read_error_word("jsgrad_hip_attn_decode_status", workspace, host_out_error)) return e;
+  if (*host_out_error != 0) {
+    // the merging block had cleared the words it saw and the late chunks stored afterwards: the workspace is not zero any
+    // more.  Clear all of it (the error word included), so that it can be used again.
+    JSG_REQUIRE(n_heads > 0 && n_kv_heads > 0 && head_dim > 0, "jsgrad_hip_attn_decode_status: n_heads %d / n_kv_heads %d / head_dim %d", n_heads, n_kv_heads, head_dim);
+    JSG_HIP(hipMemsetAsync(workspace, 0, jsgrad_hip_attn_workspace_bytes(n_heads, n_kv_heads, head_dim), state().stream));
+    JSG_HIP(hipStreamSynchronize(state().stream));
+    *host_out_error = 1;
+  }
+  return 0;
+}
+
+int jsgrad_hip_attn_decode_static_status(int *host_out_error) {
+  JSG_READY();
+  const int dev = state().device;
+  JSG_REQUIRE(dev >= 0 && dev < NOALLOC_MAX_DEVICES && g_scratch_ptr[dev] != nullptr, "jsgrad_hip_attn_decode_static_status: no built-in workspace on device %d", dev);
+  if (int e = read_error_word("jsgrad_hip_attn_decode_static_status", g_scratch_ptr[dev], host_out_error)) return e;
+  if (*host_out_error != 0) {      // the partial results are cleared by every call; only the error word is sticky
+    JSG_HIP(hipMemsetAsync(g_scratch_ptr[dev], 0, 256, state().stream));
+    JSG_HIP(hipStreamSynchronize(state().stream));
+    *host_out_error = 1;
+  }
+  return 0;
+}
+
 int jsgrad_hip_attn_decode_static(const void *q, const void *cache_k, const void *cache_v, const int32_t *st, void *out, int n_heads, int n_kv_heads,
                                   int head_dim, int max_context, int act) {
   JSG_READY();
   JSG_REQUIRE(q && cache_k && cache_v && st && out, "jsgrad_hip_attn_decode_static: null pointer argument");
-  JSG_REQUIRE(n_heads > 0 && n_kv_heads > 0 && max_context > 0, "jsgrad_hip_attn_decode_static: n_heads %d / n_kv_heads %d / max_context %d", n_heads, n_kv_heads, max_context);
-  JSG_REQUIRE(max_context <= 256 * ATT_CHUNK_MAX, "jsgrad_hip_attn_decode_static: max_context %d exceeds %d", max_context, 256 * ATT_CHUNK_MAX);
-  // 256 bytes of counters (used by the kernels that run many layers in one launch, not here), then one partial result per
-  // (head, chunk): only the chunks this max_context can produce are needed
+  if (int e = attn_decode_check("jsgrad_hip_attn_decode_static", n_heads, n_kv_heads, head_dim, max_context, act)) return e;
+  // 256 bytes of header (the error word), then one partial result per (head, chunk): only the chunks this max_context can
+  // produce are needed
   const int cap = max_context <= ATT_SHORT_CONTEXT ? ATT_NW * 16 : ATT_CHUNK_MAX;
   const size_t need = 256 + (size_t)n_heads * att_max_chunks(max_context, cap) * ((size_t)head_dim + 2) * sizeof(float);
   JSG_REQUIRE(need <= NOALLOC_SCRATCH_BYTES,
               "jsgrad_hip_attn_decode_static: %d heads of %d at max_context %d need %zu bytes of workspace, the built-in one holds %zu; use jsgrad_hip_attn_decode "
               "with a workspace of its own", n_heads, head_dim, max_context, need, (size_t)NOALLOC_SCRATCH_BYTES);
   const int dev = state().device;
-  JSG_REQUIRE(dev >= 0 && dev < NOALLOC_MAX_DEVICES, "jsgrad_hip_attn_decode_static: device %d", dev);
-  if (g_scratch_ptr[dev] == nullptr) {   // once per device, with that device current (jsgrad_hip_init made it so)
-    void *p = nullptr;
-    JSG_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
-    JSG_REQUIRE(p != nullptr, "jsgrad_hip_attn_decode_static: no device address for the built-in workspace");
-    g_scratch_ptr[dev] = p;
-  }
+  JSG_REQUIRE(dev >= 0 && dev < NOALLOC_MAX_DEVICES && g_scratch_ptr[dev] != nullptr, "jsgrad_hip_attn_decode_static: no built-in workspace on device %d", dev);
   void *ws = g_scratch_ptr[dev];
-  const int words = (int)((need + 3) / 4);
-  hipLaunchKernelGGL(zero_words_kernel, dim3((words + 255) / 256), dim3(256), 0, state().stream, (int *)ws, words);
+  const int words = (int)((need - 256 + 3) / 4);
+  hipLaunchKernelGGL(zero_words_kernel, dim3((words + 255) / 256), dim3(256), 0, state().stream, (int *)((char *)ws + 256), words);
   JSG_LAUNCHED();
   return jsgrad_hip_attn_decode(q, cache_k, cache_v, st, out, ws, n_heads, n_kv_heads, head_dim, max_context, act);
 }
@@ -181,13 +235,11 @@ int jsgrad_hip_attn_decode(const void *q, const void *cache_k, const void *cache
                            int n_kv_heads, int head_dim, int max_context, int act) {
   JSG_READY();
   JSG_REQUIRE(q && cache_k && cache_v && st && out && workspace, "jsgrad_hip_attn_decode: null pointer argument");
-  JSG_REQUIRE(act == JSGRAD_F16 || act == JSGRAD_F32, "jsgrad_hip_attn_decode: unknown activation dtype %d", act);
-  JSG_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_kv_heads <= 64 && n_heads % n_kv_heads == 0, "jsgrad_hip_attn_decode: n_heads %d / n_kv_heads %d", n_heads, n_kv_heads);
-  JSG_REQUIRE(head_dim == 64 || head_dim == 128, "jsgrad_hip_attn_decode: head_dim %d (64 and 128 are built)", head_dim);
-  JSG_REQUIRE(max_context > 0 && max_context <= 256 * ATT_CHUNK_MAX, "jsgrad_hip_attn_decode: max_context %d exceeds %d", max_context, 256 * ATT_CHUNK_MAX);
+  if (int e = attn_decode_check("jsgrad_hip_attn_decode", n_heads, n_kv_heads, head_dim, max_context, act)) return e;
   AttnArgs a;
   a.q = q; a.cache_k = cache_k; a.cache_v = cache_v; a.st = st; a.out = out;
-  a.counters = (int *)workspace;
+  a.counters = nullptr;              // this kernel's partial results say by themselves whether they are there
+  a.err = (int *)workspace;          // set when the merging block's bounded wait runs out (jsgrad_hip_attn_decode_status)
   a.partial = (float *)((char *)workspace + 256);
   const bool short_ctx = max_context <= ATT_SHORT_CONTEXT;
   a.n_kv_heads = n_kv_heads; a.nsplit = att_max_chunks(max_context, short_ctx ? ATT_NW * 16 : ATT_CHUNK_MAX); a.max_context = max_context;

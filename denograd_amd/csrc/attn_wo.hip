@@ -7,9 +7,13 @@
 // version tag, common.h): the wo part of a block asks for the row until every word carries the tag of this launch, then
 // multiplies with weights that are already in registers.
 //
-// Deadlock freedom: only the wo part waits, and only for the blocks with attention items, which have the lowest block ids
-// and are dispatched first; those never wait for anyone (the last block of a kv head to arrive merges, nobody waits for
-// that).  The wait is bounded all the same and reports through an error word.
+// Deadlock freedom.  Two kinds of block wait on the device for blocks of the same launch: blocks [0, n_kv_heads) run chunk 0
+// of a kv head and then wait for that head's other chunks (attention_core.h), and the wo part of every block waits for the
+// merged attention row.  Nobody waits for a block that waits: an item block publishes its partial result before it waits
+// for anything.  So the launch finishes if every block that runs an item gets onto the device while the others wait
+// there, i.e. if the items fit the device at once: the host asks the occupancy calculator (blocks per CU x CUs, which
+// assumes this process has the device to itself) and refuses a launch with more items than that.  Every wait is bounded
+// all the same, reports through the error word of the workspace, and the host raises when it reads the word.
 //
 // Reference: models/llama.ts:89-96 (repeat_kv + scaled_dot_product_attention + wo) and :125 (the residual add).
 #include "attention_core.h"

@@ -19,6 +19,7 @@ struct State {
   bool capturing = false;
 };
 State &state();
+int attn_static_init(int dev);   // attention.hip: resolves the built-in attention workspace's device address (jsgrad_hip_init)
 int fail(const char *fmt, ...);
 int fail_hip(hipError_t e, const char *what);
 

@@ -340,6 +340,10 @@ int jsgrad_hip_decode_step(const jsgrad_hip_step_t *d) {
   s.trace = d->trace;
   const int grid = state().cu_count;   // one block of 16 wavefronts per CU: every block is resident, which the barriers need
   JSG_REQUIRE(grid <= 1024, "jsgrad_hip_decode_step: %d CUs exceed the argmax partial buffer", grid);
+  // Attention items (kv head, chunk) are dealt to the blocks round-robin, and the item of a head's chunk 0 waits for that
+  // head's other chunks.  With at least as many blocks as a head has chunks, two waiting items can never each sit in
+  // front of a chunk the other waits for (that takes a head of more chunks than there are blocks), so the waits end.
+  JSG_REQUIRE(nsplit <= grid, "jsgrad_hip_decode_step: %d compute units are fewer than the %d chunks a kv head can have", grid, nsplit);
   const int n_rep = d->n_heads / d->n_kv_heads;
 #define JSG_KIND(K)                                                                                  \
   case K:                                                                                            \

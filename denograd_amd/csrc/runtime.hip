@@ -6,6 +6,7 @@
 
 #include <stdlib.h>
 
+#include <mutex>
 #include <unordered_map>
 #include <vector>
 
@@ -63,10 +64,15 @@ struct MemCache {
   size_t live_bytes = 0, idle_bytes = 0;
   size_t limit = 0;                                       // idle bytes beyond which the next stream wait gives them back
   bool enabled = true;                                    // LRU=0 switches the cache off (allocator.ts:73)
+  // Frees arrive from finalisers on whatever thread runs them (ctypes releases the interpreter lock during a call), so the
+  // books are kept under a lock; the stream waits and driver calls made while it is held are short and rare.
+  std::mutex lock;
 };
 static MemCache g_mem;
 
 // Classes are fine enough to waste under 2 % and coarse enough that tensors of nearly one size share blocks.
+// n <= MEM_MAX_REQUEST (checked by the caller): rounding up cannot wrap.
+constexpr size_t MEM_MAX_REQUEST = (size_t)1 << 48;
 static size_t mem_class(size_t n) {
   const size_t step = n <= (64u << 10) ? 256 : n <= (4u << 20) ? (4u << 10) : n <= (256u << 20) ? (256u << 10) : (4u << 20);
   return (n + step - 1) / step * step;
@@ -111,6 +117,7 @@ int jsgrad_hip_init(int device) {
     jsg::g_mem.limit = mb ? (size_t)strtoull(mb, nullptr, 10) << 20 : p.totalGlobalMem / 8;
   }
   s.device = device;
+  if (int e = jsg::attn_static_init(device)) return e;
   s.ready = true;
   return 0;
 }
@@ -131,8 +138,10 @@ int jsgrad_hip_cu_count(int *host_out) {
 int jsgrad_hip_malloc(size_t nbytes, void **host_out_ptr) {
   JSG_READY();
   JSG_REQUIRE(nbytes > 0, "alloc size must be positive, getting %zu", nbytes);
+  JSG_REQUIRE(nbytes <= jsg::MEM_MAX_REQUEST, "alloc size %zu is beyond any device", nbytes);
   JSG_REQUIRE(!state().capturing, "jsgrad_hip_malloc during graph capture");
   jsg::MemCache &m = jsg::g_mem;
+  std::lock_guard<std::mutex> guard(m.lock);
   const size_t cls = jsg::mem_class(nbytes);
   auto it = m.idle.find(cls);
   void *p = nullptr;
@@ -168,6 +177,7 @@ int jsgrad_hip_free(void *ptr) {
   if (!ptr) return 0;
   JSG_REQUIRE(!state().capturing, "jsgrad_hip_free during graph capture");
   jsg::MemCache &m = jsg::g_mem;
+  std::lock_guard<std::mutex> guard(m.lock);
   auto it = m.live.find(ptr);
   JSG_REQUIRE(it != m.live.end(), "jsgrad_hip_free: %p was not handed out by jsgrad_hip_malloc (or was freed already)", ptr);
   const size_t cls = it->second;
@@ -186,10 +196,12 @@ int jsgrad_hip_free_cache(void) {
   JSG_READY();
   JSG_REQUIRE(!state().capturing, "jsgrad_hip_free_cache during graph capture");
   JSG_HIP(hipStreamSynchronize(state().stream));
+  std::lock_guard<std::mutex> guard(jsg::g_mem.lock);
   return jsg::mem_release_idle();
 }
 int jsgrad_hip_mem_info(size_t *host_out_live_bytes, size_t *host_out_idle_bytes) {
   JSG_READY();
+  std::lock_guard<std::mutex> guard(jsg::g_mem.lock);
   if (host_out_live_bytes) *host_out_live_bytes = jsg::g_mem.live_bytes;
   if (host_out_idle_bytes) *host_out_idle_bytes = jsg::g_mem.idle_bytes;
   return 0;
@@ -220,7 +232,10 @@ int jsgrad_hip_sync(void) {
   JSG_READY();
   JSG_REQUIRE(!state().capturing, "jsgrad_hip_sync during graph capture");
   JSG_HIP(hipStreamSynchronize(state().stream));
-  if (jsg::g_mem.idle_bytes > jsg::g_mem.limit) return jsg::mem_release_idle();
+  {
+    std::lock_guard<std::mutex> guard(jsg::g_mem.lock);
+    if (jsg::g_mem.idle_bytes > jsg::g_mem.limit) return jsg::mem_release_idle();
+  }
   return 0;
 }
 

@@ -117,12 +117,25 @@ class HIPCompiler:
 
     FLAGS = ["-O3", "-include", "hip/hip_runtime.h", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
-    def __init__(self, arch: str = "gfx950", hipcc: str = "/opt/rocm/bin/hipcc", cachekey: str | None = "compile_hip_gfx950"):
+    def __init__(self, arch: str = "gfx950", hipcc: str = "/opt/rocm/bin/hipcc", cachekey: str | None = "auto"):
         self.arch, self.hipcc = arch, hipcc
+        if cachekey == "auto":
+            # one table per (architecture, flags, compiler): a code object made for another of these must never be loaded
+            cachekey = f"compile_hip_{arch}_{self._toolchain_id()}"
         # Compiler's constructor (allocator.ts:125-127): no key, no cache
         self.cachekey = None if os.environ.get("DISABLE_COMPILER_CACHE") else cachekey
         self.cache: dict[str, bytes] = {}
         self.compiles = 0       # hipcc runs of this object (tests and DEBUG output)
+
+    def _toolchain_id(self) -> str:
+        """Eight hex digits over the flags and the compiler's own version line (empty where hipcc cannot be run: the
+        compile itself will say so)."""
+        import hashlib
+        try:
+            ver = subprocess.run([self.hipcc, "--version"], capture_output=True, text=True, timeout=60).stdout
+        except (OSError, subprocess.SubprocessError):
+            ver = ""
+        return hashlib.sha256((" ".join(self.FLAGS) + "\n" + ver).encode()).hexdigest()[:8]
 
     def compile(self, src: str) -> bytes:
         self.compiles += 1

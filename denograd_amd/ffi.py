@@ -60,8 +60,10 @@ SIGNATURES: dict[str, tuple[list, object]] = {
     "jsgrad_hip_qkv_rope": ([_i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32], _i32),
     "jsgrad_hip_attn_workspace_bytes": ([_i32, _i32, _i32], _sz),
     "jsgrad_hip_attn_decode": ([_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32], _i32),
+    "jsgrad_hip_attn_decode_status": ([_vp, _i32, _i32, _i32, C.POINTER(_i32)], _i32),
     "jsgrad_hip_attn_decode_static_max_bytes": ([], _sz),
     "jsgrad_hip_attn_decode_static": ([_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32], _i32),
+    "jsgrad_hip_attn_decode_static_status": ([C.POINTER(_i32)], _i32),
     "jsgrad_hip_attn_wo_workspace_bytes": ([_i32, _i32, _i32], _sz),
     "jsgrad_hip_attn_wo": ([_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp, _i32], _i32),
     "jsgrad_hip_attn_wo_status": ([_vp, C.POINTER(_i32)], _i32),

@@ -318,12 +318,23 @@ class Transformer:
         check(ffi.load().jsgrad_hip_attn_wo_status(self._ctx.attn_wo_ws.ptr, C.byref(e)))
         return e.value
 
+    def attn_decode_error(self) -> int:
+        """1 if a bounded wait inside a jsgrad_hip_attn_decode launch ran out since the last call (the path of models whose
+        attention and wo do not share a launch).  Reading it clears the workspace for further use."""
+        if self._ctx is None or self._ctx.fuse_attn_wo:
+            return 0
+        e = C.c_int(0)
+        check(ffi.load().jsgrad_hip_attn_decode_status(self._ctx.workspace.ptr, self.n_heads, self.n_kv_heads, self.dim // self.n_heads, C.byref(e)))
+        return e.value
+
     def check_errors(self) -> None:
-        """Raise if a bounded wait inside a fused attention + wo launch ran out since the model was made (another process
-        holding compute units, or a device fault): the tokens after that point are not to be trusted.  Called wherever
-        the host waits for the device anyway (the per-token read of Llama3._call, the end of Llama3.generate)."""
+        """Raise if a bounded wait inside an attention launch ran out since the model was made (another process holding
+        compute units, or a device fault): the tokens after that point are not to be trusted.  Called wherever the host
+        waits for the device anyway (the per-token read of Llama3._call, the end of Llama3.generate)."""
         if self.attn_wo_error():
             raise ffi.HipError("a fused attention + wo launch gave up waiting for its attention row; results after that launch are invalid")
+        if self.attn_decode_error():
+            raise ffi.HipError("an attention launch gave up waiting for its partial results; results after that launch are invalid")
 
 
     # ---- plumbing

@@ -145,10 +145,16 @@ int jsgrad_hip_qkv_rope(int kind, const void *wq, const void *sq, const void *wk
 /* repeat_kv + scaled_dot_product_attention over cache rows [0, state[1]] (models/llama.ts:89-95,
  * tensor.ts:3920-3934), grouped-query: query head h reads kv head h / (n_heads/n_kv_heads).
  * workspace: jsgrad_hip_attn_workspace_bytes() bytes, zero-filled once before first use: a zero word means `partial result not
- * written yet`, and every launch leaves the workspace zero again. */
+ * written yet`, and every launch leaves the workspace zero again.  Inside the launch the block of a kv head's first chunk waits
+ * for the other chunks' results; the wait is bounded, and if it ever runs out (the blocks of the launch were kept off the
+ * device, by another process for instance) the output row is NaN, the first word of the workspace is set, and the workspace
+ * is NOT zero any more: results of later launches on it are invalid until jsgrad_hip_attn_decode_status has been called, which
+ * reports the word (*host_out_error = 1) and, when it was set, clears the whole workspace for further use.  _status waits
+ * for the stream; callers check it where they wait for the device anyway. */
 size_t jsgrad_hip_attn_workspace_bytes(int n_heads, int n_kv_heads, int head_dim);
 int jsgrad_hip_attn_decode(const void *q, const void *cache_k, const void *cache_v, const int32_t *state, void *out, void *workspace,
                            int n_heads, int n_kv_heads, int head_dim, int max_context, int act);
+int jsgrad_hip_attn_decode_status(void *workspace, int n_heads, int n_kv_heads, int head_dim, int *host_out_error);
 
 /* jsgrad_hip_attn_decode without the workspace argument, for callers that cannot allocate device memory (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The partial
@@ -156,10 +162,14 @@ int jsgrad_hip_attn_decode(const void *q, const void *cache_k, const void *cache
  * (8 MiB) on every GPU the library runs on, held until the process ends.  The call allocates and frees nothing; shapes whose
  * workspace (256 + n_heads * chunks(max_context) * (head_dim + 2) * 4 bytes, chunks <= 256) does not fit are refused with an
  * error.  All calls on one GPU share the array: they are ordered by the library's stream; calls that overlap on one GPU
- * (other streams, other threads) race.  Same results as jsgrad_hip_attn_decode, bit for bit. */
+ * (other streams, other threads) race.  Same results as jsgrad_hip_attn_decode, bit for bit.  The array's device address is
+ * resolved by jsgrad_hip_init, so the call itself only launches kernels (a fill of the partial results it will use, then
+ * the attention) and may be captured into a graph.  jsgrad_hip_attn_decode_static_status reports, and clears, the error word
+ * of a bounded wait that ran out (see jsgrad_hip_attn_decode); the partial results are cleared by every call anyway. */
 size_t jsgrad_hip_attn_decode_static_max_bytes(void);
 int jsgrad_hip_attn_decode_static(const void *q, const void *cache_k, const void *cache_v, const int32_t *state, void *out,
                                   int n_heads, int n_kv_heads, int head_dim, int max_context, int act);
+int jsgrad_hip_attn_decode_static_status(int *host_out_error);
 
 /* ffn_norm + w1, w3 + SwiGLU (FeedForward.call, models/llama.ts:108-110): g[hidden] = silu(w1 x) * (w3 x). */
 int jsgrad_hip_ffn_gate(int kind, const void *w1, const void *s1, const void *w3, const void *s3, const void *x,

@@ -144,6 +144,10 @@ export class HipDecoder {
       const err = c.out_i32()
       c.check(S.jsgrad_hip_attn_wo_status(ptr(this.attn_wo_ws), err)) // waits for the stream, like the caller's .item()
       if (err[0]) throw new Error('jsgrad_hip_attn_wo: a bounded wait ran out; the tokens of this step are not to be trusted')
+    } else {
+      const a = this.model.layers[0].attention, err = c.out_i32()
+      c.check(S.jsgrad_hip_attn_decode_status(ptr(this.attn_ws), a.n_heads, a.n_kv_heads, a.head_dim, err)) // reports and clears
+      if (err[0]) throw new Error('jsgrad_hip_attn_decode: a bounded wait ran out; the tokens of this step are not to be trusted')
     }
     return this.state.shrink([[0, 1]])
   }

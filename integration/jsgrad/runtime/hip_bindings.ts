@@ -46,8 +46,10 @@ const SYMBOLS = {
   jsgrad_hip_qkv_rope: { parameters: [I, P, P, P, P, P, P, P, P, F, P, P, P, P, P, I, I, I, I, I, I], result: I }, // kind, wq, sq, wk, sk, wv, sv, x, norm_weight, eps, rope_table, state, q_out, cache_k, cache_v, dim, n_heads, n_kv_heads, head_dim, max_context, act
   jsgrad_hip_attn_workspace_bytes: { parameters: [I, I, I], result: U }, // n_heads, n_kv_heads, head_dim
   jsgrad_hip_attn_decode: { parameters: [P, P, P, P, P, P, I, I, I, I, I], result: I }, // q, cache_k, cache_v, state, out, workspace, n_heads, n_kv_heads, head_dim, max_context, act
+  jsgrad_hip_attn_decode_status: { parameters: [P, I, I, I, B], result: I }, // workspace, n_heads, n_kv_heads, head_dim, host_out_error
   jsgrad_hip_attn_decode_static_max_bytes: { parameters: [], result: U },
   jsgrad_hip_attn_decode_static: { parameters: [P, P, P, P, P, I, I, I, I, I], result: I }, // q, cache_k, cache_v, state, out, n_heads, n_kv_heads, head_dim, max_context, act
+  jsgrad_hip_attn_decode_static_status: { parameters: [B], result: I }, // host_out_error
   jsgrad_hip_ffn_gate: { parameters: [I, P, P, P, P, P, P, F, P, I, I, I], result: I }, // kind, w1, s1, w3, s3, x, norm_weight, eps, g, dim, hidden, act
   jsgrad_hip_argmax: { parameters: [P, I, P, P, I, I, I], result: I }, // logits, n, state, tokens_out, tokens_cap, advance, act
   jsgrad_hip_embed_rows: { parameters: [I, P, P, P, I, P, I, I], result: I }, // kind, table, scale, tokens, rows, out, dim, vocab

@@ -62,15 +62,24 @@ export class HIPProgram extends Program {
   }
 }
 
+// packed fp32 instructions stay off on this hardware generation
+const HIPCC_FLAGS = ['-O3', '-x', 'hip', '-include', 'hip/hip_runtime.h', '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops']
+// A short stable number over the flags, so that a change of flags starts a new table of the disk cache.  (The Python twin
+// also folds in `hipcc --version`; here a new compiler is told apart by ROCM_VERSION in the environment, when set.)
+const flags_id = () => {
+  let h = 2166136261
+  for (const ch of HIPCC_FLAGS.join(' ') + '\n' + (vars.get('ROCM_VERSION') || '')) h = Math.imul(h ^ ch.charCodeAt(0), 16777619) >>> 0
+  return h.toString(16).padStart(8, '0')
+}
+
 export class HIPCompiler extends Compiler {
-  constructor(public arch = 'gfx950', cachekey = `compile_hip_${arch}`) {
+  constructor(public arch = 'gfx950', cachekey = `compile_hip_${arch}_${flags_id()}`) {
     super(cachekey) // compile_cached keeps code objects in env's disk cache under this key (allocator.ts:129-137)
   }
   override compile = async (src: string): Promise<Uint8Array> => {
     const code = await env.tempFile(), bin = await env.tempFile()
     await env.writeTextFile(code, src)
-    // packed fp32 instructions stay off on this hardware generation
-    const args = ['hipcc', '--genco', `--offload-arch=${this.arch}`, '-O3', '-x', 'hip', '-include', 'hip/hip_runtime.h', '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops', code, '-o', bin]
+    const args = ['hipcc', '--genco', `--offload-arch=${this.arch}`, ...HIPCC_FLAGS, code, '-o', bin]
     try {
       await env.exec(args.join(' '))
     } catch (e) {

@@ -58,6 +58,20 @@ def test_compile_cached_survives_the_process_object(cache_db):
     assert other.compile_cached("k1") == b"CODE:k1" and other.compiles == 1
 
 
+def test_compile_cache_table_follows_architecture_flags_and_compiler():
+    """A code object made for another architecture, with other flags or by another compiler must never come back from the
+    disk cache: each of the three is part of the table's name."""
+    base = HIPCompiler().cachekey
+    assert base.startswith("compile_hip_gfx950_")
+    assert HIPCompiler(arch="gfx942").cachekey.startswith("compile_hip_gfx942_")
+
+    class OtherFlags(HIPCompiler):
+        FLAGS = HIPCompiler.FLAGS + ["-ffast-math"]
+    assert OtherFlags().cachekey != base
+    assert HIPCompiler(hipcc="/nonexistent/hipcc").cachekey != base      # no version line: another table, not an exception
+    assert HIPCompiler().cachekey == base
+
+
 def test_compile_cache_switches(cache_db, monkeypatch):
     CountingCompiler().compile_cached("k1")
     monkeypatch.setenv("ASSERT_COMPILE", "1")
