@@ -409,7 +409,7 @@ def run_batched(name, bsz, prompt_len, steps):
             "prefill": prefill, "decode": decode}
 
 
-def traffic_probe(name, batch=1):
+def traffic_probe(name, batch=1, position=0):
     from denograd_amd import ffi, synthetic
     from denograd_amd.ffi import check
     from denograd_amd.llama3 import Llama3
@@ -420,9 +420,10 @@ def traffic_probe(name, batch=1):
     check(lib.jsgrad_hip_sync())
     check(lib.jsgrad_hip_copy(dst.ptr, src.ptr, n))      # reads 512 MiB, writes 512 MiB
     check(lib.jsgrad_hip_sync())
-    cfg = synthetic.config(name, max_context=64)
+    cfg = synthetic.config(name, max_context=position + 64)
     llm = Llama3.from_config(cfg).random_init(seed=0, tied=cfg["tied"])
     llm.model.forward_jit = None
+    llm.start_pos = position      # the cache rows before it are whatever the allocation holds: the counters do not care
     for t in (1, 2, 3, 4):
         llm._call(t)
         llm.start_pos += 1
@@ -542,6 +543,7 @@ def main():
     ap.add_argument("--traffic-probe", action="store_true", help="for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: one 512 MiB device-to-device copy "
                     "(a plain copy kernel of known size, to scale the counters) followed by 4 eager decode steps of --workload; prints nothing")
     ap.add_argument("--traffic-batch", type=int, default=1, help="with --traffic-probe: also two batched decode steps of this many sequences")
+    ap.add_argument("--traffic-position", type=int, default=0, help="with --traffic-probe: the position the four decode steps start from (attention then reads that many cache rows)")
     ap.add_argument("--fused-step", action="store_true", help="run each token as one persistent kernel (jsgrad_hip_decode_step) instead of one launch per fused op")
     ap.add_argument("--stream-step", action="store_true", help="run each token as one persistent kernel with streaming wavefronts (jsgrad_hip_stream_step)")
     ap.add_argument("--formats-only", action="store_true", help="only the load-time kernels of the checkpoint path (GGML dequantisation, casts, row permutation); prints their JSON")
@@ -561,7 +563,7 @@ def main():
     log(f"device: {dev.name}, {dev.cu_count} CUs")
 
     if args.traffic_probe:
-        traffic_probe(args.workload, args.traffic_batch)
+        traffic_probe(args.workload, args.traffic_batch, args.traffic_position)
         return
     if args.formats_only:
         print(json.dumps({"formats": run_formats()}), flush=True)

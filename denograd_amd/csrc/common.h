@@ -200,7 +200,10 @@ __device__ __forceinline__ void trace_stamp(int row, int slot) {
 // The same stamps kept in LDS and copied out when the block ends: a stamp written to memory is a store, and the next wait for
 // a load waits for it too, which stretches whatever follows it.  JSG_LCLEAR() first, JSG_LFLUSH(row) last (both block-wide).
 static __shared__ unsigned long long jsg_tl[32];
-#define JSG_LSTAMP(slot) do { if (threadIdx.x == 0) jsg::jsg_tl[slot] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#ifndef JSG_TRACE_THREAD
+#define JSG_TRACE_THREAD 0      // the thread whose time is kept: 0, or the first lane of another wavefront of the block
+#endif
+#define JSG_LSTAMP(slot) do { if (threadIdx.x == JSG_TRACE_THREAD) jsg::jsg_tl[slot] = __builtin_amdgcn_s_memrealtime(); } while (0)
 #define JSG_LCLEAR() do { if (threadIdx.x < 32) jsg::jsg_tl[threadIdx.x] = 0; __syncthreads(); } while (0)
 #define JSG_LFLUSH(row) do { __syncthreads(); const int row_ = (row); if (row_ >= 0 && threadIdx.x < 32) jsg::g_trace[row_][threadIdx.x] = jsg::jsg_tl[threadIdx.x]; } while (0)
 #define JSG_TRACE_ENTRY(name)                                                                              \
@@ -303,6 +306,20 @@ static __device__ __constant__ float NF4_CODE[16] = {JSG_C16(-1.0f), JSG_C16(-0.
                                               JSG_C16(-0.28444138169288635f), JSG_C16(-0.18477343022823334f), JSG_C16(-0.09105003625154495f), JSG_C16(0.0f),
                                               JSG_C16(0.07958029955625534f), JSG_C16(0.16093020141124725f), JSG_C16(0.24611230194568634f), JSG_C16(0.33791524171829224f),
                                               JSG_C16(0.44070982933044434f), JSG_C16(0.5626170039176941f), JSG_C16(0.7229568362236023f), JSG_C16(1.0f)};
+
+// NF4 code n as fp16 bits, selected from literals by the four bits of n: a table in memory would cost its readers a memory
+// round trip per entry, and the look-up tables are built at the head of a launch, in front of everything else.
+#define JSG_H16(x) ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)(x)))
+__device__ __forceinline__ uint32_t nf4_code_bits(int n) {
+  const bool b0 = n & 1, b1 = n & 2, b2 = n & 4, b3 = n & 8;
+  const uint32_t q0 = b0 ? JSG_H16(-0.6961928009986877f) : JSG_H16(-1.0f), q1 = b0 ? JSG_H16(-0.39491748809814453f) : JSG_H16(-0.5250730514526367f);
+  const uint32_t q2 = b0 ? JSG_H16(-0.18477343022823334f) : JSG_H16(-0.28444138169288635f), q3 = b0 ? JSG_H16(0.0f) : JSG_H16(-0.09105003625154495f);
+  const uint32_t q4 = b0 ? JSG_H16(0.16093020141124725f) : JSG_H16(0.07958029955625534f), q5 = b0 ? JSG_H16(0.33791524171829224f) : JSG_H16(0.24611230194568634f);
+  const uint32_t q6 = b0 ? JSG_H16(0.5626170039176941f) : JSG_H16(0.44070982933044434f), q7 = b0 ? JSG_H16(1.0f) : JSG_H16(0.7229568362236023f);
+  const uint32_t p0 = b1 ? q1 : q0, p1 = b1 ? q3 : q2, p2 = b1 ? q5 : q4, p3 = b1 ? q7 : q6;
+  const uint32_t o0 = b2 ? p1 : p0, o1 = b2 ? p3 : p2;
+  return b3 ? o1 : o0;
+}
 
 // silu(a) = a * 1/(1 + exp2(a * -1/ln2)) (tensor.ts:2909-2911, 3210-3226) in the activation dtype's arithmetic
 template <typename AT> __device__ __forceinline__ float silu_act(float a);

@@ -5,29 +5,44 @@
 
 namespace jsg {
 
-// fp16 activations: four blocks per CU (128 registers per lane), which the grid is sized for
+// fp16 activations: 16 wavefronts per CU (128 registers per lane), which the grid is sized for: four blocks of four (NW = 4), or,
+// for NF4 launches with rows enough for that on every CU, one block of sixteen around a per-lane look-up table of 64 KiB
+// (NW = 16, Gemv<..., WIDE>).
 // EXACT: see Gemv::load_item; the host picks it from the items a wavefront of the launch walks
-template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, int EXACT>
-__global__ __launch_bounds__(256, sizeof(AT) == 2 ? 4 : 1) void gemv_kernel(GemvArgs a) {
+template <int KIND, typename AT> constexpr bool gemv_may_be_wide() { return KIND == JSGRAD_W_NF4 && sizeof(AT) == 2; }
+template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, int EXACT, int NW = 4>
+__global__ __launch_bounds__(64 * NW, sizeof(AT) == 2 ? 4 : 1) void gemv_kernel(GemvArgs a) {
+  constexpr bool WIDE = NW == 16;
   extern __shared__ __align__(16) unsigned char smem[];
-  __shared__ float red[8];
-  __shared__ float lut[KIND == JSGRAD_W_NF4 ? NF4_LUT_WORDS : 16];
-  typedef Gemv<KIND, AT, EPI, ROWS, UNROLL, false, EXACT> G;
+  __shared__ float red[16];
+  __shared__ float lut[KIND == JSGRAD_W_NF4 ? (WIDE ? NF4_WIDE_LUT_WORDS : NF4_LUT_WORDS) : 16];
+  typedef Gemv<KIND, AT, EPI, ROWS, UNROLL, false, EXACT, WIDE> G;
   // read the position now, not in the epilogue: the load then overlaps the weight stream instead of ending the kernel
+  JSG_LCLEAR();
   const int pos = EPI == EPI_ROPE_KV ? a.st[1] : 0;
+  JSG_LSTAMP(0);
   GemvBuf buf;
   G::template run<true>(a, (AT *)smem, red, lut, buf, false, pos);
+  JSG_LSTAMP(8);
+  JSG_LFLUSH(blockIdx.x == 0 ? 0 : (blockIdx.x == gridDim.x / 2 ? 1 : (blockIdx.x == gridDim.x - 1 ? 2 : -1)));
 }
+JSG_TRACE_ENTRY(jsgrad_hip_gemv_trace)
 
 // ---- host-side dispatch ------------------------------------------------------------------------
 
-template <int KIND, typename AT, int EPI, int ROWS, int UNROLL> static int launch_cfg(const GemvArgs &a, int total_rows) {
+template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, int NW = 4> static int launch_cfg(const GemvArgs &a, int total_rows) {
   constexpr int kind = EPI == EPI_STORE ? PROF_LINEAR : (EPI == EPI_SWIGLU ? PROF_FFN_GATE : PROF_QKV_ROPE);
-  constexpr int NW = 4;
   const int ngroups = (total_rows + ROWS - 1) / ROWS;
+  if constexpr (gemv_may_be_wide<KIND, AT>() && NW == 4) {
+    // rows enough to give every CU a block of sixteen wavefronts: the per-lane table (measured on the 8B shapes: w1 | w3
+    // 20.0 -> 17.2 us; with fewer rows the launch is a few microseconds either way and the larger block's staging costs more)
+    static const int force = getenv("JSG_NF4_WAVES") ? atoi(getenv("JSG_NF4_WAVES")) : 0;
+    if (force ? force == 16 : ngroups >= 16 * state().cu_count) return launch_cfg<KIND, AT, EPI, ROWS, UNROLL, 16>(a, total_rows);
+  }
   const int need = (ngroups + NW - 1) / NW;      // one group per wavefront
-  static const int per_cu = getenv("JSG_GEMV_BLOCKS_PER_CU") ? atoi(getenv("JSG_GEMV_BLOCKS_PER_CU")) : 4;
-  const int cap = state().cu_count * per_cu;      // 16 resident wavefronts per CU; more rows than that are walked grid-stride
+  static const int waves_per_cu = getenv("JSG_GEMV_BLOCKS_PER_CU") ? 4 * atoi(getenv("JSG_GEMV_BLOCKS_PER_CU")) : 16;
+  // 16 resident wavefronts per CU; more rows than that are walked grid-stride
+  const int cap = state().cu_count * (waves_per_cu / NW > 0 ? waves_per_cu / NW : 1);
   dim3 grid(need < cap ? need : cap), block(NW * 64);
   typedef Gemv<KIND, AT, EPI, ROWS, UNROLL, false> G;
   const int most_rows = a.rows0 > a.rows1 ? (a.rows0 > a.rows2 ? a.rows0 : a.rows2) : (a.rows1 > a.rows2 ? a.rows1 : a.rows2);
@@ -37,9 +52,23 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL> static int launc
   const int waves = (int)grid.x * NW;
   const int nbatch = G::x_elems(a.in_f) / (UNROLL * G::STEP);
   const int items = ((ngroups + waves - 1) / waves) * nbatch;
-  if (items >= 3) JSG_LAUNCH(kind, (gemv_kernel<KIND, AT, EPI, ROWS, UNROLL, 2>), grid, block, lds, a);
-  else if (nbatch >= 2) JSG_LAUNCH(kind, (gemv_kernel<KIND, AT, EPI, ROWS, UNROLL, 1>), grid, block, lds, a);
-  else JSG_LAUNCH(kind, (gemv_kernel<KIND, AT, EPI, ROWS, UNROLL, 0>), grid, block, lds, a);
+  if constexpr (NW == 16) {
+    // the look-up table is static LDS of more than 64 KiB: the staged row on top of it is dynamic LDS the runtime must be told about
+    static bool told = false;
+    if (!told) {
+      const int most = 64 * 1024;
+      JSG_HIP(hipFuncSetAttribute((const void *)gemv_kernel<KIND, AT, EPI, ROWS, UNROLL, 0, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, most));
+      JSG_HIP(hipFuncSetAttribute((const void *)gemv_kernel<KIND, AT, EPI, ROWS, UNROLL, 1, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, most));
+      JSG_HIP(hipFuncSetAttribute((const void *)gemv_kernel<KIND, AT, EPI, ROWS, UNROLL, 2, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, most));
+      told = true;
+    }
+  }
+  // the second request is straight-line code where every wavefront has a second item, and also where only some have (rows
+  // of one batch, more row groups than wavefronts): a wavefront whose second request sits behind a test waits for both
+  // items before it starts on the first, which costs the launch more than the others' address arithmetic for nothing
+  if (items >= 3) JSG_LAUNCH(kind, (gemv_kernel<KIND, AT, EPI, ROWS, UNROLL, 2, NW>), grid, block, lds, a);
+  else if (nbatch >= 2 || ngroups > waves) JSG_LAUNCH(kind, (gemv_kernel<KIND, AT, EPI, ROWS, UNROLL, 1, NW>), grid, block, lds, a);
+  else JSG_LAUNCH(kind, (gemv_kernel<KIND, AT, EPI, ROWS, UNROLL, 0, NW>), grid, block, lds, a);
   return 0;
 }
 // Two register buffers of UNROLL x NM x ROWS 16-byte loads each: (2 rows, 4 steps) for one matrix, (2 rows, 2 steps)

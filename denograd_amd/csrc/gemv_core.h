@@ -166,6 +166,14 @@ template <> struct Dot<JSGRAD_W_NF4, _Float16> {
   }
 };
 
+// The same table kept once PER LANE, for launches with enough rows to give every CU one block of sixteen wavefronts
+// (Gemv<..., WIDE>): entry e of lane l is the word at byte e * 256 + l * 4 behind NF4_TAB_OFFSET, 64 KiB in all.  The weight
+// bytes are as good as random, and 64 lanes asking one shared table for 64 random entries keep the 32 LDS banks busy for
+// ~7 cycles instead of 2 (counted: 4.8 conflict cycles per look-up).  With a copy per lane, lane l only ever touches bank
+// l % 32, and the address is one byte permute: byte 1 = the weight byte, byte 0 = 4 l, no shift, no add.
+constexpr int NF4_TAB_OFFSET = 256, NF4_TAB_BYTES = 256 * 256;
+constexpr int NF4_WIDE_LUT_WORDS = (NF4_TAB_OFFSET + NF4_TAB_BYTES) / 4;
+
 // Stage x (optionally RMSNorm'ed) into LDS in the activation dtype.  Every thread moves 16-byte chunks; with a
 // norm the chunks stay in registers between the sum of squares and the scaling, so x is read from memory once and
 // the whole prologue costs one round of loads and two barriers.  Ends with a barrier.
@@ -440,7 +448,8 @@ __device__ __forceinline__ void set_extra(GemvBuf &b, int r, _Float16 v) { b.ext
 // consumed, and the first item is requested before x is staged (or, with `preloaded`, before the caller even waited
 // for the previous phase), so a wavefront always has a batch of 128-bit loads in flight.
 // COHERENT: x, residual and outputs cross between blocks of the same launch.
-template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT, int EXACT = 0> struct Gemv {
+// WIDE (NF4 weights, fp16 activations): the look-up table is kept per lane (NF4_TAB_OFFSET); lut then has NF4_WIDE_LUT_WORDS words.
+template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT, int EXACT = 0, bool WIDE = false> struct Gemv {
   static constexpr int VEC = WFmt<KIND>::VEC;
   static constexpr int BITS = KIND == JSGRAD_W_F32 ? 32 : KIND == JSGRAD_W_F16 ? 16 : KIND == JSGRAD_W_I8 ? 8 : 4;
   static constexpr int STEP = 64 * VEC;                 // elements one wavefront covers per k-step
@@ -609,16 +618,55 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT, i
       const int k = (b * UNROLL + u) * STEP + lane * VEC;   // may lie in the zero padding of xs
       XFrag<AT, VEC> xf;
       xf.load(xs + k);
+      if constexpr (WIDE && KIND == JSGRAD_W_NF4 && sizeof(AT) == 2) {
+        // The NM x ROWS vectors of this k-step in stages of eight weight bytes: the table look-ups of stage s + 1 are sent
+        // before the products of stage s are formed.  Written vector by vector, every wavefront asks the table for eight
+        // entries and then waits for them with nothing else to do, and the wavefronts of a CU do so in step: the vector
+        // ALUs and the LDS pipe took turns (counted: each busy 44 % of the launch, and the launch as long as both together).
+        constexpr int NVU = NM * ROWS, NST = NVU * 2;
+        const char *tab = (const char *)lut + NF4_TAB_OFFSET;
+        const uint32_t lane4 = (uint32_t)lane << 2;
+        uint32_t ent[2][8];
+        float sv[NVU];
 #pragma unroll
-      for (int j = 0; j < NM; j++)
+        for (int v = 0; v < NVU; v++) sv[v] = 0.0f;
+        auto issue = [&](int st, uint32_t (&e)[8]) {
+          const u4_t wv = buf.w[wi(u, 0, 0) + (st >> 1)];      // wi(u, j, r) = wi(u, 0, 0) + j * ROWS + r
 #pragma unroll
-        for (int r = 0; r < ROWS; r++) {
-          float bs = 1.0f;
-          if constexpr (KIND == JSGRAD_W_NF4) bs = (float)buf.nscale[wi(u, j, r)];
-          // every 16-byte vector is summed on its own and then added: eight short dependent chains per item
-          // instead of two long ones
-          acc[j][r] += Dot<KIND, AT>::run(buf.w[wi(u, j, r)], xf, 0.0f, bs, lut);
+          for (int q = 0; q < 2; q++) {
+            const uint32_t d = wv[(st & 1) * 2 + q];
+#pragma unroll
+            for (int bb = 0; bb < 4; bb++) e[q * 4 + bb] = *(const uint32_t *)(tab + __builtin_amdgcn_perm(lane4, d, 0x0c0c0004u | ((uint32_t)bb << 8)));
+          }
+        };
+        issue(0, ent[0]);
+#pragma unroll
+        for (int st = 0; st < NST; st++) {
+          if (st + 1 < NST) issue(st + 1, ent[(st + 1) & 1]);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int q = 0; q < 2; q++)
+#pragma unroll
+            for (int bb = 0; bb < 4; bb++)
+              sv[st >> 1] = __builtin_amdgcn_fdot2(as_h2(ent[st & 1][q * 4 + bb]), xf.v[((st & 1) * 2 + q) * 4 + bb], sv[st >> 1], false);
+          __builtin_amdgcn_sched_barrier(0);
         }
+#pragma unroll
+        for (int j = 0; j < NM; j++)
+#pragma unroll
+          for (int r = 0; r < ROWS; r++) acc[j][r] += sv[j * ROWS + r] * (float)buf.nscale[wi(u, j, r)];
+      } else {
+#pragma unroll
+        for (int j = 0; j < NM; j++)
+#pragma unroll
+          for (int r = 0; r < ROWS; r++) {
+            float bs = 1.0f;
+            if constexpr (KIND == JSGRAD_W_NF4) bs = (float)buf.nscale[wi(u, j, r)];
+            // every 16-byte vector is summed on its own and then added: eight short dependent chains per item
+            // instead of two long ones
+            acc[j][r] += Dot<KIND, AT>::run(buf.w[wi(u, j, r)], xf, 0.0f, bs, lut);
+          }
+      }
     }
     if (b != nbatch(a) - 1) return;
 
@@ -668,14 +716,22 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT, i
     }
   }
 
-  // the NF4 tables in LDS (published by the barrier at the end of stage_x)
+  // the NF4 tables in LDS (published by the barrier at the end of stage_x).  The code values come from literals
+  // (nf4_code_bits): read from a table in memory they cost a round trip at the head of every launch.
   __device__ static __forceinline__ void fill_lut(float *lut) {
     if constexpr (KIND == JSGRAD_W_NF4) {
-      if (threadIdx.x < 16) lut[threadIdx.x] = NF4_CODE[threadIdx.x];
-      if constexpr (sizeof(AT) == 2) {   // the table of code pairs, one entry per byte value (lut has NF4_LUT_WORDS words then)
-        for (int e = threadIdx.x; e < 256; e += blockDim.x) {
-          const h2_t pr = {(_Float16)NF4_CODE[e >> 4], (_Float16)NF4_CODE[e & 15]};
-          ((uint32_t *)lut)[16 + e] = __builtin_bit_cast(uint32_t, pr);
+      if (threadIdx.x < 16) lut[threadIdx.x] = (float)__builtin_bit_cast(_Float16, (uint16_t)nf4_code_bits(threadIdx.x));
+      if constexpr (sizeof(AT) == 2) {   // the table of code pairs, one entry per byte value: element 2j (the high nibble) in the low half
+        if constexpr (WIDE) {            // ... and per lane: thread e writes entry e's 256-byte row
+          u4_t *tab = (u4_t *)((char *)lut + NF4_TAB_OFFSET);
+          if (threadIdx.x < 256) {
+            const int e = threadIdx.x;
+            const uint32_t w = nf4_code_bits(e >> 4) | (nf4_code_bits(e & 15) << 16);
+#pragma unroll
+            for (int c = 0; c < 16; c++) tab[e * 16 + c] = u4_t{w, w, w, w};
+          }
+        } else {
+          for (int e = threadIdx.x; e < 256; e += blockDim.x) ((uint32_t *)lut)[16 + e] = nf4_code_bits(e >> 4) | (nf4_code_bits(e & 15) << 16);
         }
       }
     }
@@ -694,34 +750,37 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT, i
     if constexpr (EARLY_X) stage_x_issue<AT>(a, xst);
     fill_lut(lut);
     int grp = first_group(blk, nblk), b = 0;
-    // the first item is straight-line code in every launch (the staging of x below then waits for x and not for it)
-    if (!preloaded) load_item_as<true>(a, bufA, grp, 0, pos, grp < ng);
     auto advance = [&](int &g, int &bb) {
       if (++bb == nb) { bb = 0; g += gstride; }
     };
-    // the second item goes out before x is staged too: staging (a read of x, the RMSNorm reduction, a block barrier)
-    // would otherwise be a stretch with nothing new in flight
     Buf bufB;
     int gB = grp, bB = b;
     advance(gB, bB);
+    // the first item is straight-line code in every launch (the staging of x below then waits for x and not for it)
+    if (!preloaded) load_item_as<true>(a, bufA, grp, 0, pos, grp < ng);
     // block-wide, ends with a barrier (which also publishes lut)
     if constexpr (EARLY_X) {
       // x is back after one round trip; its registers are free again before the second item's are needed
       stage_x_finish<AT>(a, xst, xs, red, nb * UNROLL * STEP);
       load_item_as<(EXACT >= 1)>(a, bufB, gB, bB, pos, gB < ng);
     } else {
+      // the second item goes out before x is staged too: staging (a read of x, the RMSNorm reduction, a block barrier)
+      // would otherwise be a stretch with nothing new in flight
       load_item_as<(EXACT >= 1)>(a, bufB, gB, bB, pos, gB < ng);
       stage_x<AT, COHERENT>(a, xs, red, nb * UNROLL * STEP);
     }
 
     float acc[NM][ROWS];
+    JSG_LSTAMP(23);
     while (grp < ng) {
       use_item(a, bufA, grp, b, acc, xs, lut, pos);
+      JSG_LSTAMP(24);
       if (gB >= ng) break;
       grp = gB; b = bB;
       advance(grp, b);                                   // the item after B goes into A
       load_item(a, bufA, grp, b, pos, grp < ng);
       use_item(a, bufB, gB, bB, acc, xs, lut, pos);
+      JSG_LSTAMP(25);
       gB = grp; bB = b;
       advance(gB, bB);                                   // and the one after that into B
       load_item(a, bufB, gB, bB, pos, grp < ng && gB < ng);
