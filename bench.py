@@ -436,6 +436,62 @@ def traffic_probe(name, batch=1, position=0):
         check(lib.jsgrad_hip_sync())
 
 
+STAMP_NAMES = {0: "position word read", 10: "attention item starts", 11: "query rows in LDS", 12: "scores done", 13: "softmax done", 14: "P.V in the wavefronts' slots",
+               15: "partial result stored", 16: "every chunk's (m, l) seen", 17: "merge weights ready", 18: "merged row stored", 1: "attention item done",
+               2: "wo: hint of the attention row seen", 3: "wo: hint barrier", 4: "wo: attention row staged", 21: "wo rows done",
+               23: "x staged, first two items requested", 24: "first item used", 25: "second item used", 8: "end"}
+
+
+def stamps(name, position, layers=8):
+    """Time stamps taken INSIDE the kernels (a library built with `make TRACE=1`): the 100 MHz device clock kept in LDS by one
+    thread of three blocks per launch and copied out when the block ends.  Runs a few eager decode steps of `name` (cut to
+    `layers` layers) from `position` and prints, for the last attention launch and the last w1 | w3 launch, microseconds
+    since the earliest stamp of that launch."""
+    from denograd_amd import ffi, synthetic
+    from denograd_amd.ffi import check
+    from denograd_amd.llama3 import Llama3
+    lib = ffi.load()
+    raw = C.CDLL(ffi.LIB_PATH)
+    if not hasattr(raw, "jsgrad_hip_gemv_trace"):
+        raise SystemExit("this library has no time stamps: build it with `make -B -C denograd_amd/csrc TRACE=1`")
+    cfg = synthetic.config(name, max_context=position + 64, n_layers=layers)
+    llm = Llama3.from_config(cfg).random_init(seed=0, tied=cfg["tied"])
+    m = llm.model
+    m.forward_jit = None
+    llm.start_pos = position
+    for t in (1, 2, 3):
+        llm._call(t)
+        llm.start_pos += 1
+    buf = (C.c_ulonglong * 96)()
+    out = {}
+
+    def read(entry, rows):
+        fn = getattr(raw, entry)
+        fn.argtypes, fn.restype = [C.c_void_p], C.c_int
+        check(fn(buf))
+        t = np.array(buf[:], dtype=np.uint64).reshape(3, 32).astype(np.int64)
+        if not (t > 0).any():
+            return None
+        t0 = t[t > 0].min()
+        return {who: {STAMP_NAMES[s_]: round((int(t[r][s_]) - int(t0)) / 100.0, 2) for s_ in sorted(STAMP_NAMES, key=lambda k: t[r][k]) if t[r][s_] > 0}
+                for r, who in enumerate(rows)}
+    fused = m._ctx.fuse_attn_wo
+    llm._call(4)
+    llm.start_pos += 1
+    if fused:
+        out["attn_wo_kernel"] = read("jsgrad_hip_attn_wo_trace", ["block 0 (chunk 0 of kv head 0: merges)", "block n_kv_heads (chunk 1 of kv head 0, then wo rows)", "last block (wo rows only)"])
+    else:
+        out["attn_decode_kernel"] = read("jsgrad_hip_attn_decode_trace", ["chunk 0 of kv head 0 (merges)", "chunk 1 of kv head 0", "last chunk of the last kv head"])
+    # the w1 | w3 launch of one layer, alone (the trace keeps the last launch of its translation unit)
+    blk, ctx = m.layers[layers - 1], m._ctx
+    f = blk.feed_forward
+    sp = lambda l: l.scale.ptr if l.scale is not None else None
+    check(lib.jsgrad_hip_ffn_gate(f.w1.kind, f.w1.weight.ptr, sp(f.w1), f.w3.weight.ptr, sp(f.w3), ctx.h.ptr, blk.ffn_norm.weight.ptr, blk.ffn_norm.eps, ctx.g.ptr,
+                                  m.dim, m.hidden_dim, ffi.F16))
+    out["gemv_kernel<EPI_SWIGLU> (w1 | w3)"] = read("jsgrad_hip_gemv_trace", ["block 0", "middle block", "last block"])
+    return {"workload": name, "position": position, "layers": layers, "microseconds_since_first_stamp": out}
+
+
 def run_rows_gemm(workload="8B-int8", rows=16, only=""):
     """The several-row Linear launches of one decode step of `rows` sequences, one shape at a time: wq|wk|wv (as one plain
     matrix of their combined height), wo, w1|w3 + SwiGLU, w2, lm_head.  Weights are rotated over cold copies (more than the
@@ -544,6 +600,8 @@ def main():
                     "(a plain copy kernel of known size, to scale the counters) followed by 4 eager decode steps of --workload; prints nothing")
     ap.add_argument("--traffic-batch", type=int, default=1, help="with --traffic-probe: also two batched decode steps of this many sequences")
     ap.add_argument("--traffic-position", type=int, default=0, help="with --traffic-probe: the position the four decode steps start from (attention then reads that many cache rows)")
+    ap.add_argument("--stamps", action="store_true", help="with a library built by `make TRACE=1`: time stamps taken inside the attention and w1 | w3 kernels of --workload "
+                    "at --traffic-position; prints their JSON")
     ap.add_argument("--fused-step", action="store_true", help="run each token as one persistent kernel (jsgrad_hip_decode_step) instead of one launch per fused op")
     ap.add_argument("--stream-step", action="store_true", help="run each token as one persistent kernel with streaming wavefronts (jsgrad_hip_stream_step)")
     ap.add_argument("--formats-only", action="store_true", help="only the load-time kernels of the checkpoint path (GGML dequantisation, casts, row permutation); prints their JSON")
@@ -559,11 +617,16 @@ def main():
 
     from denograd_amd import ffi
     from denograd_amd.device import Device
+    if args.stamps:
+        ffi.LIB_PATH = ffi.LIB_PATH.replace(".so", "_trace.so")      # the library `make TRACE=1` builds beside the product
     dev = Device.get("HIP").init()
     log(f"device: {dev.name}, {dev.cu_count} CUs")
 
     if args.traffic_probe:
         traffic_probe(args.workload, args.traffic_batch, args.traffic_position)
+        return
+    if args.stamps:
+        print(json.dumps({"stamps": stamps(args.workload, args.traffic_position)}), flush=True)
         return
     if args.formats_only:
         print(json.dumps({"formats": run_formats()}), flush=True)

@@ -12,19 +12,25 @@ namespace jsg {
 // the two agree bit for bit wherever both apply.
 constexpr int ATT_NW = 8, ATT_NW_LONG = 16;
 constexpr int ATT_SHORT_CONTEXT = (ATT_NW * 16) * (ATT_NW * 16);
-template <typename AT, int HD, int NREP, int NW>
+template <typename AT, int HD, int NREP, int NW, bool SLICED>
 __global__ __launch_bounds__(NW * 64) void attn_decode_kernel(AttnArgs a) {
-  typedef Attn<AT, HD, NREP, NW, false> A;
+  typedef Attn<AT, HD, NREP, NW, false, SLICED> A;
   __shared__ typename A::Smem sm;
   const int g = blockIdx.x, split = blockIdx.y;
+  JSG_LCLEAR();
   const int pos = a.st[1];
+  JSG_LSTAMP(0);
   if (pos < 0 || pos >= a.max_context) return;
   const int T = pos + 1;
   const int chunk = att_policy_rows(T, A::CHUNK_CAP);            // the host sized nsplit for max_context and this cap
   const int n_active = att_chunk_count(T, chunk);
   if (split >= n_active) return;
   A::item(a, sm, g, split, T, chunk, n_active);
+  JSG_LSTAMP(1);
+  // traced builds: the block that merges kv head 0, the block of that head's chunk 1, the block of the last kv head's last chunk
+  JSG_LFLUSH(g == 0 && split == 0 ? 0 : (g == 0 && split == 1 ? 1 : (g == (int)gridDim.x - 1 && split == n_active - 1 ? 2 : -1)));
 }
+JSG_TRACE_ENTRY(jsgrad_hip_attn_decode_trace)
 
 // Many sequences at the same position (grid z): blocks of 4 wavefronts that stream their rows (attention_stream.h).
 constexpr int ATT_STREAM_NW = 4;
@@ -66,9 +72,12 @@ static int stream_nsplit(int max_context, int heads_x_batch) {
 
 template <typename AT, int HD, int NW> static int launch_attn(const AttnArgs &a, int n_rep) {
   dim3 grid(a.n_kv_heads, a.nsplit, 1), block(NW * 64);
+  // the merge shared by several threads per output element for contexts that would cost the plain one three round trips
+  const bool sliced = att_sliced_merge(a.max_context, NW * 16 < ATT_CHUNK_MAX ? NW * 16 : ATT_CHUNK_MAX);
 #define JSG_REP(N)                                                                                   \
   case N:                                                                                            \
-    JSG_LAUNCH(PROF_ATTN, (attn_decode_kernel<AT, HD, N, NW>), grid, block, 0, a);                     \
+    if (sliced) JSG_LAUNCH(PROF_ATTN, (attn_decode_kernel<AT, HD, N, NW, true>), grid, block, 0, a);   \
+    else JSG_LAUNCH(PROF_ATTN, (attn_decode_kernel<AT, HD, N, NW, false>), grid, block, 0, a);         \
     break;
   switch (n_rep) {
     JSG_REP(1) JSG_REP(2) JSG_REP(3) JSG_REP(4) JSG_REP(8)

@@ -52,6 +52,10 @@ __host__ __device__ __forceinline__ int att_policy_rows(int T, int cap) {
 // chunks a launch must provide for every T up to max_context.  The rows per chunk never shrink as T grows, so for each
 // chunk length r the most chunks are asked for at the largest T that still gets r rows: sqrt(K T) <= r, i.e.
 // T <= ((r + 1)^2 - 1) / K (any T for the shortest and up to max_context for the longest).
+constexpr int ATT_MERGE_BATCH = 16;    // chunks whose partial sums the merge requests in one round trip
+__host__ __device__ __forceinline__ int att_max_chunks(int max_context, int cap);   // below
+// Whether a launch for this max_context takes the sliced merge: from three round trips of the plain one on (see Attn::item).
+__host__ __device__ __forceinline__ bool att_sliced_merge(int max_context, int cap) { return att_max_chunks(max_context, cap) > 2 * ATT_MERGE_BATCH; }
 __host__ __device__ __forceinline__ int att_max_chunks(int max_context, int cap = ATT_CHUNK_MAX) {
   int most = 1;
   for (int r = ATT_CHUNK_MIN; ; r += 16) {
@@ -99,7 +103,9 @@ template <int G> __device__ __forceinline__ float group_sum(float v) {
 // wavefront load); the dot products are reduced inside the group with DPP.  P.V: a lane takes ONE dword of a V row, so the 64
 // lanes cover a whole row (or two rows of 32 dwords) and every lane accumulates its own output elements over the rows of
 // its wavefront: no reduction across lanes at the end (with 16 wavefronts a CU that alone would cost as much as the item).
-template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
+// SLICED: the merge of a kv head's chunks is shared by several threads per output element (below); chosen by the host for
+// contexts long enough to need it (att_sliced_merge), because the larger code costs the short ones a little.
+template <typename AT, int HD, int NREP, int NW, bool COHERENT, bool SLICED = false> struct Attn {
   static constexpr int EPL = 16 / sizeof(AT);  // K: elements per lane per 128-bit load
   static constexpr int G = HD / EPL;           // K: lanes per cache row
   static constexpr int RPI = 64 / G;           // K: rows per wavefront load
@@ -362,19 +368,38 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       // before they store, and the launch keeps them all on the device, so this ends; it is bounded all the same, reports
       // through the error word where one is given, and the result is then NaN.
       const float *base = a.partial + (size_t)g * a.nsplit * NREP * (HD + 2);
-      constexpr int MB = 16;                       // chunks per batch of requests
+      constexpr int MB = SLICED ? ATT_MERGE_BATCH + 2 : ATT_MERGE_BATCH;   // chunks per batch of requests (sliced: 36 chunks in one batch per slice)
       constexpr int NPAIR = NREP * HD / 2;         // element pairs of this kv head's query heads
       constexpr int POLL_LIMIT = 1 << 18;
-      auto pair_at = [&](const float *po, int s_) { return po + (size_t)(s_ < n_active ? s_ : n_active - 1) * NREP * (HD + 2); };
+      // Folding the chunks is a chain of round trips, one per batch of MB chunks, and a thread folds one pair of output
+      // elements.  SLICED: with more threads than pairs, the chunks are cut into slices, thread (slice, pair) folds its
+      // slice, and the slices' sums are added in order through LDS.  (4100 positions in chunks of 128 rows: 33 chunks, three
+      // round trips for one thread, one for two threads with 17 chunks each.)
+      static_assert(NPAIR <= NW * 64, "a thread folds at most one pair");
+      constexpr int SL_FIT = (NW * 64) / NPAIR < NW ? (NW * 64) / NPAIR : NW;   // the slices' sums fit the wavefronts' output slots
+      constexpr int SL = !SLICED ? 1 : (SL_FIT < 4 ? SL_FIT : 4);
+      const int nsl = (SL > 1 && n_active > MB) ? SL : 1;
+      const int per = (n_active + nsl - 1) / nsl;
+      const int sl = SLICED ? tid / NPAIR : 0, pr = SLICED ? tid - sl * NPAIR : tid;     // this thread's slice and pair
+      const int sb = sl * per;
+      const bool folds = SLICED ? (sl < nsl && sb < n_active) : tid < NPAIR;
+      const int send = (SLICED && folds) ? min(n_active, sb + per) : n_active;   // chunks [sb, send) are this thread's
+      // a chunk index past the end stands for the last chunk (of the head for the (m, l) words, of the slice for the sums),
+      // whose words are checked and cleared again and enter the sum with weight zero
+      auto pair_at = [&](const float *po, int s_) { return po + (size_t)(s_ < send ? s_ : send - 1) * NREP * (HD + 2); };
+      auto ml_at = [&](const float *po, int s_) { return po + (size_t)(s_ < n_active ? s_ : n_active - 1) * NREP * (HD + 2); };
       auto ld_pair = [&](const float *po, int s_) -> uint64_t {   // two floats of chunk s_ (8-byte aligned: HD + 2 is even)
         return __hip_atomic_load(as_global<uint64_t>(pair_at(po, s_)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      };
+      auto ld_ml = [&](const float *po, int s_) -> uint64_t {
+        return __hip_atomic_load(as_global<uint64_t>(ml_at(po, s_)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       };
       auto clear_pair = [&](const float *po, int s_) {
         __hip_atomic_store(as_global_mut<uint64_t>(const_cast<float *>(pair_at(po, s_))), 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       };
       auto written = [](uint64_t w) { return (uint32_t)w != 0u && (uint32_t)(w >> 32) != 0u; };
       auto gave_up = [&]() { if (a.err != nullptr) st_coherent(a.err, 1); };
-      const int p0 = tid < NPAIR ? tid : 0;        // threads beyond the pairs request pair 0 again (their result is not stored)
+      const int p0 = folds ? pr : 0;               // threads with nothing to fold request nothing
       const int j0 = (2 * p0) / HD, d0 = (2 * p0) % HD;
       const float *po0 = base + (size_t)j0 * (HD + 2) + d0;
       constexpr int MSL = (CHUNK_CAP + 63) / 64;   // chunks per lane (the host keeps n_active <= CHUNK_CAP)
@@ -382,7 +407,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
       if (wave < NREP) {
   #pragma unroll
         for (int i = 0; i < MSL; i++)
-          if (i * 64 < n_active) mls[i] = ld_pair(base + (size_t)wave * (HD + 2) + HD, lane + i * 64);   // same test for the whole wavefront
+          if (i * 64 < n_active) mls[i] = ld_ml(base + (size_t)wave * (HD + 2) + HD, lane + i * 64);   // same test for the whole wavefront
       }
       // The partial sums of this thread's first pair are asked for as soon as its wavefront has seen every chunk's (m, l)
       // (the owners of pairs are threads of those wavefronts: NREP * HD / 128 <= NREP of them): asked for before that, the
@@ -398,7 +423,7 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
           if (j != wave || it > 0) {
   #pragma unroll
             for (int i = 0; i < MSL; i++)
-              if (i * 64 < n_active) mls[i] = ld_pair(pml, lane + i * 64);
+              if (i * 64 < n_active) mls[i] = ld_ml(pml, lane + i * 64);
           }
           if constexpr (!WORDS) break;
           bool ok = true;
@@ -409,16 +434,16 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
           if (it >= POLL_LIMIT) { lost = true; gave_up(); break; }
           __builtin_amdgcn_s_sleep(1);
         }
-        if (!asked && tid < NPAIR) {
+        if (!asked && folds) {
   #pragma unroll
-          for (int u = 0; u < MB; u++) part[u] = ld_pair(po0, u);
+          for (int u = 0; u < MB; u++) part[u] = ld_pair(po0, sb + u);
         }
         asked = true;
         JSG_LSTAMP(16);
         if constexpr (WORDS) {
   #pragma unroll
           for (int i = 0; i < MSL; i++)
-            if (lane + i * 64 < n_active) clear_pair(pml, lane + i * 64);
+            if (lane + i * 64 < n_active) __hip_atomic_store(as_global_mut<uint64_t>(const_cast<float *>(ml_at(pml, lane + i * 64))), 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         float M = -INFINITY;
   #pragma unroll
@@ -439,11 +464,19 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
         if (__builtin_amdgcn_ballot_w64(lost) != 0) L = __builtin_nanf("");
         if (lane == 0) sm.l_sh[j] = 1.0f / L;  // softmax normalisation is e * (1/sum) (tensor.ts:2211-2214)
       }
-      if (!asked && tid < NPAIR) {        // a wavefront without a query head of its own (no built shape has one that owns pairs)
+      if constexpr (!SLICED) {
+        if (!asked && folds) {        // a wavefront without a query head of its own (no built shape has one that owns pairs)
   #pragma unroll
-        for (int u = 0; u < MB; u++) part[u] = ld_pair(po0, u);
+          for (int u = 0; u < MB; u++) part[u] = ld_pair(po0, sb + u);
+        }
       }
       lds_barrier();
+      if constexpr (SLICED) {
+        if (!asked && folds) {        // a wavefront without a query head of its own asks now that every chunk's (m, l) has been seen
+  #pragma unroll
+          for (int u = 0; u < MB; u++) part[u] = ld_pair(po0, sb + u);
+        }
+      }
       JSG_LSTAMP(17);
       auto finish = [&](int i, float O) {
         const int j = i / HD, d = i % HD;
@@ -453,43 +486,90 @@ template <typename AT, int HD, int NREP, int NW, bool COHERENT> struct Attn {
         else if constexpr (COHERENT) st_coherent(dst, (AT)r);
         else *dst = (AT)r;
       };
-      for (int p = tid; p < NPAIR; p += nthreads) {
-        const int j = (2 * p) / HD, d = (2 * p) % HD;
-        const float *po = base + (size_t)j * (HD + 2) + d;
+      if constexpr (SLICED) {
         float Oa = 0.0f, Ob = 0.0f;
-        for (int s0 = 0; s0 < n_active; s0 += MB) {
-          for (int it = 0;; it++) {
-            if (s0 > 0 || p != tid || it > 0) {     // the first batch of the first pair is already here
+        if (folds) {
+          const float *po = po0;
+          for (int s0 = sb; s0 < send; s0 += MB) {
+            for (int it = 0;; it++) {
+              if (s0 > sb || it > 0) {     // the first batch is already here
   #pragma unroll
-              for (int u = 0; u < MB; u++) part[u] = ld_pair(po, s0 + u);
+                for (int u = 0; u < MB; u++) part[u] = ld_pair(po, s0 + u);
+              }
+              if constexpr (!WORDS) break;
+              bool ok = true;              // no branches from here to the sums (see pair_at)
+  #pragma unroll
+              for (int u = 0; u < MB; u++) ok = ok & written(part[u]);
+              if (ok) break;
+              if (it >= POLL_LIMIT) { Oa = Ob = __builtin_nanf(""); gave_up(); break; }
+              __builtin_amdgcn_s_sleep(1);
             }
-            if constexpr (!WORDS) break;
-            // no branches from here to the sums: a chunk index past the end stands for the last chunk (ld_pair, clear_pair),
-            // whose words are checked and cleared again and enter the sum with weight zero
-            bool ok = true;
+            if constexpr (WORDS) {
   #pragma unroll
-            for (int u = 0; u < MB; u++) ok = ok & written(part[u]);
-            if (ok) break;
-            if (it >= POLL_LIMIT) { Oa = Ob = __builtin_nanf(""); gave_up(); break; }
-            __builtin_amdgcn_s_sleep(1);
-          }
-          if constexpr (WORDS) {
+              for (int u = 0; u < MB; u++) clear_pair(po, s0 + u);
+            }
+            float wgt[MB];
   #pragma unroll
-            for (int u = 0; u < MB; u++) clear_pair(po, s0 + u);
-          }
-          float wgt[MB];
+            for (int u = 0; u < MB; u++) wgt[u] = sm.sc[j0][s0 + u < send ? s0 + u : send - 1];
   #pragma unroll
-          for (int u = 0; u < MB; u++) wgt[u] = sm.sc[j][s0 + u < n_active ? s0 + u : n_active - 1];
-  #pragma unroll
-          for (int u = 0; u < MB; u++) {
-            const bool in = s0 + u < n_active;
-            const float w = in ? wgt[u] : 0.0f;
-            Oa = fmaf(in ? dec((uint32_t)part[u]) : 0.0f, w, Oa);
-            Ob = fmaf(in ? dec((uint32_t)(part[u] >> 32)) : 0.0f, w, Ob);
+            for (int u = 0; u < MB; u++) {
+              const bool in = s0 + u < send;
+              const float w = in ? wgt[u] : 0.0f;
+              Oa = fmaf(in ? dec((uint32_t)part[u]) : 0.0f, w, Oa);
+              Ob = fmaf(in ? dec((uint32_t)(part[u] >> 32)) : 0.0f, w, Ob);
+            }
           }
         }
-        finish(2 * p, Oa);
-        finish(2 * p + 1, Ob);
+        if (nsl > 1) {      // the same for the whole block: the slices' sums meet in LDS (the wavefronts' output slots are free by now)
+          float *ps = &sm.o_part[0][0][0];
+          if (sl < nsl) { ps[tid * 2] = Oa; ps[tid * 2 + 1] = Ob; }      // tid = sl * NPAIR + pr; a slice without chunks adds zeros
+          lds_barrier();
+          if (sl == 0)
+            for (int q = 1; q < nsl; q++) { Oa += ps[(q * NPAIR + pr) * 2]; Ob += ps[(q * NPAIR + pr) * 2 + 1]; }
+        }
+        if (sl == 0) {
+          finish(2 * pr, Oa);
+          finish(2 * pr + 1, Ob);
+        }
+      } else {
+        for (int p = tid; p < NPAIR; p += nthreads) {
+          const int j = (2 * p) / HD, d = (2 * p) % HD;
+          const float *po = base + (size_t)j * (HD + 2) + d;
+          float Oa = 0.0f, Ob = 0.0f;
+          for (int s0 = 0; s0 < n_active; s0 += MB) {
+            for (int it = 0;; it++) {
+              if (s0 > 0 || p != tid || it > 0) {     // the first batch of the first pair is already here
+    #pragma unroll
+                for (int u = 0; u < MB; u++) part[u] = ld_pair(po, s0 + u);
+              }
+              if constexpr (!WORDS) break;
+              // no branches from here to the sums: a chunk index past the end stands for the last chunk (ld_pair, clear_pair),
+              // whose words are checked and cleared again and enter the sum with weight zero
+              bool ok = true;
+    #pragma unroll
+              for (int u = 0; u < MB; u++) ok = ok & written(part[u]);
+              if (ok) break;
+              if (it >= POLL_LIMIT) { Oa = Ob = __builtin_nanf(""); gave_up(); break; }
+              __builtin_amdgcn_s_sleep(1);
+            }
+            if constexpr (WORDS) {
+    #pragma unroll
+              for (int u = 0; u < MB; u++) clear_pair(po, s0 + u);
+            }
+            float wgt[MB];
+    #pragma unroll
+            for (int u = 0; u < MB; u++) wgt[u] = sm.sc[j][s0 + u < n_active ? s0 + u : n_active - 1];
+    #pragma unroll
+            for (int u = 0; u < MB; u++) {
+              const bool in = s0 + u < n_active;
+              const float w = in ? wgt[u] : 0.0f;
+              Oa = fmaf(in ? dec((uint32_t)part[u]) : 0.0f, w, Oa);
+              Ob = fmaf(in ? dec((uint32_t)(part[u] >> 32)) : 0.0f, w, Ob);
+            }
+          }
+          finish(2 * p, Oa);
+          finish(2 * p + 1, Ob);
+        }
       }
       JSG_LSTAMP(18);
     }

@@ -32,10 +32,10 @@ constexpr int AW_THREADS = JSG_AW_THREADS;
 constexpr int AW_WAVES = AW_THREADS / 64;
 constexpr int AW_CHUNK_CAP = AW_WAVES * 16 < ATT_CHUNK_MAX ? AW_WAVES * 16 : ATT_CHUNK_MAX;   // attention_core.h: 16 rows per wavefront
 
-template <int KIND, int HD, int NREP>
+template <int KIND, int HD, int NREP, bool SLICED>
 __global__ __launch_bounds__(AW_THREADS) void attn_wo_kernel(AttnArgs at, GemvArgs a, int layer) {
   typedef _Float16 AT;
-  typedef Attn<AT, HD, NREP, AW_THREADS / 64, false> A;
+  typedef Attn<AT, HD, NREP, AW_THREADS / 64, false, SLICED> A;   // SLICED: as jsgrad_hip_attn_decode picks it, so that the two agree bit for bit
   typedef Gemv<KIND, AT, EPI_STORE, 2, 4, false> G;
   extern __shared__ __align__(16) unsigned char smem[];   // the staged input row of wo
   __shared__ typename A::Smem sm;
@@ -105,7 +105,7 @@ template <int KIND, int HD> static int aw_capacity(int n_rep, size_t lds, int *o
   int per_cu = 0;
 #define JSG_REP(N)                                                                                                                      \
   case N:                                                                                                                               \
-    JSG_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void *)attn_wo_kernel<KIND, HD, N>, AW_THREADS, lds));          \
+    JSG_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void *)attn_wo_kernel<KIND, HD, N, true>, AW_THREADS, lds));          \
     break;
   switch (n_rep) {
     JSG_REP(1) JSG_REP(2) JSG_REP(3) JSG_REP(4)
@@ -135,9 +135,11 @@ template <int KIND, int HD> static int launch_attn_wo(const AttnArgs &at, const 
   JSG_REQUIRE(items <= cached_capacity[n_rep],
               "jsgrad_hip_attn_wo: %d attention items (%d kv heads x %d chunks of the context) but the device holds %d blocks of this kernel at once; "
               "use jsgrad_hip_attn_decode + jsgrad_hip_linear for this shape", items, at.n_kv_heads, at.nsplit, cached_capacity[n_rep]);
+  const bool sliced = att_sliced_merge(at.max_context, AW_CHUNK_CAP);
 #define JSG_REP(N)                                                                                                   \
   case N:                                                                                                            \
-    JSG_LAUNCH(PROF_ATTN_WO, (attn_wo_kernel<KIND, HD, N>), dim3(blocks), dim3(AW_THREADS), lds, at, a, layer);       \
+    if (sliced) JSG_LAUNCH(PROF_ATTN_WO, (attn_wo_kernel<KIND, HD, N, true>), dim3(blocks), dim3(AW_THREADS), lds, at, a, layer);   \
+    else JSG_LAUNCH(PROF_ATTN_WO, (attn_wo_kernel<KIND, HD, N, false>), dim3(blocks), dim3(AW_THREADS), lds, at, a, layer);         \
     break;
   switch (n_rep) {
     JSG_REP(1) JSG_REP(2) JSG_REP(3) JSG_REP(4)

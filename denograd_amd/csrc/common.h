@@ -300,13 +300,7 @@ __device__ __forceinline__ float xexp2h(float d) {
 // Tensor.exp on float tensors (tensor.ts:147-154)
 __device__ __forceinline__ float exp_f32(float x) { return xexp2f(__fmul_rn(x, 1.4426950408889634f)); }
 
-// NF4 code book (llama3.ts:80-81); the CODE tensor is float16, so every literal is rounded to fp16 first
-#define JSG_C16(x) ((float)(_Float16)(x))
-static __device__ __constant__ float NF4_CODE[16] = {JSG_C16(-1.0f), JSG_C16(-0.6961928009986877f), JSG_C16(-0.5250730514526367f), JSG_C16(-0.39491748809814453f),
-                                              JSG_C16(-0.28444138169288635f), JSG_C16(-0.18477343022823334f), JSG_C16(-0.09105003625154495f), JSG_C16(0.0f),
-                                              JSG_C16(0.07958029955625534f), JSG_C16(0.16093020141124725f), JSG_C16(0.24611230194568634f), JSG_C16(0.33791524171829224f),
-                                              JSG_C16(0.44070982933044434f), JSG_C16(0.5626170039176941f), JSG_C16(0.7229568362236023f), JSG_C16(1.0f)};
-
+// NF4 code book (llama3.ts:80-81); the CODE tensor is float16, so every literal is rounded to fp16 first.
 // NF4 code n as fp16 bits, selected from literals by the four bits of n: a table in memory would cost its readers a memory
 // round trip per entry, and the look-up tables are built at the head of a launch, in front of everything else.
 #define JSG_H16(x) ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)(x)))

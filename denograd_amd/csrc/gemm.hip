@@ -88,8 +88,7 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
   // llama3.ts:92-94), so a byte costs one LDS read and one packed multiplication by the block scale
   uint32_t *pairs = (uint32_t *)(lut + 16);
   if constexpr (KIND == JSGRAD_W_NF4) {
-    const h2_t c = {(_Float16)NF4_CODE[tid >> 4], (_Float16)NF4_CODE[tid & 15]};
-    pairs[tid] = __builtin_bit_cast(uint32_t, c);
+    pairs[tid] = nf4_code_bits(tid >> 4) | (nf4_code_bits(tid & 15) << 16);   // from literals: no memory round trip at the head of the launch
   }
 
   // ---- tile id: XCD-contiguous, then grouped so that neighbouring ids share an x tile column-block
