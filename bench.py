@@ -439,6 +439,8 @@ def traffic_probe(name, batch=1, position=0):
 STAMP_NAMES = {0: "position word read", 10: "attention item starts", 11: "query rows in LDS", 12: "scores done", 13: "softmax done", 14: "P.V in the wavefronts' slots",
                15: "partial result stored", 16: "every chunk's (m, l) seen", 17: "merge weights ready", 18: "merged row stored", 1: "attention item done",
                2: "wo: hint of the attention row seen", 3: "wo: hint barrier", 4: "wo: attention row staged", 21: "wo rows done",
+               5: "x requested, table written", 6: "first item requested", 7: "x arrived, squares summed", 9: "sum of squares exchanged",
+               26: "... by the block's last wavefront", 27: "first item requested by the last wavefront", 28: "x arrived in the last wavefront",
                23: "x staged, first two items requested", 24: "first item used", 25: "second item used", 8: "end"}
 
 
@@ -462,19 +464,24 @@ def stamps(name, position, layers=8):
     for t in (1, 2, 3):
         llm._call(t)
         llm.start_pos += 1
-    buf = (C.c_ulonglong * 96)()
+    buf = (C.c_ulonglong * 128)()
     out = {}
 
     def read(entry, rows):
         fn = getattr(raw, entry)
         fn.argtypes, fn.restype = [C.c_void_p], C.c_int
         check(fn(buf))
-        t = np.array(buf[:], dtype=np.uint64).reshape(3, 32).astype(np.int64)
+        t4 = np.array(buf[:], dtype=np.uint64).reshape(4, 32)
+        t, whole = t4[:3].astype(np.int64), t4[3]       # row 3: over all blocks of the launch (earliest start kept complemented)
         if not (t > 0).any():
             return None
         t0 = t[t > 0].min()
-        return {who: {STAMP_NAMES[s_]: round((int(t[r][s_]) - int(t0)) / 100.0, 2) for s_ in sorted(STAMP_NAMES, key=lambda k: t[r][k]) if t[r][s_] > 0}
-                for r, who in enumerate(rows)}
+        res = {who: {STAMP_NAMES[s_]: round((int(t[r][s_]) - int(t0)) / 100.0, 2) for s_ in sorted(STAMP_NAMES, key=lambda k: t[r][k]) if t[r][s_] > 0}
+               for r, who in enumerate(rows)}
+        if whole[2]:
+            us = lambda v: round((int(v) - int(t0)) / 100.0, 2)
+            res["all blocks of the launch"] = {"latest block end": us(whole[2])}
+        return res
     fused = m._ctx.fuse_attn_wo
     llm._call(4)
     llm.start_pos += 1

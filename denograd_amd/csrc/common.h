@@ -190,7 +190,7 @@ __device__ __forceinline__ float row8_sum(float v) {
 #ifndef JSG_TRACE_BLOCK
 #define JSG_TRACE_BLOCK 0
 #endif
-static __device__ unsigned long long g_trace[3][32];
+static __device__ unsigned long long g_trace[4][32];   // row 3: over all blocks of the launch (JSG_LALL)
 __device__ __forceinline__ int trace_row() { return blockIdx.x == JSG_TRACE_BLOCK ? 0 : (blockIdx.x == gridDim.x - 1 ? 2 : -1); }
 __device__ __forceinline__ void trace_stamp(int row, int slot) {
   if (row >= 0 && threadIdx.x == 0) g_trace[row][slot] = __builtin_amdgcn_s_memrealtime();
@@ -204,13 +204,15 @@ static __shared__ unsigned long long jsg_tl[32];
 #define JSG_TRACE_THREAD 0      // the thread whose time is kept: 0, or the first lane of another wavefront of the block
 #endif
 #define JSG_LSTAMP(slot) do { if (threadIdx.x == JSG_TRACE_THREAD) jsg::jsg_tl[slot] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#define JSG_LMAX(slot) do { if ((threadIdx.x & 63) == 0) atomicMax(&jsg::jsg_tl[slot], (unsigned long long)__builtin_amdgcn_s_memrealtime()); } while (0)   /* the last wavefront to get here */
+#define JSG_LALL(slot, late) do { if (threadIdx.x == 0) { const unsigned long long t_ = __builtin_amdgcn_s_memrealtime(); atomicMax(&jsg::g_trace[3][slot], (late) ? t_ : ~t_); } } while (0)   /* latest (or, complemented, earliest) block */
 #define JSG_LCLEAR() do { if (threadIdx.x < 32) jsg::jsg_tl[threadIdx.x] = 0; __syncthreads(); } while (0)
 #define JSG_LFLUSH(row) do { __syncthreads(); const int row_ = (row); if (row_ >= 0 && threadIdx.x < 32) jsg::g_trace[row_][threadIdx.x] = jsg::jsg_tl[threadIdx.x]; } while (0)
 #define JSG_TRACE_ENTRY(name)                                                                              \
   extern "C" int name(unsigned long long *host_out) {                                                      \
     JSG_HIP(hipStreamSynchronize(jsg::state().stream));                                                    \
     JSG_HIP(hipMemcpyFromSymbol(host_out, HIP_SYMBOL(jsg::g_trace), sizeof(jsg::g_trace)));                  \
-    unsigned long long z[3][32] = {};                                                                      \
+    unsigned long long z[4][32] = {};                                                                      \
     JSG_HIP(hipMemcpyToSymbol(HIP_SYMBOL(jsg::g_trace), z, sizeof(z)));                                     \
     return 0;                                                                                              \
   }
@@ -218,6 +220,8 @@ static __shared__ unsigned long long jsg_tl[32];
 #define JSG_STAMP(slot) ((void)0)
 #define JSG_STAMP_ROW(row, slot) ((void)0)
 #define JSG_LSTAMP(slot) ((void)0)
+#define JSG_LMAX(slot) ((void)0)
+#define JSG_LALL(slot, late) ((void)0)
 #define JSG_LCLEAR() ((void)0)
 #define JSG_LFLUSH(row) ((void)0)
 #define JSG_TRACE_ENTRY(name)

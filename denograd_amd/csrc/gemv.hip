@@ -9,6 +9,10 @@ namespace jsg {
 // for NF4 launches with rows enough for that on every CU, one block of sixteen around a per-lane look-up table of 64 KiB
 // (NW = 16, Gemv<..., WIDE>).
 // EXACT: see Gemv::load_item; the host picks it from the items a wavefront of the launch walks
+// traced builds: the three blocks whose stamps are kept (first, middle, last unless the build says otherwise)
+#ifndef JSG_TRACE_ROWS
+#define JSG_TRACE_ROWS(b, n) ((b) == 0 ? 0 : ((b) == (n) / 2 ? 1 : ((b) == (n) - 1 ? 2 : -1)))
+#endif
 template <int KIND, typename AT> constexpr bool gemv_may_be_wide() { return KIND == JSGRAD_W_NF4 && sizeof(AT) == 2; }
 template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, int EXACT, int NW = 4>
 __global__ __launch_bounds__(64 * NW, sizeof(AT) == 2 ? 4 : 1) void gemv_kernel(GemvArgs a) {
@@ -24,7 +28,8 @@ __global__ __launch_bounds__(64 * NW, sizeof(AT) == 2 ? 4 : 1) void gemv_kernel(
   GemvBuf buf;
   G::template run<true>(a, (AT *)smem, red, lut, buf, false, pos);
   JSG_LSTAMP(8);
-  JSG_LFLUSH(blockIdx.x == 0 ? 0 : (blockIdx.x == gridDim.x / 2 ? 1 : (blockIdx.x == gridDim.x - 1 ? 2 : -1)));
+  JSG_LALL(2, true);
+  JSG_LFLUSH(JSG_TRACE_ROWS((int)blockIdx.x, (int)gridDim.x));
 }
 JSG_TRACE_ENTRY(jsgrad_hip_gemv_trace)
 
