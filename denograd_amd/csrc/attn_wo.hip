@@ -33,14 +33,14 @@ constexpr int AW_WAVES = AW_THREADS / 64;
 constexpr int AW_CHUNK_CAP = AW_WAVES * 16 < ATT_CHUNK_MAX ? AW_WAVES * 16 : ATT_CHUNK_MAX;   // attention_core.h: 16 rows per wavefront
 
 template <int KIND, int HD, int NREP, bool SLICED>
-__global__ __launch_bounds__(AW_THREADS) void attn_wo_kernel(AttnArgs at, GemvArgs a, int layer) {
+__global__ __launch_bounds__(AW_THREADS, 2 * AW_WAVES / 4) void attn_wo_kernel(AttnArgs at, GemvArgs a, int layer) {   // two blocks per CU (128 registers)
   typedef _Float16 AT;
   typedef Attn<AT, HD, NREP, AW_THREADS / 64, false, SLICED> A;   // SLICED: as jsgrad_hip_attn_decode picks it, so that the two agree bit for bit
   typedef Gemv<KIND, AT, EPI_STORE, 2, 4, false> G;
   extern __shared__ __align__(16) unsigned char smem[];   // the staged input row of wo
   __shared__ typename A::Smem sm;
   __shared__ float red[AW_WAVES];
-  __shared__ float lut[16];
+  __shared__ float lut[KIND == JSGRAD_W_NF4 ? NF4_LUT_WORDS : 16];   // NF4: the code book and the table of code pairs (Gemv::fill_lut)
 
   // The position first, and nothing else until it is here: a small request issued into an idle memory system is back in a
   // fraction of a microsecond, behind the bursts of weight requests of all blocks it takes several times as long, and every
@@ -167,7 +167,7 @@ static int attn_wo_impl(const void *q, const void *cache_k, const void *cache_v,
                         int *query_capacity) {
   JSG_READY();
   if (!query_capacity) JSG_REQUIRE(q && cache_k && cache_v && st && workspace && wo && y, "jsgrad_hip_attn_wo: null pointer argument");
-  JSG_REQUIRE(kind == JSGRAD_W_F16 || kind == JSGRAD_W_I8, "jsgrad_hip_attn_wo: weight kind %d (fp16 and int8 are built)", kind);
+  JSG_REQUIRE(kind == JSGRAD_W_F16 || kind == JSGRAD_W_I8 || kind == JSGRAD_W_NF4, "jsgrad_hip_attn_wo: weight kind %d (fp16, int8 and nf4 are built)", kind);
   JSG_REQUIRE(kind == JSGRAD_W_F16 || so || query_capacity, "jsgrad_hip_attn_wo: quantised weight needs a scale");
   JSG_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_kv_heads <= 64 && n_heads % n_kv_heads == 0, "jsgrad_hip_attn_wo: n_heads %d / n_kv_heads %d", n_heads, n_kv_heads);
   JSG_REQUIRE(head_dim == 64 || head_dim == 128, "jsgrad_hip_attn_wo: head_dim %d (64 and 128 are built)", head_dim);
@@ -176,6 +176,7 @@ static int attn_wo_impl(const void *q, const void *cache_k, const void *cache_v,
   const int qdim = n_heads * head_dim;
   JSG_REQUIRE(dim > 0 && dim % 2 == 0 && qdim % 16 == 0 && (size_t)qdim * 2 <= 64 * 1024, "jsgrad_hip_attn_wo: dim %d / n_heads*head_dim %d", dim, qdim);
   JSG_REQUIRE(fits_buffer_offsets((size_t)dim, (size_t)qdim, 16), "jsgrad_hip_attn_wo: wo of %d x %d elements reaches 4 GiB (32-bit byte offsets)", dim, qdim);
+  JSG_REQUIRE(kind != JSGRAD_W_NF4 || qdim % 64 == 0, "jsgrad_hip_attn_wo: nf4 rows of %d elements (blocks of 64)", qdim);
   char *ws = (char *)workspace;
   AttnArgs at;
   at.q = q; at.cache_k = cache_k; at.cache_v = cache_v; at.st = st; at.out = nullptr;
@@ -198,6 +199,7 @@ static int attn_wo_impl(const void *q, const void *cache_k, const void *cache_v,
   switch (kind) {
     JSG_KIND(JSGRAD_W_F16)
     JSG_KIND(JSGRAD_W_I8)
+    JSG_KIND(JSGRAD_W_NF4)
   }
 #undef JSG_KIND
   return fail("jsgrad_hip_attn_wo: weight kind %d", kind);

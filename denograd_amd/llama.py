@@ -354,7 +354,7 @@ class Transformer:
                 layer.attention._ensure_cache(self.dtype, self.device)
                 layer.attention.layer_id = i
             wo = self.layers[0].attention.wo
-            if (self.fuse_attn_wo and self.dtype == "float16" and wo.kind in (ffi.W_F16, ffi.W_I8) and 2 <= len(self.layers) <= 128 and hd in (64, 128)
+            if (self.fuse_attn_wo and self.dtype == "float16" and wo.kind in (ffi.W_F16, ffi.W_I8, ffi.W_NF4) and 2 <= len(self.layers) <= 128 and hd in (64, 128)
                     and self.n_heads // self.n_kv_heads in (1, 2, 3, 4) and self.max_context <= 64 * 128 and self.n_heads * hd * 2 <= 64 * 1024
                     and self.n_kv_heads <= 64 and attn_wo_fits(self.n_heads, self.n_kv_heads, hd, self.max_context, wo.kind, self.dim)):
                 self._ctx.enable_attn_wo(self.n_heads, self.n_kv_heads, hd, self.device)

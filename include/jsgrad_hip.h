@@ -283,8 +283,8 @@ int jsgrad_hip_stream_status(const void *workspace, int *host_out_error);
 
 /* jsgrad_hip_attn_decode followed by jsgrad_hip_linear(wo, residual) of one layer as ONE launch (models/llama.ts:89-96 and the
  * residual add of :125): y[dim] = residual + wo . attention(q, cache).  The first wo weights of every wavefront are requested
- * before the attention items run, and the attention row reaches the wo part inside the launch.  fp16 activations, fp16 or int8
- * wo.  layer: index of the layer in the model (0..127; launches that share a workspace must differ in layer or position, so
+ * before the attention items run, and the attention row reaches the wo part inside the launch.  fp16 activations; fp16, int8
+ * or nf4 wo.  layer: index of the layer in the model (0..127; launches that share a workspace must differ in layer or position, so
  * a model needs at least two layers).  workspace: jsgrad_hip_attn_wo_workspace_bytes() bytes, zero-filled once before first
  * use, one per model.  The wait inside the launch is bounded; jsgrad_hip_attn_wo_status reads whether one ever ran out. */
 size_t jsgrad_hip_attn_wo_workspace_bytes(int n_heads, int n_kv_heads, int head_dim);

@@ -357,7 +357,8 @@ def test_attention_decode_unrounded_probabilities(hip, H, KV, hd, ctx):
         assert np.max(np.abs(got - rounded)) <= bound + 2 * float(ulp.max()), f"T={T}"
 
 
-@pytest.mark.parametrize("kind,H,KV,hd,ctx", [("f16", 32, 8, 64, 1024), ("i8", 8, 2, 128, 4096), ("f16", 4, 4, 64, 96), ("i8", 24, 8, 128, 640), ("f16", 8, 2, 64, 8192)])
+@pytest.mark.parametrize("kind,H,KV,hd,ctx", [("f16", 32, 8, 64, 1024), ("i8", 8, 2, 128, 4096), ("f16", 4, 4, 64, 96), ("i8", 24, 8, 128, 640), ("f16", 8, 2, 64, 8192),
+                                              ("nf4", 32, 8, 128, 640), ("nf4", 8, 2, 64, 4160)])
 def test_attention_and_wo_in_one_launch(hip, kind, H, KV, hd, ctx):
     """jsgrad_hip_attn_wo == jsgrad_hip_attn_decode followed by jsgrad_hip_linear(wo, residual), bit for bit, for several T,
     two layers sharing one workspace (the version tag tells their rows apart), and no bounded wait ever running out."""
@@ -370,6 +371,9 @@ def test_attention_and_wo_in_one_launch(hip, kind, H, KV, hd, ctx):
     if kind == "i8":
         wq, sc = orc.int8_quantize(w)
         tw, ts, code = Tensor(wq), Tensor(sc), ffi.W_I8
+    elif kind == "nf4":
+        wq, sc = orc.nf4_quantize(w)
+        tw, ts, code = Tensor(wq), Tensor(sc), ffi.W_NF4
     else:
         tw, ts, code = Tensor(w.astype(np.float16)), None, ffi.W_F16
     tK, tV, tq, tres = Tensor(K), Tensor(V), Tensor(q), Tensor(res)
