@@ -78,7 +78,7 @@ export class HipDecoder {
     // attention and wo share a launch when every attention block fits the device at once and the format allows it
     const wo = l0.wo as Lin, items = c.out_i32(), cap = c.out_i32()
     c.check(S.jsgrad_hip_attn_wo_fits(l0.n_heads, l0.n_kv_heads, l0.head_dim, model.max_context, kind_of(wo), dim, items, cap))
-    if (act === c.JSGRAD_F16 && model.layers.length >= 2 && model.layers.length <= 128 && [c.JSGRAD_W_F16, c.JSGRAD_W_I8].includes(kind_of(wo)) && items[0] <= cap[0]) {
+    if (act === c.JSGRAD_F16 && model.layers.length >= 2 && model.layers.length <= 128 && [c.JSGRAD_W_F16, c.JSGRAD_W_I8, c.JSGRAD_W_NF4].includes(kind_of(wo)) && items[0] <= cap[0]) {
       d.attn_wo_ws = await bytes(Number(S.jsgrad_hip_attn_wo_workspace_bytes(l0.n_heads, l0.n_kv_heads, l0.head_dim)))
     }
     return d
