@@ -106,10 +106,12 @@ __device__ __forceinline__ u4_t ldg_stream16(const void *p) { return __builtin_n
 constexpr uint32_t BUF_END = 0xFFFFFF00u;
 // host side: a matrix read this way must end below BUF_END
 inline bool fits_buffer_offsets(size_t rows, size_t row_elems, int bits) { return rows * row_elems * (size_t)bits / 8 < (size_t)BUF_END; }
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t wave_buffer(const void *p) {   // p: the same for every lane of the wavefront
+// p, nbytes: the same for every lane of the wavefront.  nbytes is the size of what p points to: a load that reaches past it
+// returns zeros without touching memory, whatever the offset arithmetic of the caller did (BUF_END is past every size).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t wave_buffer(const void *p, uint32_t nbytes) {
   const uint64_t v = (uint64_t)p;
   const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-  return __builtin_amdgcn_make_buffer_rsrc((void *)(((uint64_t)hi << 32) | lo), 0, (int)BUF_END, 0x00020000);
+  return __builtin_amdgcn_make_buffer_rsrc((void *)(((uint64_t)hi << 32) | lo), 0, (int)__builtin_amdgcn_readfirstlane(nbytes), 0x00020000);
 }
 __device__ __forceinline__ u4_t buf_stream16(__amdgpu_buffer_rsrc_t rs, uint32_t off) {
   return __builtin_bit_cast(u4_t, __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, 0, 2));   // 2: nontemporal

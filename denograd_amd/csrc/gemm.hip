@@ -404,9 +404,10 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
 //
 // With a handful of rows the launch is bound by reading W once, so it is laid out like the one-row GEMV, not like a tiled
 // GEMM.  v_mfma_f32_16x16x32_f16 takes, per lane, 8 consecutive K elements of one weight row as B and of one x row as
-// A; a lane's 16-byte load is 8 fp16 or 16 int8 codes of weight row n0 + lane % 16, i.e. one or two MFMAs, and goes from
-// memory to registers with nothing in between (the int8 codes become RN16(code * scale) in registers: the realised
-// fp16 matrix the reference multiplies by).  The loads run through a register ring of 12 to 16 loads per wavefront.
+// A; a lane's 16-byte load is 8 fp16, 16 int8 codes or 32 nf4 codes of weight row n0 + lane % 16, i.e. one, two or four
+// MFMAs, and goes from memory to registers with nothing in between (int8 and nf4 codes become RN16(code * scale) in
+// registers: the realised fp16 matrix the reference multiplies by; nf4 through a 256-entry table of code pairs in LDS, one
+// look-up per byte, with the scale of the lane's 64-element block loaded beside the codes).  The loads run through a register ring of 12 to 16 loads per wavefront.
 // Only x goes through LDS, in K chunks of 512, four buffers.  The fifth wavefront of a block does nothing but move
 // x chunks from memory to LDS (direct loads, no registers), up to three chunks ahead: a wavefront's loads return in order, so x loads issued by
 // the arithmetic wavefronts would have to be waited for together with every weight load issued before them, which
@@ -417,7 +418,7 @@ __global__ __launch_bounds__(GEMM_THREADS, (TM * TN > 8 ? 1 : (TM * TN > 4 ? 2 :
 // N = 4096.  (A block shape with 128 weight rows, which reads x once for all of them instead of once per 16, was tried for
 // the wide layers: faster for the lm_head only, and its register ring did not survive the register allocator.)
 template <int KIND> struct SkFmt {
-  static constexpr int VEC = KIND == JSGRAD_W_F16 ? 8 : 16;   // K elements per 16-byte load of a lane
+  static constexpr int VEC = KIND == JSGRAD_W_F16 ? 8 : (KIND == JSGRAD_W_I8 ? 16 : 32);   // K elements per 16-byte load of a lane
   static constexpr int KB = 4 * VEC;                          // K elements per wavefront load (a k-block)
   static constexpr int KC = 512;                              // K elements per x chunk: 1 KiB per x row, one direct load
   static constexpr int KBC = KC / KB;                         // k-blocks per chunk
@@ -441,7 +442,7 @@ __device__ __forceinline__ void sk_barrier() { asm volatile("s_waitcnt lgkmcnt(0
 
 template <int KIND, int EPI, int MB, int RTW>
 __global__ __launch_bounds__(SK_THREADS, 2) void skinny_gemm_kernel(GemmArgs a) {
-  static_assert(KIND == JSGRAD_W_F16 || KIND == JSGRAD_W_I8, "fp16 and int8 weights");
+  static_assert(KIND == JSGRAD_W_F16 || KIND == JSGRAD_W_I8 || KIND == JSGRAD_W_NF4, "fp16, int8 and nf4 weights");
   typedef SkFmt<KIND> F;
   typedef SkShape<KIND, EPI, RTW> S;
   constexpr int NMAT = S::NMAT, SPC = S::SPC, RS = S::RS;
@@ -455,6 +456,12 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_gemm_kernel(GemmArgs a) 
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l16 = lane & 15, lq = lane >> 4;
   const int nchunks = a.K / F::KC;
+  // NF4: one table entry per BYTE, the code values of its two nibbles as a packed pair (element 2j, the high nibble, in the
+  // low half: llama3.ts:92-94); written here, read after the first barrier of either path below
+  __shared__ uint32_t pairs[KIND == JSGRAD_W_NF4 ? 256 : 1];
+  if constexpr (KIND == JSGRAD_W_NF4) {
+    if (tid < 256) pairs[tid] = nf4_code_bits(tid >> 4) | (nf4_code_bits(tid & 15) << 16);
+  }
 
   if (wave == 4) {
     // ---- the x mover: up to three chunks ahead of the one being read (a chunk takes a trip to L2 to arrive, longer than
@@ -497,6 +504,7 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_gemm_kernel(GemmArgs a) 
   // ---- the weight rows of this lane: row n_first + rt * 16 + lane % 16 of matrix q
   const unsigned char *wrow[RTW][NMAT];
   h2_t wscale[RTW][NMAT];
+  const _Float16 *srow[RTW][NMAT];
 #pragma unroll
   for (int rt = 0; rt < RTW; rt++)
 #pragma unroll
@@ -510,8 +518,10 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_gemm_kernel(GemmArgs a) 
         else { w = a.w2; sc = a.s2; row = n - a.n0 - a.n1; }
       } else { w = a.w0; sc = a.s0; row = n; }
       const size_t e = (size_t)row * a.K;
-      wrow[rt][q] = (const unsigned char *)w + (KIND == JSGRAD_W_F16 ? e * 2 : e) + lq * 16;
+      wrow[rt][q] = (const unsigned char *)w + (KIND == JSGRAD_W_F16 ? e * 2 : (KIND == JSGRAD_W_I8 ? e : e / 2)) + lq * 16;
       if constexpr (KIND == JSGRAD_W_I8) { const _Float16 sv = sc[row]; wscale[rt][q] = h2_t{sv, sv}; }
+      // nf4: a scale per 64 elements of the flattened matrix; a lane's 32 elements of a k-block share one (two per k-block)
+      if constexpr (KIND == JSGRAD_W_NF4) srow[rt][q] = sc + (e >> 6) + (lq >> 1);
     }
   // Step s of this wavefront is k-block ks * SPC + s % SPC of chunk s / SPC: its SPC k-blocks of a chunk are neighbours, so
   // that the halves of a 128-byte line of a weight row are asked for by one wavefront, back to back.  Byte offset of the
@@ -526,6 +536,7 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_gemm_kernel(GemmArgs a) 
   };
 
   u4_t ring[RS][RTW][NMAT];
+  _Float16 rsc[KIND == JSGRAD_W_NF4 ? RS : 1][RTW][NMAT];   // nf4: the block scale travels with its load
   f4_t acc[NMAT][RTW][MB];
 #pragma unroll
   for (int q = 0; q < NMAT; q++)
@@ -540,6 +551,7 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_gemm_kernel(GemmArgs a) 
 #pragma unroll
       for (int q = 0; q < NMAT; q++) {
         ring[i][rt][q] = ldg_stream16(wrow[rt][q] + woff(i));
+        if constexpr (KIND == JSGRAD_W_NF4) rsc[i][rt][q] = ldg(srow[rt][q] + (woff(i) >> 5));   // 64 bytes of codes per k-block = two scales
         __builtin_amdgcn_sched_barrier(0);               // issued in the order the loop consumes them: the waits count on it
       }
   sk_barrier();                                          // x chunk 0 is in LDS
@@ -566,7 +578,20 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_gemm_kernel(GemmArgs a) 
             const u4_t raw = ring[i][rt][q];
             h8_t bf[NMF];
             if constexpr (KIND == JSGRAD_W_F16) bf[0] = __builtin_bit_cast(h8_t, raw);
-            else {
+            else if constexpr (KIND == JSGRAD_W_NF4) {
+              const _Float16 s1 = rsc[i][rt][q];
+              const h2_t sv = {s1, s1};
+              const uint32_t wds[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+              for (int d = 0; d < 4; d++) {                // a dword = 8 elements = one matrix instruction
+                u4_t o;
+                o.x = pk_mul_h2(pairs[wds[d] & 0xffu], sv);
+                o.y = pk_mul_h2(pairs[(wds[d] >> 8) & 0xffu], sv);
+                o.z = pk_mul_h2(pairs[(wds[d] >> 16) & 0xffu], sv);
+                o.w = pk_mul_h2(pairs[wds[d] >> 24], sv);
+                bf[d] = __builtin_bit_cast(h8_t, o);
+              }
+            } else {
               const h2_t sc = wscale[rt][q];
               u4_t o0, o1;
               uint32_t lo, hi;
@@ -590,7 +615,10 @@ __global__ __launch_bounds__(SK_THREADS, 2) void skinny_gemm_kernel(GemmArgs a) 
 #pragma unroll
       for (int rt = 0; rt < RTW; rt++)
 #pragma unroll
-        for (int q = 0; q < NMAT; q++) ring[i][rt][q] = ldg_stream16(wrow[rt][q] + woff(s + RS));
+        for (int q = 0; q < NMAT; q++) {
+          ring[i][rt][q] = ldg_stream16(wrow[rt][q] + woff(s + RS));
+          if constexpr (KIND == JSGRAD_W_NF4) rsc[i][rt][q] = ldg(srow[rt][q] + (woff(s + RS) >> 5));
+        }
       if (on && (s + 1) % SPC == 0) sk_barrier();        // chunk c is consumed, chunk c + 1 is in the other buffer
     }
   }
@@ -1048,6 +1076,7 @@ template <int EPI> static int dispatch_gemm(int kind, const GemmArgs &a, int pro
   if (kind == JSGRAD_W_F16) { const int rc = dispatch_skinny<JSGRAD_W_F16, EPI>(a, prof_kind, &taken); if (taken) return rc; }
   if (kind == JSGRAD_W_I8) { const int rc = dispatch_stream<EPI>(a, prof_kind, &taken); if (taken || rc) return rc; }
   if (kind == JSGRAD_W_I8) { const int rc = dispatch_skinny<JSGRAD_W_I8, EPI>(a, prof_kind, &taken); if (taken) return rc; }
+  if (kind == JSGRAD_W_NF4) { const int rc = dispatch_skinny<JSGRAD_W_NF4, EPI>(a, prof_kind, &taken); if (taken) return rc; }
 #define JSG_CASE(K)                                                                                                    \
   case K:                                                                                                              \
     if (piped) return launch_gemm<K, EPI, 2, 2, 4, 4, true>(a, prof_kind);                                            \

@@ -518,7 +518,7 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT, i
     const Where w = locate(a, grp);
     __amdgpu_buffer_rsrc_t rs[NM];
 #pragma unroll
-    for (int j = 0; j < NM; j++) rs[j] = wave_buffer(wbase(a, w.m, j));
+    for (int j = 0; j < NM; j++) rs[j] = wave_buffer(wbase(a, w.m, j), (uint32_t)(((size_t)w.mrows * (size_t)in_f * BITS) / 8));   // below 4 GiB: host-checked
 #pragma unroll
     for (int u = 0; u < UNROLL; u++) {
       // Lanes past the end of the row reload its last vector instead of branching around the load (their x is zero,

@@ -106,7 +106,7 @@ def test_few_rows_streaming_kernel_equals_tiled_kernel(hip, monkeypatch):
     kernel with one and with two tiles of 16 weight rows per block against the tiled kernel."""
     out_f, in_f = 256, 4096
     monkeypatch.setenv("JSG_GEMM_NO_STREAM", "1")      # int8 with at most 16 rows would go to the LDS-streamed kernel
-    for kind in ("float16", "int8"):
+    for kind in ("float16", "int8", "nf4"):
         for rows in (16, 29):
             w, s = make_weight(kind, out_f, in_f)
             x = RNG.standard_normal((rows, in_f)).astype(np.float16)
@@ -220,6 +220,9 @@ def test_few_rows_fused_epilogues_with_one_and_two_tiles_per_block(hip, monkeypa
     test_gemm_ffn_gate(hip, "float16", 20, 1024, 128)
     test_gemm_qkv_rope_writes_queries_and_cache(hip, "int8", 128, 16, 1, 2048)
     test_gemm_qkv_rope_writes_queries_and_cache(hip, "float16", 64, 3, 9, 2048)
+    test_gemm_ffn_gate(hip, "nf4", 16, 2048, 256)
+    test_gemm_ffn_gate(hip, "nf4", 20, 1024, 128)
+    test_gemm_qkv_rope_writes_queries_and_cache(hip, "nf4", 64, 16, 1, 2048)
 
 
 @pytest.mark.parametrize("kind", ["float16", "int8", "nf4"])
