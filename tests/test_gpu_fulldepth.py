@@ -1,6 +1,7 @@
-"""Greedy decoding at FULL depth: the Llama-3.1-8B-shaped int8 model with all 32 layers and the Llama-3.2-1B-shaped fp16
-model with all 16 layers (shapes: /root/reference/jsgrad/models/llama3.ts:119-132), random-init weights made and quantised on
-the device and copied to the host for the CPU oracle, so both sides hold the same codes and scales.
+"""Greedy decoding at FULL depth: the Llama-3.1-8B-shaped int8 and NF4 models with all 32 layers, the Llama-3.2-3B-shaped int8
+model with all 28 and the Llama-3.2-1B-shaped fp16 model with all 16 (shapes: /root/reference/jsgrad/models/llama3.ts:119-132),
+random-init weights made and quantised on the device and copied to the host for the CPU oracle, so both sides hold the same
+codes and scales.
 
 An 8-token prompt, then 32 greedy steps (/root/reference/jsgrad/models/llama.ts:210-212 with temperature 0).  Every step feeds
 both sides the oracle's previous token, so one differing pick cannot hide what comes after it.
@@ -35,7 +36,7 @@ THREADS = min(16, os.cpu_count() or 1)
 N_PROMPT, N_STEPS, N_YARD = 8, 32, 10
 
 
-@pytest.mark.parametrize("name,layers", [("8B-int8", 32), ("1B", 16)])
+@pytest.mark.parametrize("name,layers", [("8B-int8", 32), ("1B", 16), ("3B-int8", 28), ("8B-nf4", 32)])
 def test_greedy_tokens_at_full_depth(name, layers):
     cfg = synthetic.config(name, max_context=N_PROMPT + N_STEPS + 8)
     assert cfg["n_layers"] == layers
