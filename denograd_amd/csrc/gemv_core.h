@@ -750,13 +750,25 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT, i
   __device__ static __forceinline__ void run(const GemvArgs &a, AT *xs, float *red, float *lut, Buf &bufA, bool preloaded, int pos, int blk = blockIdx.x,
                                              int nblk = gridDim.x) {
     const int nw = blockDim.x >> 6;
-    const int ng = ngroups(a), nb = nbatch(a), gstride = nblk * nw;
+    const int ng = ngroups(a), nb = nbatch(a);
+    // Which row groups this wavefront walks: group first_group + i * (all wavefronts of the launch).  WIDE (one block of
+    // sixteen wavefronts per CU): every block takes one contiguous stretch of ceil(ng / nblk) groups and deals it to its
+    // wavefronts in turn, so that all blocks carry the same load and the wavefronts that come last in their CU's request queue
+    // are the ones with one item fewer (dealt launch-wide, 7168 groups over 256 blocks gave three quarters of the CUs 32
+    // items and the rest 16).
+    int gstride = nblk * nw, lim = ng, g0 = first_group(blk, nblk);
+    if constexpr (WIDE) {
+      const int per = (ng + nblk - 1) / nblk;
+      g0 = blk * per + (int)(threadIdx.x >> 6);
+      lim = (blk + 1) * per < ng ? (blk + 1) * per : ng;
+      gstride = nw;
+    }
     XStage xst;
     if constexpr (EARLY_X) stage_x_issue<AT>(a, xst);
     fill_lut(lut);
     JSG_LSTAMP(5);
     JSG_LMAX(26);
-    int grp = first_group(blk, nblk), b = 0;
+    int grp = g0, b = 0;
     auto advance = [&](int &g, int &bb) {
       if (++bb == nb) { bb = 0; g += gstride; }
     };
@@ -764,35 +776,35 @@ template <int KIND, typename AT, int EPI, int ROWS, int UNROLL, bool COHERENT, i
     int gB = grp, bB = b;
     advance(gB, bB);
     // the first item is straight-line code in every launch (the staging of x below then waits for x and not for it)
-    if (!preloaded) load_item_as<true>(a, bufA, grp, 0, pos, grp < ng);
+    if (!preloaded) load_item_as<true>(a, bufA, grp, 0, pos, grp < lim);
     JSG_LSTAMP(6);
     JSG_LMAX(27);
     // block-wide, ends with a barrier (which also publishes lut)
     if constexpr (EARLY_X) {
       // x is back after one round trip; its registers are free again before the second item's are needed
       stage_x_finish<AT>(a, xst, xs, red, nb * UNROLL * STEP);
-      load_item_as<(EXACT >= 1)>(a, bufB, gB, bB, pos, gB < ng);
+      load_item_as<(EXACT >= 1)>(a, bufB, gB, bB, pos, gB < lim);
     } else {
       // the second item goes out before x is staged too: staging (a read of x, the RMSNorm reduction, a block barrier)
       // would otherwise be a stretch with nothing new in flight
-      load_item_as<(EXACT >= 1)>(a, bufB, gB, bB, pos, gB < ng);
+      load_item_as<(EXACT >= 1)>(a, bufB, gB, bB, pos, gB < lim);
       stage_x<AT, COHERENT>(a, xs, red, nb * UNROLL * STEP);
     }
 
     float acc[NM][ROWS];
     JSG_LSTAMP(23);
-    while (grp < ng) {
+    while (grp < lim) {
       use_item(a, bufA, grp, b, acc, xs, lut, pos);
       JSG_LSTAMP(24);
-      if (gB >= ng) break;
+      if (gB >= lim) break;
       grp = gB; b = bB;
       advance(grp, b);                                   // the item after B goes into A
-      load_item(a, bufA, grp, b, pos, grp < ng);
+      load_item(a, bufA, grp, b, pos, grp < lim);
       use_item(a, bufB, gB, bB, acc, xs, lut, pos);
       JSG_LSTAMP(25);
       gB = grp; bB = b;
       advance(gB, bB);                                   // and the one after that into B
-      load_item(a, bufB, gB, bB, pos, grp < ng && gB < ng);
+      load_item(a, bufB, gB, bB, pos, grp < lim && gB < lim);
     }
   }
 };
