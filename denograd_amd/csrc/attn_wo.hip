@@ -33,7 +33,7 @@ constexpr int AW_WAVES = AW_THREADS / 64;
 constexpr int AW_CHUNK_CAP = AW_WAVES * 16 < ATT_CHUNK_MAX ? AW_WAVES * 16 : ATT_CHUNK_MAX;   // attention_core.h: 16 rows per wavefront
 
 template <int KIND, int HD, int NREP, bool SLICED>
-__global__ __launch_bounds__(AW_THREADS, 2 * AW_WAVES / 4) void attn_wo_kernel(AttnArgs at, GemvArgs a, int layer) {   // two blocks per CU (128 registers)
+__global__ __launch_bounds__(AW_THREADS, AW_WAVES <= 8 ? 2 * AW_WAVES / 4 : AW_WAVES / 4) void attn_wo_kernel(AttnArgs at, GemvArgs a, int layer) {   // 16 wavefronts per CU (128 registers): two blocks of eight
   typedef _Float16 AT;
   typedef Attn<AT, HD, NREP, AW_THREADS / 64, false, SLICED> A;   // SLICED: as jsgrad_hip_attn_decode picks it, so that the two agree bit for bit
   typedef Gemv<KIND, AT, EPI_STORE, 2, 4, false> G;
