@@ -1074,7 +1074,11 @@ template <int EPI> static int dispatch_gemm(int kind, const GemmArgs &a, int pro
   const bool small = tall && (pin ? !strcmp(pin, "small") : (!piped && blocks_of(256, 128) < cus));
   bool taken = false;
   if (kind == JSGRAD_W_F16) { const int rc = dispatch_skinny<JSGRAD_W_F16, EPI>(a, prof_kind, &taken); if (taken) return rc; }
-  if (kind == JSGRAD_W_I8) { const int rc = dispatch_stream<EPI>(a, prof_kind, &taken); if (taken || rc) return rc; }
+  // int8, at most 16 rows: the LDS-streamed kernel, except for matrices so small that its K parts cost more than they bring
+  // (wo of the 8B shape, 16.8 MB: 9.7 us against 8.5 us with the direct-operand kernel; wq|wk|wv, 25 MB: 12.3 against 13.5)
+  static const size_t stream_min = getenv("JSG_SG_MIN_BYTES") ? (size_t)atoll(getenv("JSG_SG_MIN_BYTES")) : (size_t)20 << 20;
+  const bool small_matrix = EPI == GEPI_STORE && (size_t)a.N * (size_t)a.K < stream_min;
+  if (kind == JSGRAD_W_I8 && !small_matrix) { const int rc = dispatch_stream<EPI>(a, prof_kind, &taken); if (taken || rc) return rc; }
   if (kind == JSGRAD_W_I8) { const int rc = dispatch_skinny<JSGRAD_W_I8, EPI>(a, prof_kind, &taken); if (taken) return rc; }
   if (kind == JSGRAD_W_NF4) { const int rc = dispatch_skinny<JSGRAD_W_NF4, EPI>(a, prof_kind, &taken); if (taken) return rc; }
 #define JSG_CASE(K)                                                                                                    \
